@@ -1,0 +1,173 @@
+// Deterministic, batch-invariant bf16 GEMM for gfx950:  C[M,N] = X[M,K] * W[N,K]^T.
+//
+// Replaces the kernels behind rl_engine._C.det_gemm_* (reference
+// csrc/cuda/gemm/det_gemm_kernel.cu:92-101, 250-402) and the Triton MFMA kernels of
+// rl_engine/backends/rocm/gemm/mfma_gemm.py:135-274. No split-K, no atomics, no
+// stream-K: one workgroup owns an output tile for the whole K range.
+#include "det_gemm_tile.h"
+#include "rlk_host.h"
+
+namespace rlk {
+
+template <class S, bool VEC, bool OUT_F32>
+__global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatView X, void* __restrict__ C,
+                                                                int64_t ldc, int M, int N, int K,
+                                                                int tiles_m, int tiles_n, int group_m) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  // Tile raster: XCD-compact ids, then column groups of group_m token tiles so
+  // the tiles resident on one XCD share weight and activation panels in its L2.
+  const int total = tiles_m * tiles_n;
+  const int id = xcd_compact_id(blockIdx.x, total);
+  const int per_group = group_m * tiles_n;
+  const int group = id / per_group;
+  const int first_m = group * group_m;
+  const int width = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
+  const int within = id - group * per_group;
+  const int tile_m = first_m + within % width;
+  const int tile_n = within / width;
+  const int n0 = tile_n * S::BN;
+  const int m0 = tile_m * S::BM;
+
+  f32x4_t acc[S::TN][S::TM];
+  tile_mainloop<S, VEC>(W, X, n0, m0, K, lds, acc);
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wave_n = wave % S::WN;
+  const int wave_m = wave / S::WN;
+  const int n_run = n0 + wave_n * 16 * S::TN + (lane >> 4) * S::kRun;  // first feature of this lane's run
+  const int m_lane = m0 + wave_m * 16 * S::TM + (lane & 15);
+
+#pragma unroll
+  for (int jm = 0; jm < S::TM; ++jm) {
+    const int m = m_lane + jm * 16;
+    if (m >= M) continue;
+    if (OUT_F32) {
+      float* row = reinterpret_cast<float*>(C) + (int64_t)m * ldc;
+      const bool vec_ok = (n_run + S::kRun <= N) && ((reinterpret_cast<uintptr_t>(row + n_run) & 15) == 0);
+      if (vec_ok) {
+#pragma unroll
+        for (int jn = 0; jn < S::TN; ++jn) *reinterpret_cast<f32x4_t*>(row + n_run + jn * 4) = acc[jn][jm];
+      } else {
+#pragma unroll
+        for (int jn = 0; jn < S::TN; ++jn)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (n_run + jn * 4 + q < N) row[n_run + jn * 4 + q] = acc[jn][jm][q];
+      }
+    } else {
+      bf16_bits* row = reinterpret_cast<bf16_bits*>(C) + (int64_t)m * ldc;
+      uint32_t packed[2 * S::TN];
+#pragma unroll
+      for (int jn = 0; jn < S::TN; ++jn) {
+        packed[2 * jn] = pack_bf16x2(acc[jn][jm][0], acc[jn][jm][1]);
+        packed[2 * jn + 1] = pack_bf16x2(acc[jn][jm][2], acc[jn][jm][3]);
+      }
+      constexpr int kAlign = S::TN >= 2 ? 16 : 8;
+      const bool vec_ok =
+          (n_run + S::kRun <= N) && ((reinterpret_cast<uintptr_t>(row + n_run) & (kAlign - 1)) == 0);
+      if (vec_ok) {
+        if (S::TN >= 2) {
+#pragma unroll
+          for (int v = 0; v < S::TN / 2; ++v)
+            *reinterpret_cast<u32x4_t*>(row + n_run + v * 8) =
+                u32x4_t{packed[4 * v], packed[4 * v + 1], packed[4 * v + 2], packed[4 * v + 3]};
+          if (S::TN % 2)
+            *reinterpret_cast<u32x2_t*>(row + n_run + (S::TN - 1) * 4) =
+                u32x2_t{packed[2 * S::TN - 2], packed[2 * S::TN - 1]};
+        } else {
+          *reinterpret_cast<u32x2_t*>(row + n_run) = u32x2_t{packed[0], packed[1]};
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < S::kRun; ++e)
+          if (n_run + e < N) row[n_run + e] = (bf16_bits)((packed[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+
+template <class S, bool VEC, bool OUT_F32>
+static hipError_t launch_tile(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
+                              hipStream_t stream) {
+  auto kernel = det_gemm_kernel<S, VEC, OUT_F32>;
+  static bool configured[kMaxDevices] = {};
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev >= 0 && dev < kMaxDevices && !configured[dev]) {
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              S::kLdsBytes);
+    if (err != hipSuccess) return err;
+    configured[dev] = true;
+  }
+  const int tiles_m = (M + S::BM - 1) / S::BM;
+  const int tiles_n = (N + S::BN - 1) / S::BN;
+  int group_m = tiles_m < 8 ? tiles_m : 8;
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(S::kThreads), S::kLdsBytes, stream, W, X, C, ldc, M, N,
+                     K, tiles_m, tiles_n, group_m);
+  return hipGetLastError();
+}
+
+template <class S>
+static hipError_t launch_shape(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
+                               bool vec, bool out_f32, hipStream_t stream) {
+  if (vec) {
+    return out_f32 ? launch_tile<S, true, true>(W, X, C, ldc, M, N, K, stream)
+                   : launch_tile<S, true, false>(W, X, C, ldc, M, N, K, stream);
+  }
+  return out_f32 ? launch_tile<S, false, true>(W, X, C, ldc, M, N, K, stream)
+                 : launch_tile<S, false, false>(W, X, C, ldc, M, N, K, stream);
+}
+
+// Tile shapes. Which one runs is a pure performance choice (see det_gemm_tile.h).
+using Shape256x256 = TileShape<256, 256, 2, 4>;
+using Shape256x128 = TileShape<256, 128, 4, 2>;
+using Shape128x128 = TileShape<128, 128, 2, 2>;
+using Shape128x64 = TileShape<128, 64, 4, 1>;
+using Shape64x64 = TileShape<64, 64, 2, 2>;
+using Shape64x16 = TileShape<64, 16, 4, 1>;
+using Shape16x16 = TileShape<16, 16, 1, 1>;
+
+static bool view_is_vectorizable(const MatView& v) {
+  return v.k_stride == 1 && (v.row_stride % kChunkElems) == 0 &&
+         (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0;
+}
+
+static int64_t tile_count(int M, int N, int bm, int bn) {
+  return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+}
+
+int pick_det_gemm_config(int M, int N, int K) {
+  (void)K;
+  constexpr int kCus = 256;
+  if (M <= 16) return N >= 64 * kCus ? RLK_GEMM_CFG_64x16 : RLK_GEMM_CFG_16x16;
+  if (tile_count(M, N, 256, 256) >= 2 * kCus) return RLK_GEMM_CFG_256x256;
+  if (M >= 128 && tile_count(M, N, 128, 256) >= kCus) return RLK_GEMM_CFG_256x128;
+  if (M >= 128 && tile_count(M, N, 128, 128) >= kCus) return RLK_GEMM_CFG_128x128;
+  if (M > 64 && tile_count(M, N, 64, 128) >= kCus / 2) return RLK_GEMM_CFG_128x64;
+  return RLK_GEMM_CFG_64x64;
+}
+
+hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
+                           bool out_f32, int config, hipStream_t stream) {
+  const bool vec = view_is_vectorizable(W) && view_is_vectorizable(X) && (K % kChunkElems) == 0;
+  if (config == RLK_GEMM_CFG_AUTO) config = pick_det_gemm_config(M, N, K);
+  switch (config) {
+    case RLK_GEMM_CFG_256x256: return launch_shape<Shape256x256>(W, X, C, ldc, M, N, K, vec, out_f32, stream);
+    case RLK_GEMM_CFG_256x128: return launch_shape<Shape256x128>(W, X, C, ldc, M, N, K, vec, out_f32, stream);
+    case RLK_GEMM_CFG_128x128: return launch_shape<Shape128x128>(W, X, C, ldc, M, N, K, vec, out_f32, stream);
+    case RLK_GEMM_CFG_128x64: return launch_shape<Shape128x64>(W, X, C, ldc, M, N, K, vec, out_f32, stream);
+    case RLK_GEMM_CFG_64x64: return launch_shape<Shape64x64>(W, X, C, ldc, M, N, K, vec, out_f32, stream);
+    case RLK_GEMM_CFG_64x16: return launch_shape<Shape64x16>(W, X, C, ldc, M, N, K, vec, out_f32, stream);
+    case RLK_GEMM_CFG_16x16: return launch_shape<Shape16x16>(W, X, C, ldc, M, N, K, vec, out_f32, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace rlk
