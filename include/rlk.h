@@ -82,6 +82,77 @@ int rlk_det_gemm_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stride, c
  * Stands in for select_config, rl_engine/backends/rocm/gemm/mfma_gemm.py:76-92. */
 int rlk_det_gemm_pick_config(int M, int N, int K);
 
+/* Token-tile configurations of the fused linear-LogP kernel (bit-neutral). */
+typedef enum rlk_logp_config {
+  RLK_LOGP_CFG_AUTO = 0,
+  RLK_LOGP_CFG_256 = 1, /* 256 tokens per workgroup */
+  RLK_LOGP_CFG_128 = 2,
+  RLK_LOGP_CFG_64 = 3,
+  RLK_LOGP_CFG_16 = 4,
+  RLK_LOGP_CFG_COUNT = 5
+} rlk_logp_config;
+
+/* Reduction contract identifier of the fused linear-LogP.
+ * Stands in for TRITON_LINEAR_LOGP_CONTRACT_VERSION,
+ * rl_engine/backends/shared/triton/logprob/linear_logp.py:273. */
+const char* rlk_linear_logp_contract_id(void);
+
+/* Number of fixed vocabulary splits for a local vocabulary of V rows: ceil(V / 1024),
+ * a function of V only. Stands in for TRITON_N_SPLIT_CONTRACT / N_SPLIT_CONTRACT
+ * (linear_logp.py:274; csrc/cuda/logprob/fused_linear_logp_sm90.cu:50, 2120-2124). */
+int rlk_linear_logp_split_count(int V);
+
+/* Bytes of fp32 partials rlk_linear_logp_fwd needs for T tokens and V vocabulary rows. */
+size_t rlk_linear_logp_workspace_bytes(int T, int V);
+
+/*
+ * Fused lm_head GEMM -> fixed-order online log-sum-exp -> target gather.
+ *   hidden  [T, D] bf16, row stride h_row_stride, unit stride along D
+ *   weight  [V, D] bf16, row stride w_row_stride, unit stride along D (native lm_head layout)
+ *   target  [T] int64 GLOBAL vocabulary ids; the local column is target - vocab_start
+ *   bias    [V] fp32 or NULL;  temperature [T] fp32 (> 0) or NULL
+ *   logp    [T] fp32 out (may be NULL): min(y_target - lse, 0)
+ *   lse     [T] fp32 out (may be NULL)
+ *   real_vocab_end: local column bound of the real vocabulary (columns >= it are
+ *                   padding and contribute -inf / 0); pass V for "no padding".
+ * A target outside [vocab_start, vocab_start + real_vocab_end) contributes a target
+ * logit of 0 (range checking is the caller's job, as in the reference's Python
+ * layer, linear_logp.py:664-672). The full [T, V] logits are never written.
+ *
+ * Stands in for rl_engine._C.fused_linear_logp_sm90 (csrc/bindings/ops.cpp:514-526;
+ * csrc/cuda/logprob/fused_linear_logp_sm90.cu:2040-2176), for
+ * triton_deterministic_linear_logp (linear_logp.py:631-700) and for the ROCm route
+ * DetGemmOp().linear + _C.hip_deterministic_logp_tile_stats
+ * (rl_engine/integrations/common/linear_logp.py:1083-1102; csrc/bindings/ops.cpp:122-126).
+ */
+int rlk_linear_logp_fwd(const void* hidden, int64_t h_row_stride, const void* weight, int64_t w_row_stride,
+                        const int64_t* target, const float* bias, const float* temperature, float* logp,
+                        float* lse, void* workspace, size_t workspace_bytes, int T, int D, int V,
+                        int64_t vocab_start, int real_vocab_end, int config, void* stream);
+
+/* Bytes of workspace rlk_grpo_ratio_kl_loss needs. */
+size_t rlk_grpo_workspace_bytes(int rollouts);
+
+/*
+ * GRPO epilogue on per-token log-probs (all fp32):
+ *   ratio = exp(logp - old_logp);  d = ref_logp - logp;  k3 = exp(d) - d - 1
+ *   term  = -min(ratio * A, clamp(ratio, 1 - clip_eps, 1 + clip_eps) * A)
+ *   policy_loss = sum(term) / max(active, 1e-8);  kl = sum(k3) / max(active, 1e-8)
+ *   loss = policy_loss + beta * kl          out3 = {loss, policy_loss, kl}
+ * with masked entries (mask byte == 0) set to zero and excluded from the count.
+ * logp/old/ref/ratio/k3 are [rollouts * tokens_per_rollout] sequence-major,
+ * advantages is [rollouts]; mask, ratio and k3 may be NULL. Sums run per sequence
+ * in a fixed tree, then over sequences ascending.
+ *
+ * Stands in for compute_policy_ratio / compute_reference_kl / masked_mean
+ * (rl_engine/reference/definitions.py:50-106) and NativeGRPOLossOp.apply
+ * (rl_engine/reference/loss/grpo_loss.py:96-125, 162-168).
+ */
+int rlk_grpo_ratio_kl_loss(const float* logp, const float* old_logp, const float* ref_logp,
+                           const float* advantages, const uint8_t* mask, int rollouts, int tokens_per_rollout,
+                           float clip_eps, float beta, float* ratio, float* k3, float* out3, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

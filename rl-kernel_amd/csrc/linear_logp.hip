@@ -1,0 +1,289 @@
+// Fused linear-LogP for gfx950: lm_head GEMM -> online log-sum-exp over the
+// vocabulary in a fixed order -> target-token gather. The [tokens, vocab] logits
+// never leave registers.
+//
+// Stands in for rl_engine._C.fused_linear_logp_sm90 (reference
+// csrc/cuda/logprob/fused_linear_logp_sm90.cu:104-325, 488-513, 2040-2176), for
+// triton_deterministic_linear_logp (rl_engine/backends/shared/triton/logprob/
+// linear_logp.py:277-418, 631-700) and for the unfused ROCm route
+// DetGemmOp().linear + hip_deterministic_logp_tile_stats
+// (rl_engine/integrations/common/linear_logp.py:1083-1102).
+//
+// Reduction contract (everything that decides the bits of logp / lse; all of it
+// is a function of the vocabulary axis only, never of the token count, the
+// position of a token in the batch or the launch geometry):
+//   z_v   = fp32 MFMA chain of det_gemm over the hidden dimension, + bias_v
+//   y_v   = z_v                      (v < real vocabulary bound)
+//         = -inf                     (padded lane)
+//         then y_v * (1 / temperature) when a temperature is given
+//   tile  = 256 consecutive vocabulary columns; stream j (0..15) of a tile is
+//           its columns [16 j, 16 j + 16)
+//   split = 4 consecutive tiles (1024 columns); n_split = ceil(V / 1024)
+//   stream chain (per split, per j), tiles ascending, state (m, s) = (-inf, 0):
+//           t = max of the 16 y;  n = max(m, t);
+//           if n > -inf:  s = s * e(m - n) + (((e(y0 - n) + e(y1 - n)) + ...) + e(y15 - n));  m = n
+//   split merge:  M = max_j m_j;  S = sum over j ascending of s_j * e(m_j - M)  (terms with m_j = -inf skipped)
+//   final merge over splits ascending with the same formula;
+//   lse = M + log(S);  zt = y_target;  logp = min(zt - lse, 0)
+//   e(x) = v_exp_f32(x * log2(e)) with an unfused fp32 multiply.
+#include "det_gemm_tile.h"
+#include "rlk_host.h"
+
+namespace rlk {
+
+constexpr int kLogpTileCols = 256;
+constexpr int kLogpStreams = 16;
+constexpr int kLogpSplitTiles = 4;
+constexpr int kLogpSplitCols = kLogpTileCols * kLogpSplitTiles;
+constexpr float kNegInf = -__builtin_huge_valf();
+
+__device__ __forceinline__ float pinned_exp(float x) {
+  return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
+}
+
+struct LogpArgs {
+  MatView W;  // [V, D] lm_head weight, rows = vocabulary
+  MatView H;  // [T, D] hidden states, rows = tokens
+  const int64_t* target;     // [T] global vocabulary ids
+  const float* bias;         // [V] or null
+  const float* temperature;  // [T] or null
+  float* part;               // [3][n_split][T]: max, sum, target logit
+  int T, V, D;
+  int vocab_limit;  // local column bound of the real vocabulary (<= V)
+  int64_t vocab_start;
+  int tiles_m, n_split, group_m;
+};
+
+template <class S, bool VEC>
+__global__ __launch_bounds__(S::kThreads) void linear_logp_partial_kernel(LogpArgs a) {
+  static_assert(S::BN == kLogpTileCols && S::kRun == 16 && S::WN == 4, "stream layout is pinned");
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int total = a.tiles_m * a.n_split;
+  const int id = xcd_compact_id(blockIdx.x, total);
+  const int per_group = a.group_m * a.n_split;
+  const int group = id / per_group;
+  const int first_m = group * a.group_m;
+  const int width = (a.tiles_m - first_m) < a.group_m ? (a.tiles_m - first_m) : a.group_m;
+  const int within = id - group * per_group;
+  const int tile_m = first_m + within % width;
+  const int split = within / width;
+  const int m0 = tile_m * S::BM;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wave_n = wave % S::WN;
+  const int wave_m = wave / S::WN;
+  const int l16 = lane & 15;
+  const int grp = lane >> 4;
+  const int stream = wave_n * 4 + grp;
+  const int tok_local = wave_m * 16 * S::TM + l16;
+
+  float run_m[S::TM], run_s[S::TM], run_zt[S::TM], inv_t[S::TM];
+  int tgt[S::TM];
+#pragma unroll
+  for (int jm = 0; jm < S::TM; ++jm) {
+    const int m = m0 + tok_local + jm * 16;
+    run_m[jm] = kNegInf;
+    run_s[jm] = 0.f;
+    run_zt[jm] = 0.f;
+    inv_t[jm] = 1.0f;
+    tgt[jm] = -1;
+    if (m < a.T) {
+      const int64_t local = a.target[m] - a.vocab_start;
+      tgt[jm] = (local >= 0 && local < a.vocab_limit) ? (int)local : -1;
+      if (a.temperature) inv_t[jm] = 1.0f / a.temperature[m];
+    }
+  }
+
+  for (int t = 0; t < kLogpSplitTiles; ++t) {
+    const int v0 = split * kLogpSplitCols + t * kLogpTileCols;
+    if (v0 >= a.V) break;
+    f32x4_t acc[S::TN][S::TM];
+    tile_mainloop<S, VEC>(a.W, a.H, v0, m0, a.D, lds, acc);
+
+    const int col0 = v0 + stream * 16;  // first column of this lane's run
+    float bias_run[16];
+#pragma unroll
+    for (int c = 0; c < 16; ++c) bias_run[c] = 0.f;
+    if (a.bias) {
+#pragma unroll
+      for (int c = 0; c < 16; ++c) bias_run[c] = (col0 + c < a.V) ? a.bias[col0 + c] : 0.f;
+    }
+#pragma unroll
+    for (int jm = 0; jm < S::TM; ++jm) {
+      float y[16];
+      float tmax = kNegInf;
+#pragma unroll
+      for (int c = 0; c < 16; ++c) {
+        float z = acc[c >> 2][jm][c & 3];
+        if (a.bias) z = z + bias_run[c];
+        z = (col0 + c < a.vocab_limit) ? z : kNegInf;
+        if (a.temperature) z = z * inv_t[jm];
+        y[c] = z;
+        tmax = fmaxf(tmax, z);
+      }
+      const int tl = tgt[jm] - col0;
+      if (tl >= 0 && tl < 16) {
+        float sel = y[0];
+#pragma unroll
+        for (int c = 1; c < 16; ++c) sel = (tl == c) ? y[c] : sel;
+        run_zt[jm] = sel;
+      }
+      const float old_m = run_m[jm];
+      const float new_m = fmaxf(old_m, tmax);
+      float sum = pinned_exp(y[0] - new_m);
+#pragma unroll
+      for (int c = 1; c < 16; ++c) sum = sum + pinned_exp(y[c] - new_m);
+      const float scaled = run_s[jm] * pinned_exp(old_m - new_m);
+      const bool live = new_m > kNegInf;
+      run_s[jm] = live ? (scaled + sum) : run_s[jm];
+      run_m[jm] = new_m;
+    }
+  }
+
+  // Fold the 16 streams of every token in ascending stream order. The main loop
+  // ended on a barrier, so the staging LDS is free.
+  float* xm = reinterpret_cast<float*>(lds);
+  float* xs = xm + kLogpStreams * S::BM;
+  float* xz = xs + kLogpStreams * S::BM;
+#pragma unroll
+  for (int jm = 0; jm < S::TM; ++jm) {
+    const int slot = stream * S::BM + tok_local + jm * 16;
+    xm[slot] = run_m[jm];
+    xs[slot] = run_s[jm];
+    xz[slot] = run_zt[jm];
+  }
+  __syncthreads();
+  for (int tok = threadIdx.x; tok < S::BM; tok += S::kThreads) {
+    const int m = m0 + tok;
+    if (m >= a.T) continue;
+    float big = kNegInf;
+#pragma unroll
+    for (int j = 0; j < kLogpStreams; ++j) big = fmaxf(big, xm[j * S::BM + tok]);
+    float sum = 0.f, zt = 0.f;
+#pragma unroll
+    for (int j = 0; j < kLogpStreams; ++j) {
+      const float pm = xm[j * S::BM + tok];
+      const float term = xs[j * S::BM + tok] * pinned_exp(pm - big);
+      sum = sum + ((pm > kNegInf) ? term : 0.f);
+      zt = zt + xz[j * S::BM + tok];
+    }
+    const int64_t plane = (int64_t)a.n_split * a.T;
+    const int64_t at = (int64_t)split * a.T + m;
+    a.part[at] = big;
+    a.part[plane + at] = sum;
+    a.part[2 * plane + at] = zt;
+  }
+}
+
+__global__ void linear_logp_merge_kernel(const float* __restrict__ part, float* __restrict__ logp,
+                                         float* __restrict__ lse, int T, int n_split) {
+  const int m = blockIdx.x * blockDim.x + threadIdx.x;
+  if (m >= T) return;
+  const int64_t plane = (int64_t)n_split * T;
+  float big = kNegInf;
+  for (int p = 0; p < n_split; ++p) big = fmaxf(big, part[(int64_t)p * T + m]);
+  float sum = 0.f, zt = 0.f;
+  for (int p = 0; p < n_split; ++p) {
+    const float pm = part[(int64_t)p * T + m];
+    const float term = part[plane + (int64_t)p * T + m] * pinned_exp(pm - big);
+    sum = sum + ((pm > kNegInf) ? term : 0.f);
+    zt = zt + part[2 * plane + (int64_t)p * T + m];
+  }
+  const float l = big + logf(sum);
+  if (lse) lse[m] = l;
+  if (logp) logp[m] = fminf(zt - l, 0.f);
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+
+using LogpShape256 = TileShape<256, 256, 4, 2>;
+using LogpShape128 = TileShape<256, 128, 4, 2>;
+using LogpShape64 = TileShape<256, 64, 4, 1>;
+using LogpShape16 = TileShape<256, 16, 4, 1>;
+
+int linear_logp_split_count(int V) { return (V + kLogpSplitCols - 1) / kLogpSplitCols; }
+
+size_t linear_logp_workspace_bytes(int T, int V) {
+  return (size_t)3 * linear_logp_split_count(V) * (size_t)(T > 0 ? T : 0) * sizeof(float);
+}
+
+template <class S, bool VEC>
+static hipError_t launch_logp(LogpArgs a, hipStream_t stream) {
+  auto kernel = linear_logp_partial_kernel<S, VEC>;
+  constexpr int kMergeBytes = 3 * kLogpStreams * S::BM * (int)sizeof(float);
+  constexpr int kLds = S::kLdsBytes > kMergeBytes ? S::kLdsBytes : kMergeBytes;
+  static bool configured[kMaxDevices] = {};
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev >= 0 && dev < kMaxDevices && !configured[dev]) {
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              kLds);
+    if (err != hipSuccess) return err;
+    configured[dev] = true;
+  }
+  a.tiles_m = (a.T + S::BM - 1) / S::BM;
+  a.group_m = a.tiles_m < 8 ? a.tiles_m : 8;
+  hipLaunchKernelGGL(kernel, dim3(a.tiles_m * a.n_split), dim3(S::kThreads), kLds, stream, a);
+  return hipGetLastError();
+}
+
+int pick_linear_logp_config(int T, int V) {
+  (void)V;
+  if (T <= 16) return RLK_LOGP_CFG_16;
+  if (T <= 64) return RLK_LOGP_CFG_64;
+  if (T <= 2048) return RLK_LOGP_CFG_128;
+  return RLK_LOGP_CFG_256;
+}
+
+hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t* target, const float* bias,
+                              const float* temperature, float* logp, float* lse, float* workspace, int T, int D,
+                              int V, int64_t vocab_start, int vocab_limit, int config, hipStream_t stream) {
+  LogpArgs a;
+  a.W = W;
+  a.H = H;
+  a.target = target;
+  a.bias = bias;
+  a.temperature = temperature;
+  a.part = workspace;
+  a.T = T;
+  a.V = V;
+  a.D = D;
+  a.vocab_limit = vocab_limit;
+  a.vocab_start = vocab_start;
+  a.n_split = linear_logp_split_count(V);
+  a.tiles_m = 0;
+  a.group_m = 1;
+  const bool vec = W.k_stride == 1 && H.k_stride == 1 && (W.row_stride % kChunkElems) == 0 &&
+                   (H.row_stride % kChunkElems) == 0 && (reinterpret_cast<uintptr_t>(W.ptr) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(H.ptr) & 15) == 0 && (D % kChunkElems) == 0;
+  if (config == RLK_LOGP_CFG_AUTO) config = pick_linear_logp_config(T, V);
+  if (!vec && config == RLK_LOGP_CFG_256) config = RLK_LOGP_CFG_128;
+  hipError_t err;
+  switch (config) {
+    case RLK_LOGP_CFG_256:
+      err = launch_logp<LogpShape256, true>(a, stream);
+      break;
+    case RLK_LOGP_CFG_128:
+      err = vec ? launch_logp<LogpShape128, true>(a, stream) : launch_logp<LogpShape128, false>(a, stream);
+      break;
+    case RLK_LOGP_CFG_64:
+      err = vec ? launch_logp<LogpShape64, true>(a, stream) : launch_logp<LogpShape64, false>(a, stream);
+      break;
+    case RLK_LOGP_CFG_16:
+      err = vec ? launch_logp<LogpShape16, true>(a, stream) : launch_logp<LogpShape16, false>(a, stream);
+      break;
+    default:
+      return hipErrorInvalidValue;
+  }
+  if (err != hipSuccess) return err;
+  hipLaunchKernelGGL(linear_logp_merge_kernel, dim3((T + 255) / 256), dim3(256), 0, stream, workspace, logp, lse, T,
+                     a.n_split);
+  return hipGetLastError();
+}
+
+}  // namespace rlk

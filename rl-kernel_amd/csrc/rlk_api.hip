@@ -89,4 +89,80 @@ int rlk_det_gemm_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stride, c
   return err == hipSuccess ? RLK_OK : device_error("rlk_det_gemm_bf16", err);
 }
 
+const char* rlk_linear_logp_contract_id(void) { return "rlkernel.linear_logp.hip_streams16x256_split1024_gfx950.v1"; }
+
+int rlk_linear_logp_split_count(int V) { return V > 0 ? linear_logp_split_count(V) : 0; }
+
+size_t rlk_linear_logp_workspace_bytes(int T, int V) {
+  if (T <= 0 || V <= 0) return 0;
+  return linear_logp_workspace_bytes(T, V);
+}
+
+int rlk_linear_logp_fwd(const void* hidden, int64_t h_row_stride, const void* weight, int64_t w_row_stride,
+                        const int64_t* target, const float* bias, const float* temperature, float* logp,
+                        float* lse, void* workspace, size_t workspace_bytes, int T, int D, int V,
+                        int64_t vocab_start, int real_vocab_end, int config, void* stream) {
+  if (T < 0 || D <= 0 || V <= 0) {
+    set_last_error("rlk_linear_logp_fwd: bad sizes T=%d D=%d V=%d", T, D, V);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (real_vocab_end <= 0 || real_vocab_end > V) {
+    set_last_error("rlk_linear_logp_fwd: real_vocab_end must be in [1, %d], got %d", V, real_vocab_end);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (config < 0 || config >= RLK_LOGP_CFG_COUNT) {
+    set_last_error("rlk_linear_logp_fwd: unknown config %d", config);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (T == 0) return RLK_OK;
+  if (hidden == nullptr || weight == nullptr || target == nullptr) {
+    set_last_error("rlk_linear_logp_fwd: null hidden / weight / target");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (h_row_stride < D || w_row_stride < D) {
+    set_last_error("rlk_linear_logp_fwd: row strides must be >= D");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  const size_t need = linear_logp_workspace_bytes(T, V);
+  if (workspace == nullptr || workspace_bytes < need) {
+    set_last_error("rlk_linear_logp_fwd: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  MatView H{reinterpret_cast<const bf16_bits*>(hidden), h_row_stride, 1, T};
+  MatView W{reinterpret_cast<const bf16_bits*>(weight), w_row_stride, 1, V};
+  hipError_t err = linear_logp_launch(H, W, target, bias, temperature, logp, lse, reinterpret_cast<float*>(workspace),
+                                      T, D, V, vocab_start, real_vocab_end, config,
+                                      reinterpret_cast<hipStream_t>(stream));
+  return err == hipSuccess ? RLK_OK : device_error("rlk_linear_logp_fwd", err);
+}
+
+size_t rlk_grpo_workspace_bytes(int rollouts) { return rollouts > 0 ? (size_t)3 * rollouts * sizeof(float) : 0; }
+
+int rlk_grpo_ratio_kl_loss(const float* logp, const float* old_logp, const float* ref_logp,
+                           const float* advantages, const uint8_t* mask, int rollouts, int tokens_per_rollout,
+                           float clip_eps, float beta, float* ratio, float* k3, float* out3, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+  if (rollouts < 0 || tokens_per_rollout < 0) {
+    set_last_error("rlk_grpo_ratio_kl_loss: negative sizes");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (out3 == nullptr) {
+    set_last_error("rlk_grpo_ratio_kl_loss: out3 is required");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (rollouts > 0 && (logp == nullptr || old_logp == nullptr || ref_logp == nullptr || advantages == nullptr)) {
+    set_last_error("rlk_grpo_ratio_kl_loss: null input");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (rollouts > 0 && (workspace == nullptr || workspace_bytes < rlk_grpo_workspace_bytes(rollouts))) {
+    set_last_error("rlk_grpo_ratio_kl_loss: workspace of %zu bytes needed, %zu given",
+                   rlk_grpo_workspace_bytes(rollouts), workspace_bytes);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  hipError_t err = grpo_launch(logp, old_logp, ref_logp, advantages, mask, rollouts, tokens_per_rollout, clip_eps,
+                               beta, ratio, k3, out3, reinterpret_cast<float*>(workspace),
+                               reinterpret_cast<hipStream_t>(stream));
+  return err == hipSuccess ? RLK_OK : device_error("rlk_grpo_ratio_kl_loss", err);
+}
+
 }  // extern "C"

@@ -21,6 +21,21 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
 hipError_t fill_zero_launch(void* dst, int64_t rows, int64_t cols, int64_t ld, int elem_bytes,
                             hipStream_t stream);
 
+int pick_linear_logp_config(int T, int V);
+int linear_logp_split_count(int V);
+size_t linear_logp_workspace_bytes(int T, int V);
+
+// H[T,D] hidden states, W[V,D] lm_head weight; workspace holds
+// linear_logp_workspace_bytes(T, V) bytes of fp32 partials.
+hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t* target, const float* bias,
+                              const float* temperature, float* logp, float* lse, float* workspace, int T, int D,
+                              int V, int64_t vocab_start, int vocab_limit, int config, hipStream_t stream);
+
+// workspace: 3 * rollouts floats.
+hipError_t grpo_launch(const float* logp, const float* old_logp, const float* ref_logp, const float* advantages,
+                       const uint8_t* mask, int rollouts, int tokens, float clip_eps, float beta, float* ratio,
+                       float* k3, float* out3, float* workspace, hipStream_t stream);
+
 void set_last_error(const char* fmt, ...);
 
 }  // namespace rlk
