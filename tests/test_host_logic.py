@@ -1,0 +1,206 @@
+"""Host-side checks that need no GPU: the C ABI exports what include/rlk.h
+declares, shape heuristics are pure functions, and the Python layer raises the
+reference's errors before any kernel is launched."""
+
+from __future__ import annotations
+
+import ctypes
+import re
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+import torch
+
+REPO_ROOT = Path(__file__).resolve().parent.parent
+HEADER = REPO_ROOT / "include" / "rlk.h"
+
+
+def _declared_functions() -> list[str]:
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(rlk_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = _declared_functions()
+    for required in ("rlk_det_gemm_bf16", "rlk_linear_logp_fwd", "rlk_grpo_ratio_kl_loss", "rlk_contract_id"):
+        assert required in names
+
+
+def test_library_exports_every_declared_symbol(rlk_lib):
+    for name in _declared_functions():
+        assert hasattr(rlk_lib, name), f"{name} declared in include/rlk.h but not exported"
+
+
+def test_python_binding_lists_the_same_symbols():
+    from rl_engine import _lib
+
+    assert sorted(_lib.EXPORTED_SYMBOLS) == _declared_functions()
+
+
+def test_header_compiles_as_plain_c(tmp_path):
+    src = tmp_path / "use_rlk.c"
+    src.write_text('#include "rlk.h"\nint main(void) { return (int)RLK_GEMM_CFG_COUNT - 8; }\n')
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", str(HEADER.parent), "-c", str(src), "-o", str(tmp_path / "o.o")], check=True)
+
+
+def test_contract_ids_and_version(rlk_lib):
+    assert rlk_lib.rlk_contract_id().decode().startswith("rlkernel.det_gemm.")
+    assert rlk_lib.rlk_linear_logp_contract_id().decode().startswith("rlkernel.linear_logp.")
+    assert re.fullmatch(r"\d+\.\d+\.\d+", rlk_lib.rlk_version().decode())
+
+
+def test_split_count_is_a_function_of_vocab_only(rlk_lib):
+    assert rlk_lib.rlk_linear_logp_split_count(151936) == 149  # ceil(151936 / 1024)
+    assert rlk_lib.rlk_linear_logp_split_count(1024) == 1
+    assert rlk_lib.rlk_linear_logp_split_count(1025) == 2
+    assert rlk_lib.rlk_linear_logp_split_count(0) == 0
+    assert rlk_lib.rlk_linear_logp_workspace_bytes(8192, 151936) == 3 * 149 * 8192 * 4
+    assert rlk_lib.rlk_grpo_workspace_bytes(64) == 3 * 64 * 4
+
+
+def test_config_pick_is_deterministic_and_in_range(rlk_lib):
+    from rl_engine import _lib
+
+    for m, n, k in ((1, 4096, 12288), (16, 24576, 4096), (256, 24576, 4096), (4096, 24576, 4096), (16384, 6144, 4096)):
+        first = rlk_lib.rlk_det_gemm_pick_config(m, n, k)
+        assert first == rlk_lib.rlk_det_gemm_pick_config(m, n, k)
+        assert 1 <= first < len(_lib.GEMM_CONFIGS)
+    assert rlk_lib.rlk_det_gemm_pick_config(4096, 24576, 4096) == _lib.GEMM_CONFIGS["256x256"]
+
+
+def test_argument_errors_are_reported_without_touching_the_gpu(rlk_lib):
+    # Invalid arguments are rejected before any HIP call, so this runs on a CPU-only host.
+    rc = rlk_lib.rlk_det_gemm_bf16(None, 4, 1, None, 1, 4, None, 4, -1, 4, 4, 0, 0, None)
+    assert rc == -1 and b"negative size" in rlk_lib.rlk_last_error()
+    rc = rlk_lib.rlk_det_gemm_bf16(None, -4, 1, None, 1, 4, None, 4, 2, 4, 4, 0, 0, None)
+    assert rc == -1 and b"negative strides" in rlk_lib.rlk_last_error()
+    rc = rlk_lib.rlk_det_gemm_bf16(None, 4, 1, None, 1, 4, None, 4, 2, 4, 4, 0, 99, None)
+    assert rc == -1 and b"unknown config" in rlk_lib.rlk_last_error()
+    assert rlk_lib.rlk_det_gemm_bf16(None, 4, 1, None, 1, 4, None, 4, 0, 4, 4, 0, 0, None) == 0  # empty M: no-op
+    rc = rlk_lib.rlk_linear_logp_fwd(None, 8, None, 8, None, None, None, None, None, None, 0, 4, 8, 16, 0, 17, 0, None)
+    assert rc == -1 and b"real_vocab_end" in rlk_lib.rlk_last_error()
+    rc = rlk_lib.rlk_linear_logp_fwd(None, 8, None, 8, None, None, None, None, None, None, 0, 4, 8, 16, 0, 16, 0, None)
+    assert rc == -1 and b"null hidden" in rlk_lib.rlk_last_error()
+    rc = rlk_lib.rlk_grpo_ratio_kl_loss(None, None, None, None, None, 2, 4, 0.2, 0.0, None, None, None, None, 0, None)
+    assert rc == -1 and b"out3" in rlk_lib.rlk_last_error()
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    code = (
+        "import os, sys\n"
+        f"sys.path.insert(0, {str(REPO_ROOT / 'rl-kernel_amd')!r})\n"
+        f"os.environ['RLK_LIBRARY'] = {str(tmp_path / 'nope.so')!r}\n"
+        "from rl_engine import _lib\n"
+        "try:\n"
+        "    _lib.load()\n"
+        "except _lib.RlkLibraryMissing as e:\n"
+        "    assert 'no fallback' in str(e).lower()\n"
+        "    sys.exit(0)\n"
+        "sys.exit(1)\n"
+    )
+    assert subprocess.run([sys.executable, "-c", code]).returncode == 0
+
+
+def test_product_never_imports_the_oracle():
+    pkg = REPO_ROOT / "rl-kernel_amd"
+    for path in list(pkg.rglob("*.py")) + list(pkg.rglob("*.hip")) + list(pkg.rglob("*.h")):
+        text = path.read_text()
+        assert "oracle" not in text.lower(), f"{path} mentions the oracle"
+
+
+# ---------------------------------------------------------------------------
+# Python surface: names and pre-launch validation (CPU tensors)
+# ---------------------------------------------------------------------------
+
+
+def test_ops_gemm_exports_the_reference_names():
+    import rl_engine.ops.gemm as pkg
+    import rl_engine.ops.gemm.det_gemm as mod
+
+    assert sorted(mod.__all__) == sorted(
+        [
+            "DetGemmOp",
+            "det_gemm_backend",
+            "det_gemm_backend_id",
+            "det_gemm_fallback_reason",
+            "det_gemm_linear",
+            "det_gemm_linear_input_gradient",
+            "det_gemm_linear_weight_gradient",
+            "deterministic_gemm",
+        ]
+    )
+    assert pkg.__all__ == ["DetGemmOp", "deterministic_gemm"]
+    assert mod.det_gemm_fallback_reason() is None
+    assert mod.det_gemm_backend() == "hip_mfma"
+    assert mod.det_gemm_backend_id().startswith("rlkernel.det_gemm.")
+    from rl_engine.backends.rocm.gemm import det_gemm as facade
+
+    for name in ("prepare_det_gemm_linear_weight", "det_gemm_linear_prepared", "refresh_cached_weight_transposes", "RocmDetGemmOp"):
+        assert hasattr(facade, name)
+
+
+def test_native_module_has_the_reference_function_names():
+    from rl_engine import _C
+
+    for name in ("det_gemm_sm90_compiled", "det_gemm_fwd", "det_gemm_fwd_rhs_transposed", "det_gemm_da", "det_gemm_db", "det_gemm_db_transposed", "fused_linear_logp"):
+        assert callable(getattr(_C, name))
+    assert _C.det_gemm_sm90_compiled() is False
+
+
+def test_native_checks_use_the_reference_error_strings():
+    from rl_engine import _C
+
+    a = torch.zeros((2, 4), dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="A must be CUDA"):
+        _C.det_gemm_fwd(a, a)
+    with pytest.raises(RuntimeError, match="dC must be CUDA"):
+        _C.det_gemm_da(a, a)
+
+
+def test_facade_validation_matches_the_reference_error_types():
+    from rl_engine.backends.rocm.gemm import det_gemm as facade
+
+    a = torch.zeros((2, 4), dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="two 2-D tensors"):
+        facade.mfma_gemm(a[0], a)
+    with pytest.raises(ValueError, match="K mismatch"):
+        facade.mfma_gemm(a, a)
+    with pytest.raises(TypeError, match="requires BF16 inputs"):
+        facade.mfma_gemm(a.float(), a.float().t())
+    with pytest.raises(RuntimeError, match="share one ROCm device"):
+        facade.mfma_gemm(a, a.t())
+    op = facade.DetGemmOp()
+    with pytest.raises(AssertionError, match="BF16 only"):
+        op(a.float(), a.float().t())
+    with pytest.raises(AssertionError, match="ROCm device"):
+        op(a, a.t())
+    with pytest.raises(TypeError, match="must be BF16"):
+        facade.prepare_det_gemm_linear_weight(a.float())
+    with pytest.raises(ValueError, match="must be 2-D"):
+        facade.prepare_det_gemm_linear_weight(a[0])
+
+
+def test_linear_logp_python_validation():
+    from rl_engine.ops.logprob import LinearLogpOp, deterministic_linear_logp
+
+    h = torch.zeros((3, 8), dtype=torch.bfloat16)
+    w = torch.zeros((16, 8), dtype=torch.bfloat16)
+    t = torch.zeros((3,), dtype=torch.long)
+    with pytest.raises(RuntimeError, match="requires a GPU tensor"):
+        deterministic_linear_logp(h, w, t)
+    op = LinearLogpOp()
+    with pytest.raises(ValueError, match="leading shape"):
+        op(h, w, t[:2])
+    with pytest.raises(ValueError, match="must match lm_head_weight dim"):
+        op(h, torch.zeros((16, 4), dtype=torch.bfloat16), t)
+
+
+def test_ctypes_prototypes_cover_every_argument(rlk_lib):
+    # A prototype with the wrong arity would corrupt the call; compare with the header.
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    for name in ("rlk_det_gemm_bf16", "rlk_linear_logp_fwd", "rlk_grpo_ratio_kl_loss"):
+        params = re.search(name + r"\s*\((.*?)\)\s*;", text, flags=re.S).group(1)
+        assert len(getattr(rlk_lib, name).argtypes) == params.count(",") + 1, name
+    assert rlk_lib.rlk_linear_logp_workspace_bytes.restype is ctypes.c_size_t

@@ -1,0 +1,296 @@
+"""Fused linear-LogP and the GRPO epilogue on a real MI355X, through the C ABI.
+
+Tolerance for this path: |logp - oracle| <= 1e-3 nats (the reference's own bar
+against the fp32-upcast native op is 2e-2, tests/ops/logprob/test_linear_logp.py:617);
+determinism and batch invariance are bit-exact."""
+
+from __future__ import annotations
+
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import inputs
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+TOL_NATS = 1e-3
+GOLDEN = Path(__file__).parent / "golden"
+
+
+@pytest.fixture(scope="module")
+def logp_mod():
+    from rl_engine.ops import logprob
+
+    return logprob
+
+
+@pytest.fixture(scope="module")
+def loss_mod():
+    from rl_engine.ops import loss
+
+    return loss
+
+
+def _same_bits(x: torch.Tensor, y: torch.Tensor) -> bool:
+    return torch.equal(x.contiguous().view(torch.int32), y.contiguous().view(torch.int32))
+
+
+def test_golden_small_case(logp_mod):
+    d = np.load(GOLDEN / "small_linear_logp.npz")
+    h = inputs.from_bits(d["hidden_bits"], DEV)
+    w = inputs.from_bits(d["weight_bits"], DEV)
+    t = torch.from_numpy(d["target"]).to(DEV)
+    logp, lse = logp_mod.deterministic_linear_logp(h, w, t)
+    assert logp.dtype == torch.float32 and logp.shape == (48,)
+    assert np.abs(logp.cpu().numpy() - d["logp"]).max() < 1e-4
+    assert np.abs(lse.cpu().numpy() - d["lse"]).max() < 1e-4
+    logp2, lse2 = logp_mod.deterministic_linear_logp(
+        h,
+        w,
+        t % 1900,
+        torch.from_numpy(d["bias"]).to(DEV),
+        temperature=torch.from_numpy(d["temperature"]).to(DEV),
+        real_vocab_size=1900,
+    )
+    assert np.abs(logp2.cpu().numpy() - d["logp_bias_temp_pad"]).max() < 1e-4
+    assert np.abs(lse2.cpu().numpy() - d["lse_bias_temp_pad"]).max() < 1e-4
+    assert bool((logp2 <= 0).all())
+
+
+@pytest.mark.parametrize("shape", [(40, 3000, 264), (300, 2500, 128), (5, 1024, 64), (130, 5000, 512), (96, 4099, 320)])
+def test_parity_with_oracle_and_config_neutrality(logp_mod, oracle, shape):
+    from rl_engine import _lib
+
+    t, v, d = shape
+    h, w, target = inputs.logp_inputs(t, vocab=v, hidden=d, seed=4200 + t, rms_norm=False)
+    w = (w.float() * 2.5).to(torch.bfloat16)  # sigma 0.05: a wider logit spread than N(0, 0.02)
+    ref_logp, ref_lse = oracle.linear_logp_chunked(inputs.bits(h), inputs.bits(w), target.numpy(), chunk_elems=t * 700)[:2]
+    dense_logp = oracle.linear_logp_dense(inputs.bits(h), inputs.bits(w), target.numpy())[0]
+    h_d, w_d, t_d = h.to(DEV), w.to(DEV), target.to(DEV)
+    base = None
+    for name in ("256", "128", "64", "16", "auto"):
+        logp, lse = logp_mod.deterministic_linear_logp(h_d, w_d, t_d, config=name)
+        assert np.abs(logp.cpu().numpy() - ref_logp).max() <= TOL_NATS
+        assert np.abs(lse.cpu().numpy() - ref_lse).max() <= TOL_NATS
+        assert np.abs(logp.cpu().numpy() - dense_logp).max() <= TOL_NATS
+        if base is None:
+            base = (logp, lse)
+        assert _same_bits(logp, base[0]) and _same_bits(lse, base[1]), name
+    assert np.abs(base[0].cpu().numpy() - ref_logp).max() < 5e-5  # what the kernel actually achieves
+
+
+def test_row_alone_equals_row_in_batch_with_bias_temperature_padding(logp_mod):
+    # The strict-contract invariance check: row 37 alone vs inside N=96, int32 views,
+    # with bias + temperature + padded vocabulary (tests/ops/logprob/test_linear_logp.py:1428-1463).
+    n, d, v, real = 96, 256, 3072, 3000
+    h, w, target = inputs.logp_inputs(n, vocab=v, hidden=d, seed=4300, rms_norm=False)
+    target = target % real
+    g = torch.Generator().manual_seed(4301)
+    bias = (torch.randn(v, generator=g) * 0.3).to(DEV)
+    temp = (0.5 + torch.rand(n, generator=g)).to(DEV)
+    h_d, w_d, t_d = h.to(DEV), w.to(DEV), target.to(DEV)
+    logp, lse = logp_mod.deterministic_linear_logp(h_d, w_d, t_d, bias, temperature=temp, real_vocab_size=real)
+    for row in (0, 37, 95):
+        one_lp, one_lse = logp_mod.deterministic_linear_logp(
+            h_d[row : row + 1], w_d, t_d[row : row + 1], bias, temperature=temp[row : row + 1], real_vocab_size=real
+        )
+        assert _same_bits(one_lp, logp[row : row + 1]) and _same_bits(one_lse, lse[row : row + 1]), row
+    # return_logits must not change logp / lse bits and exposes unscaled, bias-applied, padded logits
+    lp2, lse2, logits = logp_mod.deterministic_linear_logp(
+        h_d, w_d, t_d, bias, temperature=temp, real_vocab_size=real, return_logits=True
+    )
+    assert _same_bits(lp2, logp) and _same_bits(lse2, lse)
+    assert logits.shape == (n, v) and bool(torch.isinf(logits[:, real:]).all()) and bool((logp <= 0).all())
+    probs = torch.softmax(logits.double() * (1.0 / temp.double())[:, None], dim=-1)
+    picked = probs[torch.arange(n, device=DEV), t_d].log()
+    assert float((picked - logp.double()).abs().max()) < 1e-4
+
+
+def test_layout_packing_invariance(logp_mod):
+    # Rows permuted across [2,3] / [3,2] / [1,6] layouts give the same per-row bits
+    # (tests/ops/logprob/test_linear_logp.py:339-367).
+    h, w, target = inputs.logp_inputs(6, vocab=2048, hidden=128, seed=4400, rms_norm=False)
+    h_d, w_d, t_d = h.to(DEV), w.to(DEV), target.to(DEV)
+    flat, _ = logp_mod.deterministic_linear_logp(h_d, w_d, t_d)
+    for lead in ((2, 3), (3, 2), (1, 6)):
+        out, lse = logp_mod.deterministic_linear_logp(h_d.view(*lead, 128), w_d, t_d.view(*lead))
+        assert out.shape == lead and lse.shape == lead and _same_bits(out.reshape(-1), flat)
+    perm = torch.tensor([4, 0, 5, 2, 1, 3], device=DEV)
+    out, _ = logp_mod.deterministic_linear_logp(h_d[perm], w_d, t_d[perm])
+    assert _same_bits(out, flat[perm])
+    op = logp_mod.LinearLogpOp()
+    assert _same_bits(op(h_d.view(2, 3, 128), w_d, t_d.view(2, 3)).reshape(-1), flat)
+    assert _same_bits(logp_mod.linear_logp(h_d, w_d, t_d), flat)
+
+
+def test_uniform_logits_and_target_checks(logp_mod):
+    v, d = 5000, 64
+    h = torch.zeros((4, d), dtype=torch.bfloat16, device=DEV)
+    w = inputs.randn_bf16(4500, v, d).to(DEV)
+    t = torch.tensor([0, 1, 4999, 2500], device=DEV)
+    logp, lse = logp_mod.deterministic_linear_logp(h, w, t)
+    assert torch.allclose(logp, torch.full_like(logp, -float(np.log(v))), atol=1e-5)
+    assert torch.allclose(lse, torch.full_like(lse, float(np.log(v))), atol=1e-5)
+    with pytest.raises(ValueError, match="real vocabulary"):
+        logp_mod.deterministic_linear_logp(h, w, torch.tensor([0, 1, 5000, 2], device=DEV))
+    with pytest.raises(ValueError, match="real_vocab_size"):
+        logp_mod.deterministic_linear_logp(h, w, t, real_vocab_size=v + 1)
+    with pytest.raises(ValueError, match="temperature"):
+        logp_mod.deterministic_linear_logp(h, w, t, temperature=torch.tensor([1.0, 0.0, 1.0, 1.0]))
+    with pytest.raises(ValueError, match="one id per hidden row"):
+        logp_mod.deterministic_linear_logp(h, w, t[:3])
+    hg = h.clone().requires_grad_(True)
+    with pytest.raises(RuntimeError, match="forward-only"):
+        logp_mod.deterministic_linear_logp(hg, w, t)
+
+
+def test_vocab_start_index_offsets_targets(logp_mod):
+    h, w, target = inputs.logp_inputs(9, vocab=1500, hidden=64, seed=4600, rms_norm=False)
+    h_d, w_d, t_d = h.to(DEV), w.to(DEV), target.to(DEV)
+    base, _ = logp_mod.deterministic_linear_logp(h_d, w_d, t_d)
+    shifted, _ = logp_mod.deterministic_linear_logp(h_d, w_d, t_d + 7000, vocab_start_index=7000)
+    assert _same_bits(base, shifted)
+
+
+# ---------------------------------------------------------------------------
+# Config 4 at full size: T=8192, V=151936, D=4096
+# ---------------------------------------------------------------------------
+
+
+@pytest.fixture(scope="module")
+def config4():
+    h, w, target = inputs.logp_inputs(8192)
+    return {"h": h, "w": w, "t": target, "h_d": h.to(DEV), "w_d": w.to(DEV), "t_d": target.to(DEV)}
+
+
+def test_config4_full_size(logp_mod, oracle, config4):
+    c = config4
+    logp, lse = logp_mod.deterministic_linear_logp(c["h_d"], c["w_d"], c["t_d"])
+    assert logp.shape == (8192,) and bool(torch.isfinite(logp).all()) and bool((logp <= 0).all())
+    # bit-exact run to run
+    logp_b, lse_b = logp_mod.deterministic_linear_logp(c["h_d"], c["w_d"], c["t_d"])
+    assert _same_bits(logp, logp_b) and _same_bits(lse, lse_b)
+    # bit-exact per row: M=1, M=7 and a ragged cut against the M=8192 batch
+    for lo, hi in ((0, 1), (0, 7), (4095, 4096), (8191, 8192), (5000, 5130)):
+        part, part_lse = logp_mod.deterministic_linear_logp(c["h_d"][lo:hi], c["w_d"], c["t_d"][lo:hi])
+        assert _same_bits(part, logp[lo:hi]) and _same_bits(part_lse, lse[lo:hi]), (lo, hi)
+    # a different packing of the same rows
+    perm = torch.randperm(8192, generator=torch.Generator().manual_seed(4002)).to(DEV)
+    packed, _ = logp_mod.deterministic_linear_logp(c["h_d"][perm], c["w_d"], c["t_d"][perm])
+    assert _same_bits(packed, logp[perm])
+    # parity with the oracle's chunked online LSE on a random 256-row sample
+    sample = torch.randperm(8192, generator=torch.Generator().manual_seed(4003))[:256].sort().values
+    ref_logp, ref_lse = oracle.linear_logp_chunked(
+        inputs.bits(c["h"][sample]), inputs.bits(c["w"]), c["t"][sample].numpy(), chunk_elems=256 * 2048
+    )[:2]
+    err = np.abs(logp.cpu().numpy()[sample.numpy()] - ref_logp).max()
+    err_lse = np.abs(lse.cpu().numpy()[sample.numpy()] - ref_lse).max()
+    assert err <= TOL_NATS and err_lse <= TOL_NATS, (err, err_lse)
+    assert err < 1e-4, err
+
+
+def test_config4_probabilities_of_all_columns_sum_to_one(logp_mod, config4):
+    # size-independent property: for one row, exp(logp) summed over every target id is 1
+    c = config4
+    v = c["w"].size(0)
+    ids = torch.arange(v, device=DEV)
+    row = c["h_d"][123:124].expand(4096, -1).contiguous()
+    total = 0.0
+    lse0 = None
+    for v0 in range(0, v, 4096):
+        chunk = ids[v0 : v0 + 4096]
+        lp, lse = logp_mod.deterministic_linear_logp(row[: chunk.numel()], c["w_d"], chunk)
+        total += float(lp.double().exp().sum())
+        lse0 = lse[0] if lse0 is None else lse0
+        assert bool((lse == lse0).all())  # the same row gives the same lse in every slot
+    assert abs(total - 1.0) < 1e-4
+
+
+# ---------------------------------------------------------------------------
+# GRPO epilogue and config 5
+# ---------------------------------------------------------------------------
+
+
+def test_grpo_golden_small_case(loss_mod):
+    d = np.load(GOLDEN / "small_grpo.npz")
+    out = loss_mod.grpo_ratio_kl_loss(
+        torch.from_numpy(d["logp"]).to(DEV),
+        torch.from_numpy(d["old"]).to(DEV),
+        torch.from_numpy(d["ref"]).to(DEV),
+        torch.from_numpy(d["adv"]).to(DEV),
+        torch.from_numpy(d["mask"]).to(DEV),
+        clip_eps=0.2,
+        beta=0.01,
+    )
+    got3 = torch.stack([out.loss, out.policy_loss, out.kl]).cpu().numpy()
+    assert np.allclose(got3, d["loss3"], rtol=2e-5, atol=1e-7)
+    assert np.allclose(out.ratio.cpu().numpy(), d["ratio"], rtol=2e-6, atol=0)
+    assert np.allclose(out.k3.cpu().numpy(), d["k3"], rtol=0, atol=3e-7)
+    again = loss_mod.grpo_ratio_kl_loss(
+        torch.from_numpy(d["logp"]).to(DEV),
+        torch.from_numpy(d["old"]).to(DEV),
+        torch.from_numpy(d["ref"]).to(DEV),
+        torch.from_numpy(d["adv"]).to(DEV),
+        torch.from_numpy(d["mask"]).to(DEV),
+        clip_eps=0.2,
+        beta=0.01,
+    )
+    assert _same_bits(again.loss.reshape(1), out.loss.reshape(1)) and _same_bits(again.ratio, out.ratio)
+
+
+def test_grpo_closed_forms(loss_mod):
+    g = torch.Generator().manual_seed(5200)
+    logp = (-torch.randn((7, 130), generator=g).abs()).to(DEV)
+    adv = torch.randn(7, generator=g).to(DEV)
+    same = loss_mod.grpo_ratio_kl_loss(logp, logp, logp, adv, beta=0.5)
+    assert bool((same.ratio == 1.0).all()) and bool((same.k3 == 0.0).all()) and float(same.kl) == 0.0
+    assert float(same.policy_loss) == pytest.approx(-float(adv.mean()), rel=1e-5)
+    hi = loss_mod.grpo_ratio_kl_loss(logp, logp - 1.0, logp, torch.full((7,), 2.0, device=DEV), clip_eps=0.2)
+    assert float(hi.policy_loss) == pytest.approx(-2.4, rel=1e-6)
+    lo = loss_mod.grpo_ratio_kl_loss(logp, logp - 1.0, logp, torch.full((7,), -2.0, device=DEV), clip_eps=0.2)
+    assert float(lo.policy_loss) == pytest.approx(2.0 * float(np.e), rel=1e-6)
+    mask = torch.zeros((7, 130), dtype=torch.bool, device=DEV)
+    none = loss_mod.grpo_ratio_kl_loss(logp, logp - 1.0, logp + 0.3, adv, mask, beta=0.1)
+    assert float(none.loss) == 0.0 and bool((none.ratio == 0).all()) and bool((none.k3 == 0).all())
+    quarter = loss_mod.compute_policy_ratio(logp, logp - 0.25)
+    assert torch.allclose(quarter, torch.full_like(quarter, float(np.exp(0.25))), rtol=1e-6)
+    assert bool((loss_mod.compute_reference_kl(logp, logp + 0.01) >= 0).all())
+
+
+def test_config5_rollout_scale(logp_mod, loss_mod, oracle, config4):
+    """64 rollouts x 1024 tokens through linear-LogP then the GRPO epilogue."""
+    rollouts, per = 64, 1024
+    tokens = rollouts * per
+    h = inputs.hidden_states(tokens, seed=5001, rms_norm=False)
+    gt = torch.Generator().manual_seed(5003)
+    target = torch.randint(0, inputs.QWEN3_VOCAB, (tokens,), generator=gt)
+    w, w_d = config4["w"], config4["w_d"]
+    h_d, t_d = h.to(DEV), target.to(DEV)
+    logp, lse = logp_mod.deterministic_linear_logp(h_d, w_d, t_d)
+    assert logp.shape == (tokens,) and bool(torch.isfinite(logp).all()) and bool((logp <= 0).all())
+    # per-rollout recomputation is bit-identical to the packed 65536-token call
+    for r in (0, 31, 63):
+        part, _ = logp_mod.deterministic_linear_logp(h_d[r * per : (r + 1) * per], w_d, t_d[r * per : (r + 1) * per])
+        assert _same_bits(part, logp[r * per : (r + 1) * per]), r
+    sample = torch.randperm(tokens, generator=torch.Generator().manual_seed(5004))[:128].sort().values
+    ref_logp = oracle.linear_logp_chunked(inputs.bits(h[sample]), inputs.bits(w), target[sample].numpy(), chunk_elems=128 * 2048)[0]
+    assert np.abs(logp.cpu().numpy()[sample.numpy()] - ref_logp).max() <= TOL_NATS
+
+    old, ref, adv = inputs.grpo_side_inputs(logp, rollouts)
+    lp2d = logp.view(rollouts, per)
+    for beta in (0.0, 0.01):
+        out = loss_mod.grpo_ratio_kl_loss(lp2d, old.view(rollouts, per).to(DEV), ref.view(rollouts, per).to(DEV), adv.to(DEV), clip_eps=0.2, beta=beta)
+        e_loss, e_policy, e_kl, e_ratio, e_k3 = oracle.grpo_ratio_kl_loss(
+            lp2d.cpu().numpy(), old.view(rollouts, per).numpy(), ref.view(rollouts, per).numpy(), adv.numpy(), clip_eps=0.2, beta=beta
+        )
+        assert np.allclose(out.ratio.cpu().numpy(), e_ratio, rtol=2e-6)
+        assert np.allclose(out.k3.cpu().numpy(), e_k3, atol=3e-7)
+        assert float(out.policy_loss) == pytest.approx(float(e_policy), rel=1e-4, abs=1e-6)
+        assert float(out.kl) == pytest.approx(float(e_kl), rel=1e-4)
+        assert float(out.loss) == pytest.approx(float(e_loss), rel=1e-4, abs=1e-6)
+        rerun = loss_mod.grpo_ratio_kl_loss(lp2d, old.view(rollouts, per).to(DEV), ref.view(rollouts, per).to(DEV), adv.to(DEV), clip_eps=0.2, beta=beta)
+        assert _same_bits(rerun.loss.reshape(1), out.loss.reshape(1))

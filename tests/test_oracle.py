@@ -1,0 +1,366 @@
+"""Pins the CPU oracle: every function is checked against something a plausible
+mistake (dropped term, wrong sign or index, transposed operand) would break --
+closed forms, brute force in fp64, and the known-answer values the reference's
+own tests hold for this path. Runs without a GPU."""
+
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import pytest
+
+
+def _bits(oracle, arr):
+    return oracle.f32_to_bf16(np.asarray(arr, dtype=np.float32))
+
+
+# ---------------------------------------------------------------------------
+# bf16 conversion
+# ---------------------------------------------------------------------------
+
+
+def test_bf16_known_bit_patterns(oracle):
+    cases = {
+        1.0: 0x3F80,
+        -1.0: 0xBF80,
+        0.0: 0x0000,
+        2.0: 0x4000,
+        0.5: 0x3F00,
+        float("inf"): 0x7F80,
+        float("-inf"): 0xFF80,
+        3.0: 0x4040,
+    }
+    for value, pattern in cases.items():
+        assert int(oracle.f32_to_bf16(np.float32(value)).reshape(-1)[0]) == pattern, value
+    assert int(_bits(oracle, [-0.0])[0]) == 0x8000
+
+
+def test_bf16_round_to_nearest_even_ties(oracle):
+    # 1 + 2^-8 lies exactly between 1.0 (even mantissa) and 1 + 2^-7: ties to even -> 1.0.
+    assert int(_bits(oracle, [1.0 + 2.0**-8])[0]) == 0x3F80
+    # 1 + 3*2^-8 lies between 1+2^-7 (odd) and 1+2^-6 (even): ties to even -> 1 + 2^-6.
+    assert int(_bits(oracle, [1.0 + 3 * 2.0**-8])[0]) == 0x3F82
+    # Just above the tie rounds up.
+    assert int(_bits(oracle, [np.float32(1.0 + 2.0**-8) + np.float32(2.0**-20)])[0]) == 0x3F81
+    # Largest finite fp32 rounds to +inf in bf16.
+    assert int(_bits(oracle, [np.finfo(np.float32).max])[0]) == 0x7F80
+    assert np.isnan(oracle.bf16_to_f32(_bits(oracle, [np.nan])))[0]
+
+
+def test_bf16_roundtrip_is_identity_on_bf16_values(oracle):
+    all_bits = np.arange(0, 1 << 16, dtype=np.uint32).astype(np.uint16)
+    f = oracle.bf16_to_f32(all_bits)
+    finite = np.isfinite(f)
+    assert np.array_equal(oracle.f32_to_bf16(f[finite]), all_bits[finite])
+
+
+def test_c_and_numpy_bf16_conversion_agree(oracle):
+    rng = np.random.default_rng(3)
+    x = np.concatenate(
+        [rng.standard_normal(4096).astype(np.float32) * 7, np.array([0.0, -0.0, 1e-40, 3e38, np.inf, -np.inf], np.float32)]
+    )
+    lib = oracle._c()
+    import ctypes
+
+    lib.oracle_f32_to_bf16.argtypes = [ctypes.c_float]
+    lib.oracle_f32_to_bf16.restype = ctypes.c_uint16
+    got = np.array([lib.oracle_f32_to_bf16(float(v)) for v in x], dtype=np.uint16)
+    assert np.array_equal(got, oracle.f32_to_bf16(x))
+
+
+# ---------------------------------------------------------------------------
+# det_gemm
+# ---------------------------------------------------------------------------
+
+GEMMS = ("det_gemm_ref", "det_gemm_seq")
+
+
+@pytest.mark.parametrize("fn", GEMMS)
+def test_gemm_k1_is_the_rounded_exact_product(oracle, fn):
+    rng = np.random.default_rng(1)
+    a = oracle.randn_bf16(rng, (5, 1))
+    bt = oracle.randn_bf16(rng, (7, 1))
+    expect = oracle.f32_to_bf16(oracle.bf16_to_f32(a) * oracle.bf16_to_f32(bt).T)
+    assert np.array_equal(getattr(oracle, fn)(a, bt), expect)
+
+
+@pytest.mark.parametrize("fn", GEMMS)
+def test_gemm_one_hot_rows_select_weight_columns(oracle, fn):
+    # A = one-hot rows -> C[i, :] is column k_i of B exactly; catches a transposed operand.
+    rng = np.random.default_rng(2)
+    k, n = 48, 9
+    bt = oracle.randn_bf16(rng, (n, k))
+    picks = [0, 5, 47, 17]
+    a = np.zeros((len(picks), k), dtype=np.float32)
+    for r, c in enumerate(picks):
+        a[r, c] = 1.0
+    got = getattr(oracle, fn)(oracle.f32_to_bf16(a), bt)
+    assert np.array_equal(got, bt[:, picks].T)
+
+
+@pytest.mark.parametrize("fn", GEMMS)
+def test_gemm_integer_sums_are_exact(oracle, fn):
+    # all-ones x powers of two: every partial sum is a small integer, exact in fp32 and bf16.
+    k = 96
+    a = oracle.f32_to_bf16(np.ones((3, k), np.float32))
+    b = np.zeros((4, k), np.float32)
+    b[0, :] = 1.0  # sum = 96
+    b[1, :64] = 2.0  # sum = 128
+    b[2, ::2] = -0.5  # sum = -24
+    b[3, :3] = [4.0, -4.0, 0.25]  # sum = 0.25
+    got = oracle.bf16_to_f32(getattr(oracle, fn)(a, oracle.f32_to_bf16(b)))
+    assert np.array_equal(got, np.tile(np.array([96.0, 128.0, -24.0, 0.25], np.float32), (3, 1)))
+
+
+@pytest.mark.parametrize("fn", GEMMS)
+def test_gemm_matches_fp64_brute_force_within_accumulation_bound(oracle, fn):
+    rng = np.random.default_rng(4)
+    m, n, k = 33, 29, 1000
+    a = oracle.randn_bf16(rng, (m, k))
+    bt = oracle.randn_bf16(rng, (n, k), 0.02)
+    exact = oracle.det_gemm_f64(a, bt)
+    # independent check of the C fp64 loop against numpy
+    assert np.allclose(exact, oracle.bf16_to_f32(a).astype(np.float64) @ oracle.bf16_to_f32(bt).astype(np.float64).T, rtol=1e-12, atol=1e-12)
+    got = oracle.bf16_to_f32(getattr(oracle, fn)(a, bt)).astype(np.float64)
+    abs_sum = np.abs(oracle.bf16_to_f32(a)).astype(np.float64) @ np.abs(oracle.bf16_to_f32(bt)).astype(np.float64).T
+    bound = 2.0**-8 * np.abs(got) + k * 2.0**-24 * abs_sum  # half a bf16 ulp (<= 2^-8 |x|) + fp32 summation bound
+    assert np.all(np.abs(got - exact) <= bound + 1e-30)
+
+
+def test_gemm_reference_equality_demand_at_4x16_by_9x16(oracle):
+    # The reference requires its sequential kernel to equal (a.float() @ w.float().t()).to(bf16)
+    # bit for bit at this shape (tests/test_musa_det_gemm.py:133-140).
+    rng = np.random.default_rng(5)
+    a = oracle.randn_bf16(rng, (4, 16))
+    w = oracle.randn_bf16(rng, (9, 16))
+    assert np.array_equal(oracle.det_gemm_seq(a, w), oracle.det_gemm_ref(a, w))
+
+
+def test_gemm_ref_and_seq_agree_to_one_ulp_on_config1_shape(oracle):
+    rng = np.random.default_rng(6)
+    a = oracle.randn_bf16(rng, (16, 1024))
+    bt = oracle.randn_bf16(rng, (64, 1024), 0.02)
+    ref, seq = oracle.det_gemm_ref(a, bt), oracle.det_gemm_seq(a, bt)
+    big = np.abs(oracle.bf16_to_f32(ref)) > 0.05  # away from cancellation
+    assert oracle.bf16_ulp_distance(ref, seq)[big].max() <= 1
+
+
+# ---------------------------------------------------------------------------
+# k-tree contract
+# ---------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("leaf_space", (False, True))
+def test_k_tree_with_one_leaf_is_the_sequential_gemm(oracle, leaf_space):
+    rng = np.random.default_rng(7)
+    for k in (1, 8, 31, 32):
+        a = oracle.randn_bf16(rng, (5, k))
+        bt = oracle.randn_bf16(rng, (6, k))
+        assert np.array_equal(oracle.k_tree_gemm(a, bt, leaf_space=leaf_space), oracle.det_gemm_seq(a, bt))
+
+
+def test_k_tree_two_leaves_is_bf16_add_of_leaf_sums(oracle):
+    rng = np.random.default_rng(8)
+    a = oracle.randn_bf16(rng, (4, 64))
+    bt = oracle.randn_bf16(rng, (5, 64))
+    left = oracle.bf16_to_f32(oracle.det_gemm_seq(a[:, :32], bt[:, :32]))
+    right = oracle.bf16_to_f32(oracle.det_gemm_seq(a[:, 32:], bt[:, 32:]))
+    assert np.array_equal(oracle.k_tree_gemm(a, bt), oracle.f32_to_bf16(left + right))
+
+
+def test_k_tree_element_and_leaf_space_agree_iff_leaf_count_is_power_of_two(oracle):
+    rng = np.random.default_rng(9)
+    for k in (1024, 4096):
+        a = oracle.randn_bf16(rng, (2, k))
+        bt = oracle.randn_bf16(rng, (8, k))
+        assert np.array_equal(oracle.k_tree_gemm(a, bt), oracle.k_tree_gemm(a, bt, leaf_space=True))
+    # K=12288: element space halves down to 24-wide leaves (512 of them,
+    # tests/ops/gemm/test_det_gemm.py:282-283), leaf space keeps 384 leaves of 32.
+    a = oracle.randn_bf16(rng, (4, 12288))
+    bt = oracle.randn_bf16(rng, (32, 12288))
+    assert not np.array_equal(oracle.k_tree_gemm(a, bt), oracle.k_tree_gemm(a, bt, leaf_space=True))
+
+
+def test_k_tree_balanced_k_shards_reproduce_the_full_tree(oracle):
+    # The property the contract exists for (tests/ops/gemm/test_det_gemm.py:276-300):
+    # a contiguous half-K GEMM is exactly one child of the root.
+    rng = np.random.default_rng(10)
+    k = 2048
+    a = oracle.randn_bf16(rng, (3, k))
+    bt = oracle.randn_bf16(rng, (7, k))
+    full = oracle.k_tree_gemm(a, bt)
+    lo = oracle.bf16_to_f32(oracle.k_tree_gemm(a[:, : k // 2], bt[:, : k // 2]))
+    hi = oracle.bf16_to_f32(oracle.k_tree_gemm(a[:, k // 2 :], bt[:, k // 2 :]))
+    assert np.array_equal(full, oracle.f32_to_bf16(lo + hi))
+
+
+# ---------------------------------------------------------------------------
+# linear-LogP
+# ---------------------------------------------------------------------------
+
+
+def test_logp_uniform_logits_give_minus_log_v(oracle):
+    # Zero hidden states -> all logits 0 -> logp = -log V, lse = log V.
+    n, d, v = 6, 32, 1000
+    h = np.zeros((n, d), np.uint16)
+    w = oracle.randn_bf16(np.random.default_rng(11), (v, d))
+    target = np.arange(n) * 7
+    for logp, lse in (oracle.linear_logp_chunked(h, w, target)[:2], oracle.linear_logp_dense(h, w, target)):
+        assert np.allclose(lse, math.log(v), atol=1e-6)
+        assert np.allclose(logp, -math.log(v), atol=1e-6)
+
+
+def test_logp_bias_only_closed_form(oracle):
+    # h = 0, bias = log of a known distribution -> logp of token t is log p_t exactly.
+    n, d, v = 4, 16, 50
+    rng = np.random.default_rng(12)
+    p = rng.random(v) + 0.1
+    p = p / p.sum()
+    bias = np.log(p).astype(np.float32)
+    h = np.zeros((n, d), np.uint16)
+    w = oracle.randn_bf16(rng, (v, d))
+    target = np.array([0, 13, 49, 7])
+    logp, lse = oracle.linear_logp_dense(h, w, target, bias)
+    assert np.allclose(logp, np.log(p[target]), atol=2e-6)
+    assert np.allclose(lse, 0.0, atol=2e-6)
+    logp_c = oracle.linear_logp_chunked(h, w, target, bias, chunk_elems=4 * 16)[0]
+    assert np.allclose(logp_c, np.log(p[target]), atol=2e-6)
+
+
+def test_logp_chunked_dense_and_fp64_agree_and_chunking_is_immaterial(oracle):
+    rng = np.random.default_rng(13)
+    n, d, v = 37, 96, 3001
+    h = oracle.randn_bf16(rng, (n, d))
+    w = oracle.randn_bf16(rng, (v, d), 0.1)
+    bias = (rng.standard_normal(v) * 0.3).astype(np.float32)
+    target = rng.integers(0, v, n)
+    exact, exact_lse = oracle.linear_logp_f64(h, w, target, bias)
+    dense, dense_lse = oracle.linear_logp_dense(h, w, target, bias)
+    assert np.abs(dense - exact).max() < 2e-5 and np.abs(dense_lse - exact_lse).max() < 2e-5
+    for chunk_elems in (1 << 24, n * 512, n * 100, n):  # one chunk ... one vocabulary row per chunk
+        logp, lse, m, s, zt = oracle.linear_logp_chunked(h, w, target, bias, chunk_elems=chunk_elems)
+        assert np.abs(logp - exact).max() < 2e-5, chunk_elems
+        assert np.abs(lse - exact_lse).max() < 2e-5
+    # the reference's chunk rule at config 4: 2^24 // 8192 = 2048 rows -> 75 chunks, last 384
+    chunk = max(1, min(151936, oracle.BWD_CHUNK_ELEMS // 8192))
+    assert chunk == 2048 and math.ceil(151936 / chunk) == 75 and 151936 - 74 * chunk == 384
+
+
+def test_logp_probabilities_sum_to_one_and_target_picks_the_right_column(oracle):
+    rng = np.random.default_rng(14)
+    n, d, v = 3, 64, 257
+    h = oracle.randn_bf16(rng, (n, d))
+    w = oracle.randn_bf16(rng, (v, d), 0.2)
+    # logp of every column, one call per column id; exp must sum to 1 per row.
+    total = np.zeros(n)
+    for t in range(v):
+        total += np.exp(oracle.linear_logp_chunked(h, w, np.full(n, t), chunk_elems=n * 64)[0].astype(np.float64))
+    assert np.allclose(total, 1.0, atol=1e-4)
+
+
+def test_logp_vocab_start_index_shifts_target_ownership(oracle):
+    rng = np.random.default_rng(15)
+    n, d, v = 5, 32, 300
+    h = oracle.randn_bf16(rng, (n, d))
+    w = oracle.randn_bf16(rng, (v, d), 0.2)
+    target = rng.integers(0, v, n)
+    base = oracle.linear_logp_chunked(h, w, target, chunk_elems=n * 64)[0]
+    shifted = oracle.linear_logp_chunked(h, w, target + 1000, vocab_start_index=1000, chunk_elems=n * 64)[0]
+    assert np.array_equal(base, shifted)
+
+
+def test_logp_temperature_and_padding_follow_the_strict_contract(oracle):
+    rng = np.random.default_rng(16)
+    n, d, v, real = 4, 32, 128, 100
+    h = oracle.randn_bf16(rng, (n, d))
+    w = oracle.randn_bf16(rng, (v, d), 0.3)
+    target = rng.integers(0, real, n)
+    temp = np.array([0.5, 1.0, 2.0, 0.7], np.float32)
+    logp, lse = oracle.linear_logp_dense(h, w, target, temperature=temp, real_vocab_size=real)
+    # padded lanes contribute nothing: same as dropping the rows of W
+    logp2, lse2 = oracle.linear_logp_dense(h, w[:real], target, temperature=temp)
+    # (to fp32 rounding: the BLAS may order the dot products differently for another N)
+    assert np.allclose(logp, logp2, atol=2e-6, rtol=0) and np.allclose(lse, lse2, atol=2e-6, rtol=0)
+    # temperature 1 row equals the untempered value
+    plain = oracle.linear_logp_dense(h, w[:real], target)[0]
+    assert abs(plain[1] - logp[1]) < 2e-6
+    exact = oracle.linear_logp_f64(h, w, target, temperature=temp, real_vocab_size=real)[0]
+    assert np.abs(logp - exact).max() < 2e-5
+
+
+# ---------------------------------------------------------------------------
+# GRPO
+# ---------------------------------------------------------------------------
+
+
+def test_masked_reductions_reference_known_answers(oracle):
+    # tests/reference/test_reference_ops.py:77-84
+    values = np.array([[1.0, 100.0], [3.0, 4.0]], np.float32)
+    mask = np.array([[True, False], [True, True]])
+    assert oracle.masked_mean(values, mask) == pytest.approx(8.0 / 3.0, rel=1e-6)
+    assert oracle.masked_mean(values) == pytest.approx(27.0, rel=1e-6)
+    assert oracle.masked_mean(values, np.zeros((2, 2), bool)) == 0.0
+
+
+def test_ratio_and_kl_reference_example(oracle):
+    # tests/reference/test_reference_ops.py:88-98: current - old = 0.5 and ref - current = -0.25 everywhere.
+    current = np.array([[0.0, -1.0], [-2.0, -3.0]], np.float32)
+    old = np.array([[-0.5, -1.5], [-2.5, -3.5]], np.float32)
+    ref = np.array([[-0.25, -1.25], [-2.25, -3.25]], np.float32)
+    mask = np.array([[True, False], [True, True]])
+    ratio = oracle.compute_policy_ratio(current, old, mask)
+    kl = oracle.compute_reference_kl(current, ref, mask)
+    assert ratio[0, 1] == 0.0 and kl[0, 1] == 0.0
+    assert np.allclose(ratio[mask], math.exp(0.5), rtol=1e-6)
+    assert np.allclose(kl[mask], math.exp(-0.25) + 0.25 - 1.0, rtol=1e-5)
+
+
+def test_group_advantages_reference_known_answer(oracle):
+    # tests/ops/loss/test_grpo_loss.py:112-119
+    got = oracle.group_advantages([1.0, 3.0, 10.0, 20.0, 30.0], group_boundaries=[0, 2, 5])
+    g1 = (np.array([10.0, 20.0, 30.0]) - 20.0) / math.sqrt(200.0 / 3.0)
+    assert np.allclose(got, np.concatenate([[-1.0, 1.0], g1]), atol=1e-5)
+    uniform = oracle.group_advantages([1.0, 3.0, 10.0, 30.0], samples_per_prompt=2)
+    assert np.allclose(uniform, [-1, 1, -1, 1], atol=1e-5)
+    with pytest.raises(ValueError):
+        oracle.group_advantages([1.0, 2.0])
+
+
+def test_grpo_closed_forms(oracle):
+    rng = np.random.default_rng(17)
+    logp = -np.abs(rng.standard_normal((3, 8))).astype(np.float32)
+    adv = np.array([1.0, -2.0, 0.5], np.float32)
+    # old == logp -> ratio exactly 1 -> term = -A; ref == logp -> k3 exactly 0.
+    loss, policy, kl, ratio, k3 = oracle.grpo_ratio_kl_loss(logp, logp, logp, adv, beta=0.3)
+    assert np.all(ratio == 1.0) and np.all(k3 == 0.0) and kl == 0.0
+    assert policy == pytest.approx(-adv.mean(), rel=1e-6) and loss == policy
+    # ratio far above 1+eps with A>0 saturates at -(1+eps)A; with A<0 the unclipped branch wins.
+    old = logp - 1.0
+    _, policy, _, ratio, _ = oracle.grpo_ratio_kl_loss(logp, old, logp, np.array([2.0, 2.0, 2.0], np.float32), clip_eps=0.2)
+    assert policy == pytest.approx(-1.2 * 2.0, rel=1e-6)
+    _, policy, _, _, _ = oracle.grpo_ratio_kl_loss(logp, old, logp, np.array([-2.0, -2.0, -2.0], np.float32), clip_eps=0.2)
+    assert policy == pytest.approx(math.e * 2.0, rel=1e-6)
+    # k3 is non-negative and ~ d^2/2 for small d
+    _, _, _, _, k3 = oracle.grpo_ratio_kl_loss(logp, logp, logp + np.float32(0.01), adv)
+    assert np.all(k3 >= 0) and np.allclose(k3, 0.5e-4, rtol=0.05)
+
+
+def test_grpo_hand_computed_2x2(oracle):
+    logp = np.array([[-1.0, -2.0], [-0.5, -3.0]], np.float32)
+    old = np.array([[-1.1, -1.7], [-0.5, -3.3]], np.float32)
+    ref = np.array([[-0.9, -2.0], [-0.7, -2.5]], np.float32)
+    adv = np.array([1.5, -0.5], np.float32)
+    mask = np.array([[1, 1], [0, 1]], bool)
+    loss, policy, kl, ratio, k3 = oracle.grpo_ratio_kl_loss(logp, old, ref, adv, mask, clip_eps=0.2, beta=0.01)
+    r = [math.exp(0.1), math.exp(-0.3), 0.0, math.exp(0.3)]
+    terms = [
+        -min(r[0] * 1.5, min(max(r[0], 0.8), 1.2) * 1.5),
+        -min(r[1] * 1.5, min(max(r[1], 0.8), 1.2) * 1.5),
+        -min(r[3] * -0.5, min(max(r[3], 0.8), 1.2) * -0.5),
+    ]
+    ks = [math.exp(0.1) - 0.1 - 1, 0.0, math.exp(0.5) - 0.5 - 1]
+    assert policy == pytest.approx(sum(terms) / 3, rel=1e-5)
+    assert kl == pytest.approx(sum(ks) / 3, rel=1e-4)
+    assert loss == pytest.approx(sum(terms) / 3 + 0.01 * sum(ks) / 3, rel=1e-5)
+    assert ratio[1, 0] == 0.0 and k3[1, 0] == 0.0
