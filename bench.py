@@ -1,0 +1,298 @@
+#!/usr/bin/env python3
+"""Headline benchmark: deterministic bf16 GEMM at Qwen3-8B FFN shapes on one MI355X.
+
+One "step" is one pass of the FFN hot path over one synthetic batch of T=4096
+tokens: the gate_up GEMM X[4096,4096] x W[24576,4096]^T followed by the down GEMM
+H[4096,12288] x W[4096,12288]^T, inputs resident in HBM. The JSON line also carries
+
+* ``roofline``     - the dominant kernel (the 256x256-tile MFMA kernel on gate_up)
+                     against the MI355X dense bf16 MFMA peak, timed with HIP events
+                     on the launch stream;
+* ``cpu_baseline`` - the CPU oracle (``oracle/reference_math.det_gemm_ref``) timed on
+                     this box's host cores on the same step;
+* ``shapes``       - every token count of the configuration (T = 1, 16, 256, 4096)
+                     with its own MFMA or HBM fraction;
+* ``linear_logp``  - the fused linear-LogP at T=8192, V=151936, D=4096 in tokens/s.
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-logp]
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for _p in (ROOT, ROOT / "rl-kernel_amd", ROOT / "tests"):
+    if str(_p) not in sys.path:
+        sys.path.insert(0, str(_p))
+
+# MI355X published peaks used for every fraction below.
+PEAK_BF16_TFLOPS = 2500.0  # dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0  # HBM3E
+
+HIDDEN, INTER, VOCAB = 4096, 12288, 151936
+
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs of this script (profiles/det_gemm_gate_up_T4096_pmc.md), scaled
+# by the same counters read on a plain device copy of known size. None = not measured.
+MEASURED_TRAFFIC_BYTES = {"det_gemm_gate_up_T4096": None}
+
+
+def _parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-logp", action="store_true", help="skip the linear-LogP leg")
+    ap.add_argument("--no-shapes", action="store_true", help="skip the per-T table")
+    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|logp|copy")
+    return ap.parse_args()
+
+
+def _time_calls(fn, iters: int, warmup: int) -> float:
+    """Average milliseconds per call, HIP events on the current (launch) stream."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def _gemm_bytes(m, n, k):
+    return 2.0 * (m * k + n * k + m * n)
+
+
+def main() -> int:
+    args = _parse()
+    if args.gpus != 1:
+        print(
+            f"bench.py: --gpus {args.gpus} is not supported: this build runs on exactly one GPU "
+            "(no collectives, no sharding); run with --gpus 1.",
+            file=sys.stderr,
+        )
+        return 2
+
+    import torch
+
+    from rl_engine import _lib
+    from rl_engine.backends.rocm.gemm import det_gemm as gemm
+    from rl_engine.ops.logprob import deterministic_linear_logp
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    _lib.load()  # fails loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(2000)
+
+    def randn(rows, cols, scale=1.0):
+        out = torch.empty((rows, cols), dtype=torch.bfloat16, device=dev)
+        step = 8192
+        for r0 in range(0, rows, step):
+            r1 = min(r0 + step, rows)
+            out[r0:r1] = (torch.randn((r1 - r0, cols), generator=gen, device=dev, dtype=torch.float32) * scale).to(torch.bfloat16)
+        return out
+
+    T = 4096
+    x = randn(T, HIDDEN)
+    h = randn(T, INTER)
+    w_gu = randn(2 * INTER, HIDDEN, 0.02)
+    w_d = randn(HIDDEN, INTER, 0.02)
+    out_gu = torch.empty((T, 2 * INTER), dtype=torch.bfloat16, device=dev)
+    out_d = torch.empty((T, HIDDEN), dtype=torch.bfloat16, device=dev)
+
+    def gate_up():
+        gemm.mfma_gemm(x, w_gu.t(), out=out_gu)
+
+    def down():
+        gemm.mfma_gemm(h, w_d.t(), out=out_d)
+
+    def step():
+        gate_up()
+        down()
+
+    if args.only == "copy":
+        # Calibration leg for the FETCH_SIZE / WRITE_SIZE counters: one plain device
+        # copy kernel of known size (1 GiB read + 1 GiB written per launch).
+        src = torch.empty((1 << 29,), dtype=torch.bfloat16, device=dev)
+        dst = torch.empty_like(src)
+        src.fill_(1.0)
+        for _ in range(3):
+            torch.add(src, 0.0, out=dst)
+        torch.cuda.synchronize()
+        print(json.dumps({"leg": "copy", "bytes_read": src.numel() * 2, "bytes_written": dst.numel() * 2, "launches": 3}))
+        return 0
+    if args.only in ("gate_up", "down"):
+        fn = gate_up if args.only == "gate_up" else down
+        ms = _time_calls(fn, args.steps, args.warmup)
+        print(json.dumps({"leg": args.only, "ms": ms, "launches": args.steps + args.warmup}))
+        return 0
+
+    flops_gu = 2.0 * T * (2 * INTER) * HIDDEN
+    flops_d = 2.0 * T * HIDDEN * INTER
+
+    # ---- timed region: exactly `steps` steps, synchronised on both sides
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    tflops = (flops_gu + flops_d) / wall_ms * 1e-9
+
+    # ---- dominant kernel, HIP events over the same launches
+    ms_gu = _time_calls(gate_up, args.steps, 2)
+    ms_d = _time_calls(down, args.steps, 2)
+    achieved = flops_gu / ms_gu * 1e-9
+    roofline = {
+        "kernel": "det_gemm_kernel<256x256 tile, 8 waves> on gate_up [4096x4096]x[24576x4096]^T",
+        "bound": "mfma",
+        "achieved": round(achieved, 1),
+        "peak": PEAK_BF16_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+        "ms_per_launch": round(ms_gu, 4),
+        "flops_per_launch": flops_gu,
+        "traffic": MEASURED_TRAFFIC_BYTES["det_gemm_gate_up_T4096"],
+    }
+
+    result = {
+        "metric": "bf16 det-GEMM TFLOP/s at Qwen3-8B FFN shapes (gate_up + down, T=4096)",
+        "value": round(tflops, 1),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "Qwen3-8B FFN det GEMMs: gate_up X[4096,4096]xW[24576,4096]^T then down H[4096,12288]xW[4096,12288]^T, "
+            "bf16 in, fp32 MFMA accumulate in fixed K order, bf16 out, T=4096",
+            "contract": gemm.det_gemm_backend_id(),
+        },
+        "frac_of_mfma_peak": round(tflops / PEAK_BF16_TFLOPS, 4),
+        "kernels": {
+            "gate_up_ms": round(ms_gu, 4),
+            "gate_up_tflops": round(flops_gu / ms_gu * 1e-9, 1),
+            "down_ms": round(ms_d, 4),
+            "down_tflops": round(flops_d / ms_d * 1e-9, 1),
+        },
+        "roofline": roofline,
+    }
+
+    # ---- every token count of the configuration
+    if not args.no_shapes:
+        shapes = []
+        for t in (1, 16, 256, 1024, 4096):
+            for name, act, w, n, k, out in (("gate_up", x, w_gu, 2 * INTER, HIDDEN, out_gu), ("down", h, w_d, HIDDEN, INTER, out_d)):
+                a_t, o_t = act[:t], out[:t]
+                ms = _time_calls(lambda: gemm.mfma_gemm(a_t, w.t(), out=o_t), 30 if t <= 256 else 10, 3)
+                fl = 2.0 * t * n * k
+                by = _gemm_bytes(t, n, k)
+                tf, gb = fl / ms * 1e-9, by / ms * 1e-6
+                hbm_bound = (fl / by) < (PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBPS * 1e9))
+                shapes.append(
+                    {
+                        "op": name,
+                        "T": t,
+                        "ms": round(ms, 4),
+                        "tflops": round(tf, 1),
+                        "gbps": round(gb, 1),
+                        "bound": "hbm" if hbm_bound else "mfma",
+                        "frac": round(gb / PEAK_HBM_GBPS if hbm_bound else tf / PEAK_BF16_TFLOPS, 4),
+                    }
+                )
+        result["shapes"] = shapes
+
+    # ---- fused linear-LogP at T=8192, V=151936
+    if not args.no_logp:
+        tl = 8192
+        hid = randn(tl, HIDDEN)
+        hid = (hid.float() * torch.rsqrt(hid.float().pow(2).mean(-1, keepdim=True) + 1e-6)).to(torch.bfloat16)
+        w_lm = randn(VOCAB, HIDDEN, 0.02)
+        tgt = torch.randint(0, VOCAB, (tl,), generator=gen, device=dev)
+        ms_lp = _time_calls(lambda: deterministic_linear_logp(hid, w_lm, tgt), 5, 2)
+        fl_lp = 2.0 * tl * VOCAB * HIDDEN
+        result["linear_logp"] = {
+            "workload": "hidden[8192,4096] x lm_head[151936,4096]^T -> online LSE -> target gather, fp32 logp",
+            "tokens_per_s": round(tl / ms_lp * 1e3, 1),
+            "ms": round(ms_lp, 3),
+            "tflops": round(fl_lp / ms_lp * 1e-9, 1),
+            "frac_of_mfma_peak": round(fl_lp / ms_lp * 1e-9 / PEAK_BF16_TFLOPS, 4),
+            "min_hbm_bytes": 2.0 * (VOCAB * HIDDEN + tl * HIDDEN) + 8.0 * tl,
+        }
+
+    # ---- CPU baseline: the oracle on the same step, on this box's host cores
+    if not args.no_cpu:
+        import numpy as np
+
+        import inputs
+        from oracle import reference_math as oracle
+
+        try:
+            from threadpoolctl import threadpool_info
+
+            blas_threads = max([p.get("num_threads", 1) for p in threadpool_info() if p.get("user_api") == "blas"] or [1])
+        except Exception:
+            blas_threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        xb, hb = inputs.bits(x), inputs.bits(h)
+        wgb, wdb = inputs.bits(w_gu), inputs.bits(w_d)
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            oracle.det_gemm_ref(xb, wgb)
+            oracle.det_gemm_ref(hb, wdb)
+            times.append(time.perf_counter() - t0)
+            if sum(times) > 30:
+                break
+        cpu_s = float(np.median(times))
+        result["cpu_baseline"] = {
+            "value": round((flops_gu + flops_d) / cpu_s * 1e-12, 4),
+            "unit": "TFLOP/s",
+            "cores": int(blas_threads),
+            "kind": "port",
+            "sample": f"the full step (gate_up + down at T=4096, {(flops_gu + flops_d) / 1e9:.0f} GFLOP), "
+            f"median of {len(times)} runs of oracle.det_gemm_ref (fp32 upcast, numpy sgemm, one bf16 rounding), {cpu_s:.2f} s each",
+        }
+        if not args.no_logp:
+            ts = 256
+            hb2, wb2 = inputs.bits(hid[:ts]), inputs.bits(w_lm)
+            t0 = time.perf_counter()
+            oracle.linear_logp_chunked(hb2, wb2, tgt[:ts].cpu().numpy(), chunk_elems=ts * 2048)
+            cpu_lp = time.perf_counter() - t0
+            result["linear_logp"]["cpu_baseline"] = {
+                "value": round(ts / cpu_lp, 1),
+                "unit": "tokens/s",
+                "cores": int(blas_threads),
+                "kind": "port",
+                "sample": f"first {ts} of the 8192 tokens, oracle.linear_logp_chunked (2048-row vocabulary chunks), {cpu_lp:.2f} s",
+            }
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

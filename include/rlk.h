@@ -44,7 +44,11 @@ typedef enum rlk_gemm_config {
   RLK_GEMM_CFG_64x64 = 5,
   RLK_GEMM_CFG_64x16 = 6,
   RLK_GEMM_CFG_16x16 = 7,
-  RLK_GEMM_CFG_COUNT = 8
+  RLK_GEMM_CFG_COUNT = 8,
+  /* OR-ed into a configuration: use the register-staged main loop even where the
+   * direct-to-LDS ping-pong loop applies. Bit-neutral; exists so tests can
+   * compare the two loops. */
+  RLK_GEMM_CFG_FORCE_STAGED = 0x100
 } rlk_gemm_config;
 
 /* Arithmetic contract identifier (provenance string).
@@ -89,7 +93,10 @@ typedef enum rlk_logp_config {
   RLK_LOGP_CFG_128 = 2,
   RLK_LOGP_CFG_64 = 3,
   RLK_LOGP_CFG_16 = 4,
-  RLK_LOGP_CFG_COUNT = 5
+  RLK_LOGP_CFG_COUNT = 5,
+  /* OR-ed into a configuration: register-staged main loop instead of the
+   * direct-to-LDS ping-pong loop (bit-neutral; for tests). */
+  RLK_LOGP_CFG_FORCE_STAGED = 0x100
 } rlk_logp_config;
 
 /* Reduction contract identifier of the fused linear-LogP.

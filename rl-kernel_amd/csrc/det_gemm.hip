@@ -9,7 +9,12 @@
 
 namespace rlk {
 
-template <class S, bool VEC, bool OUT_F32>
+// LOOP selects the main loop: kLoopGeneric (any strides, element loads),
+// kLoopStaged (16-byte loads through registers) or kLoopPingPong (direct-to-LDS
+// loads, two wave groups half an iteration apart). All three run the same MFMA chain.
+enum : int { kLoopGeneric = 0, kLoopStaged = 1, kLoopPingPong = 2 };
+
+template <class S, int LOOP, bool OUT_F32>
 __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatView X, void* __restrict__ C,
                                                                 int64_t ldc, int M, int N, int K,
                                                                 int tiles_m, int tiles_n, int group_m) {
@@ -30,7 +35,11 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
   const int m0 = tile_m * S::BM;
 
   f32x4_t acc[S::TN][S::TM];
-  tile_mainloop<S, VEC>(W, X, n0, m0, K, lds, acc);
+  if constexpr (LOOP == kLoopPingPong) {
+    tile_mainloop_pingpong<S>(W, X, n0, m0, K, lds, acc);
+  } else {
+    tile_mainloop_staged<S, LOOP == kLoopStaged>(W, X, n0, m0, K, lds, acc);
+  }
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -92,10 +101,10 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
 // Host side
 // ---------------------------------------------------------------------------
 
-template <class S, bool VEC, bool OUT_F32>
+template <class S, int LOOP, bool OUT_F32>
 static hipError_t launch_tile(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
                               hipStream_t stream) {
-  auto kernel = det_gemm_kernel<S, VEC, OUT_F32>;
+  auto kernel = det_gemm_kernel<S, LOOP, OUT_F32>;
   static bool configured[kMaxDevices] = {};
   int dev = 0;
   hipError_t err = hipGetDevice(&dev);
@@ -116,21 +125,27 @@ static hipError_t launch_tile(const MatView& W, const MatView& X, void* C, int64
 
 template <class S>
 static hipError_t launch_shape(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
-                               bool vec, bool out_f32, hipStream_t stream) {
-  if (vec) {
-    return out_f32 ? launch_tile<S, true, true>(W, X, C, ldc, M, N, K, stream)
-                   : launch_tile<S, true, false>(W, X, C, ldc, M, N, K, stream);
+                               bool vec, bool allow_pingpong, bool out_f32, hipStream_t stream) {
+  if constexpr (pingpong_supported<S>()) {
+    if (vec && allow_pingpong && K % kTileK == 0) {
+      return out_f32 ? launch_tile<S, kLoopPingPong, true>(W, X, C, ldc, M, N, K, stream)
+                     : launch_tile<S, kLoopPingPong, false>(W, X, C, ldc, M, N, K, stream);
+    }
   }
-  return out_f32 ? launch_tile<S, false, true>(W, X, C, ldc, M, N, K, stream)
-                 : launch_tile<S, false, false>(W, X, C, ldc, M, N, K, stream);
+  if (vec) {
+    return out_f32 ? launch_tile<S, kLoopStaged, true>(W, X, C, ldc, M, N, K, stream)
+                   : launch_tile<S, kLoopStaged, false>(W, X, C, ldc, M, N, K, stream);
+  }
+  return out_f32 ? launch_tile<S, kLoopGeneric, true>(W, X, C, ldc, M, N, K, stream)
+                 : launch_tile<S, kLoopGeneric, false>(W, X, C, ldc, M, N, K, stream);
 }
 
 // Tile shapes. Which one runs is a pure performance choice (see det_gemm_tile.h).
-using Shape256x256 = TileShape<256, 256, 2, 4>;
+using Shape256x256 = TileShape<256, 256, 4, 2>;
 using Shape256x128 = TileShape<256, 128, 4, 2>;
-using Shape128x128 = TileShape<128, 128, 2, 2>;
-using Shape128x64 = TileShape<128, 64, 4, 1>;
-using Shape64x64 = TileShape<64, 64, 2, 2>;
+using Shape128x128 = TileShape<128, 128, 4, 2>;
+using Shape128x64 = TileShape<128, 64, 4, 2>;
+using Shape64x64 = TileShape<64, 64, 4, 2>;
 using Shape64x16 = TileShape<64, 16, 4, 1>;
 using Shape16x16 = TileShape<16, 16, 1, 1>;
 
@@ -147,26 +162,57 @@ int pick_det_gemm_config(int M, int N, int K) {
   (void)K;
   constexpr int kCus = 256;
   if (M <= 16) return N >= 64 * kCus ? RLK_GEMM_CFG_64x16 : RLK_GEMM_CFG_16x16;
-  if (tile_count(M, N, 256, 256) >= 2 * kCus) return RLK_GEMM_CFG_256x256;
-  if (M >= 128 && tile_count(M, N, 128, 256) >= kCus) return RLK_GEMM_CFG_256x128;
-  if (M >= 128 && tile_count(M, N, 128, 128) >= kCus) return RLK_GEMM_CFG_128x128;
-  if (M > 64 && tile_count(M, N, 64, 128) >= kCus / 2) return RLK_GEMM_CFG_128x64;
-  return RLK_GEMM_CFG_64x64;
+  // Estimated time = (rounds of 256 workgroups) x (tile area / measured relative
+  // throughput of the shape when the chip is full). Larger tiles win ties.
+  struct Candidate {
+    int config, bn, bm;
+    double quality;
+  };
+  static const Candidate kCandidates[] = {
+      {RLK_GEMM_CFG_256x256, 256, 256, 1.00}, {RLK_GEMM_CFG_256x128, 256, 128, 0.95},
+      {RLK_GEMM_CFG_128x128, 128, 128, 0.90}, {RLK_GEMM_CFG_128x64, 128, 64, 0.70},
+      {RLK_GEMM_CFG_64x64, 64, 64, 0.55},
+  };
+  int best = RLK_GEMM_CFG_64x64;
+  double best_time = 1e300;
+  for (const Candidate& c : kCandidates) {
+    const int64_t tiles = tile_count(M, N, c.bm, c.bn);
+    const double rounds = (double)((tiles + kCus - 1) / kCus);
+    const double t = rounds * (double)(c.bn * c.bm) / c.quality;
+    if (t < best_time * 0.999) {
+      best_time = t;
+      best = c.config;
+    }
+  }
+  return best;
 }
 
 hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
                            bool out_f32, int config, hipStream_t stream) {
   const bool vec = view_is_vectorizable(W) && view_is_vectorizable(X) && (K % kChunkElems) == 0;
+  const bool allow_pingpong = (config & RLK_GEMM_CFG_FORCE_STAGED) == 0;
+  config &= ~RLK_GEMM_CFG_FORCE_STAGED;
   if (config == RLK_GEMM_CFG_AUTO) config = pick_det_gemm_config(M, N, K);
+  // The element-wise loader of the generic path keeps eight values per chunk in
+  // flight; the two largest shapes would spill registers with it.
+  if (!vec && (config == RLK_GEMM_CFG_256x256 || config == RLK_GEMM_CFG_256x128)) config = RLK_GEMM_CFG_128x128;
   switch (config) {
-    case RLK_GEMM_CFG_256x256: return launch_shape<Shape256x256>(W, X, C, ldc, M, N, K, vec, out_f32, stream);
-    case RLK_GEMM_CFG_256x128: return launch_shape<Shape256x128>(W, X, C, ldc, M, N, K, vec, out_f32, stream);
-    case RLK_GEMM_CFG_128x128: return launch_shape<Shape128x128>(W, X, C, ldc, M, N, K, vec, out_f32, stream);
-    case RLK_GEMM_CFG_128x64: return launch_shape<Shape128x64>(W, X, C, ldc, M, N, K, vec, out_f32, stream);
-    case RLK_GEMM_CFG_64x64: return launch_shape<Shape64x64>(W, X, C, ldc, M, N, K, vec, out_f32, stream);
-    case RLK_GEMM_CFG_64x16: return launch_shape<Shape64x16>(W, X, C, ldc, M, N, K, vec, out_f32, stream);
-    case RLK_GEMM_CFG_16x16: return launch_shape<Shape16x16>(W, X, C, ldc, M, N, K, vec, out_f32, stream);
-    default: return hipErrorInvalidValue;
+    case RLK_GEMM_CFG_256x256:
+      return launch_shape<Shape256x256>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);
+    case RLK_GEMM_CFG_256x128:
+      return launch_shape<Shape256x128>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);
+    case RLK_GEMM_CFG_128x128:
+      return launch_shape<Shape128x128>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);
+    case RLK_GEMM_CFG_128x64:
+      return launch_shape<Shape128x64>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);
+    case RLK_GEMM_CFG_64x64:
+      return launch_shape<Shape64x64>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);
+    case RLK_GEMM_CFG_64x16:
+      return launch_shape<Shape64x16>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);
+    case RLK_GEMM_CFG_16x16:
+      return launch_shape<Shape16x16>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);
+    default:
+      return hipErrorInvalidValue;
   }
 }
 

@@ -132,8 +132,8 @@ struct Stager {
 // of token
 //   m0 + wave_m*16*TM + jm*16 + (lane&15).
 template <class S, bool VEC>
-__device__ __forceinline__ void tile_mainloop(const MatView& W, const MatView& X, int n0, int m0, int K,
-                                              char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
+__device__ __forceinline__ void tile_mainloop_staged(const MatView& W, const MatView& X, int n0, int m0, int K,
+                                                     char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -206,6 +206,255 @@ __device__ __forceinline__ void tile_mainloop(const MatView& W, const MatView& X
     }
     __syncthreads();
   }
+}
+
+// ---------------------------------------------------------------------------
+// Fast main loop: direct global -> LDS loads and an 8-wave ping-pong schedule.
+//
+// global_load_lds_dwordx4 moves 64 x 16 bytes from 64 independent global
+// addresses into 1 KiB of consecutive LDS, i.e. eight 128-byte tile rows ("a
+// block"). Lane i lands on row (i >> 3), chunk position (i & 7) of the block, so
+// it fetches logical chunk (i & 7) ^ (i >> 3) of that row to reproduce the XOR
+// swizzle of lds_chunk_offset(). No VGPR staging and no ds_write.
+//
+// The eight waves form two groups (waves 0-3 and 4-7; one wave of each group
+// sits on every SIMD) that run half an iteration apart. While one group issues
+// its MFMAs for a K tile out of registers, the other reads its fragments of the
+// tile from LDS and starts the loads of a later tile, so the matrix pipe of a
+// SIMD always has a wave whose operands are already in registers, and a wave
+// that blocks on the memory pipeline never holds MFMAs back. Barriers are bare
+// s_barrier instructions with hand-placed s_waitcnt: the fence of
+// __syncthreads() would wait for every load in flight.
+//
+// Needs unit K stride, 16-byte aligned rows and K % 64 == 0. Same MFMA chain as
+// the staged loop, so the same bits.
+// ---------------------------------------------------------------------------
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* global_ptr_t;
+
+// s_waitcnt immediates (gfx9 encoding: vmcnt [3:0]+[15:14], expcnt [6:4], lgkmcnt [11:8]).
+constexpr int kWaitVm0 = 0x0f70;     // vmcnt(0)
+constexpr int kWaitLgkm0 = 0xc07f;   // lgkmcnt(0)
+constexpr int kWaitAll0 = 0x0070;    // vmcnt(0) lgkmcnt(0)
+constexpr int wait_vmcnt(int n) { return 0x0f70 | (n & 15) | ((n >> 4) << 14); }
+
+// s_barrier without a fence; the empty asm statements only stop the compiler
+// from moving memory operations across it.
+__device__ __forceinline__ void wg_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+// Who refills what. A block is 8 consecutive LDS rows of a stage (1 KiB, one
+// load instruction). With waves laid out 4 (features) x 2 (tokens), wave j and
+// wave 4 + j read the same 16*TN weight rows, waves 0-3 read token rows
+// [0, BM/2) and waves 4-7 token rows [BM/2, BM). A wave may overwrite a row
+// right after its own reads only if no other wave of its group reads that row
+// (a barrier orders the two groups, nothing orders the waves inside a group):
+//   late wave 4+j : the weight rows of column j, and a quarter of token rows [0, BM/2)
+//   early wave j  : a quarter of token rows [BM/2, BM)
+// For a block inside the matrix the 64 lane addresses are a uniform block base
+// plus a per-lane offset that is the same for every block, so a wave keeps a few
+// 32-bit lane offsets instead of one pointer per block; a block that crosses the
+// last row takes a slower path with per-lane clamping (rows past the edge are
+// computed and never stored).
+template <class S>
+struct DmaLoader {
+  static constexpr int kWaveRows = 16 * S::TN;
+  static constexpr int kWBlocksPerWave = kWaveRows / 8;     // late waves only
+  static constexpr int kXBlocksPerWave = (S::BM / 16) / 4;  // every wave
+  static constexpr int kLateLoads = kWBlocksPerWave + kXBlocksPerWave;
+  static constexpr int kEarlyLoads = kXBlocksPerWave;
+  static constexpr int kBlocksW = S::BN / 8;
+
+  const bf16_bits* w_base;  // W + n0 * ldw   (uniform)
+  const bf16_bits* x_base;  // X + m0 * ldx   (uniform)
+  int64_t ldw, ldx;
+  int n0, m0, n_rows, m_rows;
+  int rib;                 // row of this lane inside a block
+  int chunk_elems;         // element offset of this lane's 16-byte chunk inside a 64-wide K tile
+  uint32_t w_lane_off[2];  // by block parity: (feature offset of the lane) * ldw + chunk_elems
+  uint32_t x_lane_off;     // rib * ldx + chunk_elems
+
+  // Feature offset of lane row `rib` inside a weight block of parity p: LDS row
+  // r = 8 b + rib holds feature weight_row_of_lds_row(r), which is a block-uniform
+  // part plus (i >> 2) * kRun + (i & 3) with i = 8 p + rib.
+  static __device__ __forceinline__ int w_lane_row(int parity, int rib) {
+    const int i = parity * 8 + rib;
+    return (i >> 2) * S::kRun + (i & 3);
+  }
+
+  __device__ __forceinline__ void init(const MatView& W, const MatView& X, int n0_, int m0_, int lane) {
+    n0 = n0_;
+    m0 = m0_;
+    n_rows = W.rows;
+    m_rows = X.rows;
+    ldw = W.row_stride;
+    ldx = X.row_stride;
+    w_base = W.ptr + (int64_t)n0 * ldw;
+    x_base = X.ptr + (int64_t)m0 * ldx;
+    rib = lane >> 3;
+    chunk_elems = ((lane & 7) ^ rib) * kChunkElems;
+    w_lane_off[0] = (uint32_t)(w_lane_row(0, rib) * ldw) + chunk_elems;
+    w_lane_off[1] = (uint32_t)(w_lane_row(1, rib) * ldw) + chunk_elems;
+    x_lane_off = (uint32_t)(rib * ldx) + chunk_elems;
+  }
+
+  __device__ __forceinline__ void load_w_block(char* stage, int k0, int b) const {
+    const int r0 = b * 8;
+    const int row0 = (r0 / kWaveRows) * kWaveRows + ((r0 % kWaveRows) / 16) * 4;  // block-uniform feature offset
+    const int parity = b & 1;
+    const bf16_bits* src;
+    if (n0 + row0 + (parity * 2 + 1) * S::kRun + 3 < n_rows) {
+      src = w_base + (int64_t)row0 * ldw + k0 + w_lane_off[parity];
+    } else {
+      int g = n0 + row0 + w_lane_row(parity, rib);
+      g = g < n_rows ? g : n_rows - 1;
+      src = w_base + (int64_t)(g - n0) * ldw + k0 + chunk_elems;
+    }
+    __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + b * 1024), 16, 0, 0);
+  }
+
+  __device__ __forceinline__ void load_x_block(char* stage, int k0, int xb) const {
+    const int row0 = xb * 8;
+    const bf16_bits* src;
+    if (m0 + row0 + 7 < m_rows) {
+      src = x_base + (int64_t)row0 * ldx + k0 + x_lane_off;
+    } else {
+      int g = m0 + row0 + rib;
+      g = g < m_rows ? g : m_rows - 1;
+      src = x_base + (int64_t)(g - m0) * ldx + k0 + chunk_elems;
+    }
+    __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + (kBlocksW + xb) * 1024), 16, 0, 0);
+  }
+
+  // `wave` is the workgroup wave index 0..7.
+  __device__ __forceinline__ void issue_early(char* stage, int k0, int wave) const {
+#pragma unroll
+    for (int j = 0; j < kXBlocksPerWave; ++j) load_x_block(stage, k0, S::BM / 16 + wave * kXBlocksPerWave + j);
+  }
+  __device__ __forceinline__ void issue_late(char* stage, int k0, int wave) const {
+    const int col = wave - 4;
+#pragma unroll
+    for (int j = 0; j < kWBlocksPerWave; ++j) load_w_block(stage, k0, col * kWBlocksPerWave + j);
+#pragma unroll
+    for (int j = 0; j < kXBlocksPerWave; ++j) load_x_block(stage, k0, col * kXBlocksPerWave + j);
+  }
+};
+
+template <class S>
+constexpr bool pingpong_supported() {
+  return S::WN == 4 && S::WM == 2 && S::BM % 64 == 0;
+}
+
+template <class S>
+__device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const MatView& X, int n0, int m0, int K,
+                                                       char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
+  static_assert(pingpong_supported<S>(), "two groups of four waves, 4 x 2 wave layout");
+  using Loader = DmaLoader<S>;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_n = wave % S::WN;
+  const int wave_m = wave / S::WN;
+  const bool late_group = wave >= 4;
+
+  Loader loader;
+  loader.init(W, X, n0, m0, lane);
+
+#pragma unroll
+  for (int jn = 0; jn < S::TN; ++jn)
+#pragma unroll
+    for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const int l16 = lane & 15;
+  const int grp = lane >> 4;
+  const int frag_lo = (grp ^ (l16 & 7)) << 4;
+  const int w_row_base = (wave_n * 16 * S::TN + l16) * kRowBytes;
+  const int x_row_base = S::BN * kRowBytes + (wave_m * 16 * S::TM + l16) * kRowBytes;
+
+  const int nk = K / kTileK;
+  // Loads past the last tile re-fetch the last tile into a stage nobody reads
+  // any more; that keeps the number of loads in flight (and so every s_waitcnt
+  // immediate) the same in every iteration.
+  auto tile_k = [&](int t) { return (t < nk ? t : nk - 1) * kTileK; };
+  auto stage = [&](int t) { return lds + (t & 1) * S::kStageBytes; };
+
+  u32x4_t w0[S::TN], x0[S::TM], w1[S::TN], x1[S::TM];
+  auto read_tile = [&](int t) {
+    const char* st = stage(t);
+#pragma unroll
+    for (int jm = 0; jm < S::TM; ++jm)
+      x0[jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + frag_lo);
+#pragma unroll
+    for (int jn = 0; jn < S::TN; ++jn)
+      w0[jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + frag_lo);
+#pragma unroll
+    for (int jm = 0; jm < S::TM; ++jm)
+      x1[jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + (frag_lo ^ 64));
+#pragma unroll
+    for (int jn = 0; jn < S::TN; ++jn)
+      w1[jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + (frag_lo ^ 64));
+  };
+  auto compute = [&]() {
+    __builtin_amdgcn_s_setprio(2);
+#pragma unroll
+    for (int jn = 0; jn < S::TN; ++jn)
+#pragma unroll
+      for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = mfma_16x16x32(w0[jn], x0[jm], acc[jn][jm]);
+#pragma unroll
+    for (int jn = 0; jn < S::TN; ++jn)
+#pragma unroll
+      for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = mfma_16x16x32(w1[jn], x1[jm], acc[jn][jm]);
+    __builtin_amdgcn_s_setprio(0);
+  };
+
+  // Phases are the intervals between consecutive workgroup barriers:
+  //   phase 2t     : early group reads tile t        | late group computes tile t-1
+  //   phase 2t + 1 : early group computes tile t     | late group reads tile t
+  // Tile t lives in stage t & 1, which is read in phases 2t and 2t + 1 and first
+  // read again (tile t + 2) in phase 2t + 4. Every wave waits for its own
+  // fragment reads before the barrier that ends its read phase.
+  //   late wave, phase 2t + 1: after its own reads, starts its part of tile t + 2
+  //     (rows only it and, one phase earlier, the early group read); it confirms
+  //     that part at the end of phase 2t + 3, behind the loads it starts there.
+  //   early wave, phase 2t + 2: starts its part of tile t + 2 (rows only the late
+  //     group read, one phase earlier); confirms it at the end of phase 2t + 3.
+  if (!late_group) {
+    loader.issue_early(stage(0), 0, wave);
+    loader.issue_early(stage(1), tile_k(1), wave);
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt(Loader::kEarlyLoads));  // my part of tile 0 has landed
+    wg_barrier();
+    for (int t = 0; t < nk; ++t) {
+      read_tile(t);
+      if (t > 0) loader.issue_early(stage(t + 1), tile_k(t + 1), wave);
+      __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // my fragments are in registers
+      wg_barrier();
+      compute();
+      __builtin_amdgcn_s_waitcnt(kWaitVm0);  // my part of tile t+1 has landed
+      wg_barrier();
+    }
+    wg_barrier();  // pairs with the late group's leading barrier
+  } else {
+    loader.issue_late(stage(0), 0, wave);
+    loader.issue_late(stage(1), tile_k(1), wave);
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt(Loader::kLateLoads));  // my part of tile 0 has landed
+    wg_barrier();
+    wg_barrier();  // half an iteration behind the early group
+    for (int t = 0; t < nk; ++t) {
+      read_tile(t);
+      __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // my fragments are in registers
+      loader.issue_late(stage(t), tile_k(t + 2), wave);
+      __builtin_amdgcn_s_waitcnt(wait_vmcnt(Loader::kLateLoads));  // my part of tile t+1 has landed
+      wg_barrier();
+      compute();
+      wg_barrier();
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(kWaitAll0);
+  wg_barrier();  // callers reuse the LDS after the loop
 }
 
 }  // namespace rlk

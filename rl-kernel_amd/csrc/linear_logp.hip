@@ -54,7 +54,8 @@ struct LogpArgs {
   int tiles_m, n_split, group_m;
 };
 
-template <class S, bool VEC>
+// LOOP: 0 generic element loader, 1 register-staged 16-byte loads, 2 direct-to-LDS ping-pong.
+template <class S, int LOOP>
 __global__ __launch_bounds__(S::kThreads) void linear_logp_partial_kernel(LogpArgs a) {
   static_assert(S::BN == kLogpTileCols && S::kRun == 16 && S::WN == 4, "stream layout is pinned");
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -100,7 +101,11 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_partial_kernel(LogpAr
     const int v0 = split * kLogpSplitCols + t * kLogpTileCols;
     if (v0 >= a.V) break;
     f32x4_t acc[S::TN][S::TM];
-    tile_mainloop<S, VEC>(a.W, a.H, v0, m0, a.D, lds, acc);
+    if constexpr (LOOP == 2) {
+      tile_mainloop_pingpong<S>(a.W, a.H, v0, m0, a.D, lds, acc);
+    } else {
+      tile_mainloop_staged<S, LOOP == 1>(a.W, a.H, v0, m0, a.D, lds, acc);
+    }
 
     const int col0 = v0 + stream * 16;  // first column of this lane's run
     float bias_run[16];
@@ -202,7 +207,7 @@ __global__ void linear_logp_merge_kernel(const float* __restrict__ part, float* 
 
 using LogpShape256 = TileShape<256, 256, 4, 2>;
 using LogpShape128 = TileShape<256, 128, 4, 2>;
-using LogpShape64 = TileShape<256, 64, 4, 1>;
+using LogpShape64 = TileShape<256, 64, 4, 2>;
 using LogpShape16 = TileShape<256, 16, 4, 1>;
 
 int linear_logp_split_count(int V) { return (V + kLogpSplitCols - 1) / kLogpSplitCols; }
@@ -211,9 +216,9 @@ size_t linear_logp_workspace_bytes(int T, int V) {
   return (size_t)3 * linear_logp_split_count(V) * (size_t)(T > 0 ? T : 0) * sizeof(float);
 }
 
-template <class S, bool VEC>
+template <class S, int LOOP>
 static hipError_t launch_logp(LogpArgs a, hipStream_t stream) {
-  auto kernel = linear_logp_partial_kernel<S, VEC>;
+  auto kernel = linear_logp_partial_kernel<S, LOOP>;
   constexpr int kMergeBytes = 3 * kLogpStreams * S::BM * (int)sizeof(float);
   constexpr int kLds = S::kLdsBytes > kMergeBytes ? S::kLdsBytes : kMergeBytes;
   static bool configured[kMaxDevices] = {};
@@ -261,21 +266,28 @@ hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t*
   const bool vec = W.k_stride == 1 && H.k_stride == 1 && (W.row_stride % kChunkElems) == 0 &&
                    (H.row_stride % kChunkElems) == 0 && (reinterpret_cast<uintptr_t>(W.ptr) & 15) == 0 &&
                    (reinterpret_cast<uintptr_t>(H.ptr) & 15) == 0 && (D % kChunkElems) == 0;
+  const bool force_staged = (config & RLK_LOGP_CFG_FORCE_STAGED) != 0;
+  config &= ~RLK_LOGP_CFG_FORCE_STAGED;
   if (config == RLK_LOGP_CFG_AUTO) config = pick_linear_logp_config(T, V);
   if (!vec && config == RLK_LOGP_CFG_256) config = RLK_LOGP_CFG_128;
+  const int loop = !vec ? 0 : (D % kTileK == 0 && !force_staged) ? 2 : 1;
   hipError_t err;
   switch (config) {
     case RLK_LOGP_CFG_256:
-      err = launch_logp<LogpShape256, true>(a, stream);
+      err = loop == 2 ? launch_logp<LogpShape256, 2>(a, stream) : launch_logp<LogpShape256, 1>(a, stream);
       break;
     case RLK_LOGP_CFG_128:
-      err = vec ? launch_logp<LogpShape128, true>(a, stream) : launch_logp<LogpShape128, false>(a, stream);
+      err = loop == 2   ? launch_logp<LogpShape128, 2>(a, stream)
+            : loop == 1 ? launch_logp<LogpShape128, 1>(a, stream)
+                        : launch_logp<LogpShape128, 0>(a, stream);
       break;
     case RLK_LOGP_CFG_64:
-      err = vec ? launch_logp<LogpShape64, true>(a, stream) : launch_logp<LogpShape64, false>(a, stream);
+      err = loop == 2   ? launch_logp<LogpShape64, 2>(a, stream)
+            : loop == 1 ? launch_logp<LogpShape64, 1>(a, stream)
+                        : launch_logp<LogpShape64, 0>(a, stream);
       break;
     case RLK_LOGP_CFG_16:
-      err = vec ? launch_logp<LogpShape16, true>(a, stream) : launch_logp<LogpShape16, false>(a, stream);
+      err = loop >= 1 ? launch_logp<LogpShape16, 1>(a, stream) : launch_logp<LogpShape16, 0>(a, stream);
       break;
     default:
       return hipErrorInvalidValue;

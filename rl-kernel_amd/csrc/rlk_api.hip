@@ -64,7 +64,7 @@ int rlk_det_gemm_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stride, c
     set_last_error("rlk_det_gemm_bf16: operands must not use negative strides");
     return RLK_ERR_INVALID_ARGUMENT;
   }
-  if (config < 0 || config >= RLK_GEMM_CFG_COUNT) {
+  if (config < 0 || (config & ~RLK_GEMM_CFG_FORCE_STAGED) >= RLK_GEMM_CFG_COUNT) {
     set_last_error("rlk_det_gemm_bf16: unknown config %d", config);
     return RLK_ERR_INVALID_ARGUMENT;
   }
@@ -110,7 +110,7 @@ int rlk_linear_logp_fwd(const void* hidden, int64_t h_row_stride, const void* we
     set_last_error("rlk_linear_logp_fwd: real_vocab_end must be in [1, %d], got %d", V, real_vocab_end);
     return RLK_ERR_INVALID_ARGUMENT;
   }
-  if (config < 0 || config >= RLK_LOGP_CFG_COUNT) {
+  if (config < 0 || (config & ~RLK_LOGP_CFG_FORCE_STAGED) >= RLK_LOGP_CFG_COUNT) {
     set_last_error("rlk_linear_logp_fwd: unknown config %d", config);
     return RLK_ERR_INVALID_ARGUMENT;
   }

@@ -31,6 +31,8 @@ GEMM_CONFIGS = {
     "64x16": 6,
     "16x16": 7,
 }
+# OR-ed into a GEMM or LogP configuration: register-staged main loop (bit-neutral).
+FORCE_STAGED = 0x100
 # rlk_logp_config
 LOGP_CONFIGS = {"auto": 0, "256": 1, "128": 2, "64": 3, "16": 4}
 

@@ -115,8 +115,26 @@ def test_every_tile_configuration_gives_the_same_bits(gemm, oracle, shape):
     w = inputs.randn_bf16(22, n, k, 0.02).to(DEV)
     base = gemm.mfma_gemm(a, w.t(), config="256x256")
     _assert_parity(oracle, base, a, w, f"{shape}")
-    for name in _lib.GEMM_CONFIGS:
+    for name, value in _lib.GEMM_CONFIGS.items():
         assert _same_bits(gemm.mfma_gemm(a, w.t(), config=name), base), name
+        assert _same_bits(gemm.mfma_gemm(a, w.t(), config=value | _lib.FORCE_STAGED), base), f"{name} staged"
+
+
+@pytest.mark.parametrize("shape", [(512, 1024, 4096), (300, 520, 256), (64, 64, 64), (1000, 777 * 8, 128)])
+def test_pingpong_and_staged_main_loops_give_the_same_bits(gemm, shape):
+    """K % 64 == 0 shapes take the direct-to-LDS ping-pong loop; forcing the
+    register-staged loop must not change a bit, in any tile configuration,
+    repeatedly (the ping-pong loop is the one with hand-placed waits)."""
+    from rl_engine import _lib
+
+    m, n, k = shape
+    a = inputs.randn_bf16(23, m, k).to(DEV)
+    w = inputs.randn_bf16(24, n, k, 0.02).to(DEV)
+    base = gemm.mfma_gemm(a, w.t(), config=_lib.GEMM_CONFIGS["16x16"])
+    for name, value in _lib.GEMM_CONFIGS.items():
+        for _ in range(3):
+            assert _same_bits(gemm.mfma_gemm(a, w.t(), config=value), base), name
+        assert _same_bits(gemm.mfma_gemm(a, w.t(), config=value | _lib.FORCE_STAGED), base), f"{name} staged"
 
 
 # ---------------------------------------------------------------------------

@@ -61,7 +61,7 @@ def test_golden_small_case(logp_mod):
     assert bool((logp2 <= 0).all())
 
 
-@pytest.mark.parametrize("shape", [(40, 3000, 264), (300, 2500, 128), (5, 1024, 64), (130, 5000, 512), (96, 4099, 320)])
+@pytest.mark.parametrize("shape", [(40, 3000, 264), (300, 2500, 128), (5, 1024, 64), (130, 5000, 512), (96, 4099, 320), (700, 9000, 256)])
 def test_parity_with_oracle_and_config_neutrality(logp_mod, oracle, shape):
     from rl_engine import _lib
 
@@ -80,6 +80,9 @@ def test_parity_with_oracle_and_config_neutrality(logp_mod, oracle, shape):
         if base is None:
             base = (logp, lse)
         assert _same_bits(logp, base[0]) and _same_bits(lse, base[1]), name
+        if name != "auto":
+            staged = logp_mod.deterministic_linear_logp(h_d, w_d, t_d, config=_lib.LOGP_CONFIGS[name] | _lib.FORCE_STAGED)
+            assert _same_bits(staged[0], base[0]) and _same_bits(staged[1], base[1]), f"{name} staged"
     assert np.abs(base[0].cpu().numpy() - ref_logp).max() < 5e-5  # what the kernel actually achieves
 
 
