@@ -40,7 +40,7 @@ HIDDEN, INTER, VOCAB = 4096, 12288, 151936
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs of this script (profiles/det_gemm_gate_up_T4096_pmc.md), scaled
 # by the same counters read on a plain device copy of known size. None = not measured.
-MEASURED_TRAFFIC_BYTES = {"det_gemm_gate_up_T4096": None}
+MEASURED_TRAFFIC_BYTES = {"det_gemm_gate_up_T4096": 1.412e9}  # 1.209 GB fetched + 0.203 GB written
 
 
 def _parse():
@@ -51,7 +51,7 @@ def _parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-logp", action="store_true", help="skip the linear-LogP leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-T table")
-    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|logp|copy")
+    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|logp|copy (used for profiling)")
     return ap.parse_args()
 
 
@@ -137,6 +137,14 @@ def main() -> int:
             torch.add(src, 0.0, out=dst)
         torch.cuda.synchronize()
         print(json.dumps({"leg": "copy", "bytes_read": src.numel() * 2, "bytes_written": dst.numel() * 2, "launches": 3}))
+        return 0
+    if args.only == "logp":
+        tl = 8192
+        hid = randn(tl, HIDDEN)
+        w_lm = randn(VOCAB, HIDDEN, 0.02)
+        tgt = torch.randint(0, VOCAB, (tl,), generator=gen, device=dev)
+        ms = _time_calls(lambda: deterministic_linear_logp(hid, w_lm, tgt), args.steps, args.warmup)
+        print(json.dumps({"leg": "logp", "ms": ms, "tokens_per_s": tl / ms * 1e3, "launches": args.steps + args.warmup}))
         return 0
     if args.only in ("gate_up", "down"):
         fn = gate_up if args.only == "gate_up" else down
