@@ -44,7 +44,9 @@ typedef enum rlk_gemm_config {
   RLK_GEMM_CFG_64x64 = 5,
   RLK_GEMM_CFG_64x16 = 6,
   RLK_GEMM_CFG_16x16 = 7,
-  RLK_GEMM_CFG_COUNT = 8,
+  RLK_GEMM_CFG_STREAM16_DEEP = 8, /* M <= 16: 16-feature panel per workgroup, 512-wide ring stages */
+  RLK_GEMM_CFG_STREAM16 = 9,      /* M <= 16: same with 256-wide ring stages, two workgroups per CU */
+  RLK_GEMM_CFG_COUNT = 10,
   /* OR-ed into a configuration: use the register-staged main loop even where the
    * direct-to-LDS ping-pong loop applies. Bit-neutral; exists so tests can
    * compare the two loops. */

@@ -161,7 +161,9 @@ static int64_t tile_count(int M, int N, int bm, int bn) {
 int pick_det_gemm_config(int M, int N, int K) {
   (void)K;
   constexpr int kCus = 256;
-  if (M <= 16) return N >= 64 * kCus ? RLK_GEMM_CFG_64x16 : RLK_GEMM_CFG_16x16;
+  // Decode: many short panels keep the chip busy with one wave each; few long
+  // panels need the streaming kernel's deep ring.
+  if (M <= 16) return N >= 64 * kCus ? RLK_GEMM_CFG_16x16 : RLK_GEMM_CFG_STREAM16_DEEP;
   // Estimated time = (rounds of 256 workgroups) x (tile area / measured relative
   // throughput of the shape when the chip is full). Larger tiles win ties.
   struct Candidate {
@@ -196,6 +198,14 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
   // The element-wise loader of the generic path keeps eight values per chunk in
   // flight; the two largest shapes would spill registers with it.
   if (!vec && (config == RLK_GEMM_CFG_256x256 || config == RLK_GEMM_CFG_256x128)) config = RLK_GEMM_CFG_128x128;
+  if (config == RLK_GEMM_CFG_STREAM16_DEEP || config == RLK_GEMM_CFG_STREAM16) {
+    // The streaming kernel serves one 16-token tile and needs the fast layout; otherwise the
+    // 16x16 tile kernel computes the same bits.
+    if (M <= 16 && vec && allow_pingpong && K % kTileK == 0) {
+      return det_gemm_stream_launch(W, X, C, ldc, M, N, K, out_f32, config == RLK_GEMM_CFG_STREAM16 ? 1 : 0, stream);
+    }
+    config = M <= 16 ? RLK_GEMM_CFG_16x16 : pick_det_gemm_config(M, N, K);
+  }
   switch (config) {
     case RLK_GEMM_CFG_256x256:
       return launch_shape<Shape256x256>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);

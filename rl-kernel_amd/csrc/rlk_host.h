@@ -18,6 +18,10 @@ int pick_det_gemm_config(int M, int N, int K);
 hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
                            bool out_f32, int config, hipStream_t stream);
 
+// Decode-sized batches (M <= 16), unit K stride, K % 64 == 0.
+hipError_t det_gemm_stream_launch(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
+                                  bool out_f32, int variant, hipStream_t stream);
+
 hipError_t fill_zero_launch(void* dst, int64_t rows, int64_t cols, int64_t ld, int elem_bytes,
                             hipStream_t stream);
 

@@ -30,6 +30,8 @@ GEMM_CONFIGS = {
     "64x64": 5,
     "64x16": 6,
     "16x16": 7,
+    "stream16_deep": 8,
+    "stream16": 9,
 }
 # OR-ed into a GEMM or LogP configuration: register-staged main loop (bit-neutral).
 FORCE_STAGED = 0x100

@@ -120,7 +120,7 @@ def test_every_tile_configuration_gives_the_same_bits(gemm, oracle, shape):
         assert _same_bits(gemm.mfma_gemm(a, w.t(), config=value | _lib.FORCE_STAGED), base), f"{name} staged"
 
 
-@pytest.mark.parametrize("shape", [(512, 1024, 4096), (300, 520, 256), (64, 64, 64), (1000, 777 * 8, 128)])
+@pytest.mark.parametrize("shape", [(512, 1024, 4096), (300, 520, 256), (64, 64, 64), (1000, 777 * 8, 128), (16, 4096, 12288), (1, 1000, 4096), (8, 72, 64), (9, 40, 1600)])
 def test_pingpong_and_staged_main_loops_give_the_same_bits(gemm, shape):
     """K % 64 == 0 shapes take the direct-to-LDS ping-pong loop; forcing the
     register-staged loop must not change a bit, in any tile configuration,
