@@ -46,7 +46,8 @@ typedef enum rlk_gemm_config {
   RLK_GEMM_CFG_16x16 = 7,
   RLK_GEMM_CFG_STREAM16_DEEP = 8, /* M <= 16: 16-feature panel per workgroup, 512-wide ring stages */
   RLK_GEMM_CFG_STREAM16 = 9,      /* M <= 16: same with 256-wide ring stages, two workgroups per CU */
-  RLK_GEMM_CFG_COUNT = 10,
+  RLK_GEMM_CFG_256x64 = 10,
+  RLK_GEMM_CFG_COUNT = 11,
   /* OR-ed into a configuration: use the register-staged main loop even where the
    * direct-to-LDS ping-pong loop applies. Bit-neutral; exists so tests can
    * compare the two loops. */

@@ -12,7 +12,8 @@ namespace rlk {
 // LOOP selects the main loop: kLoopGeneric (any strides, element loads),
 // kLoopStaged (16-byte loads through registers) or kLoopPingPong (direct-to-LDS
 // loads, two wave groups half an iteration apart). All three run the same MFMA chain.
-enum : int { kLoopGeneric = 0, kLoopStaged = 1, kLoopPingPong = 2 };
+// kLoopPingPongKMajor is the ping-pong loop for a K-major weight operand (B[K,N], N contiguous).
+enum : int { kLoopGeneric = 0, kLoopStaged = 1, kLoopPingPong = 2, kLoopPingPongKMajor = 3 };
 
 template <class S, int LOOP, bool OUT_F32>
 __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatView X, void* __restrict__ C,
@@ -35,7 +36,9 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
   const int m0 = tile_m * S::BM;
 
   f32x4_t acc[S::TN][S::TM];
-  if constexpr (LOOP == kLoopPingPong) {
+  if constexpr (LOOP == kLoopPingPongKMajor) {
+    tile_mainloop_pingpong<S, true>(W, X, n0, m0, K, lds, acc);
+  } else if constexpr (LOOP == kLoopPingPong) {
     tile_mainloop_pingpong<S>(W, X, n0, m0, K, lds, acc);
   } else {
     tile_mainloop_staged<S, LOOP == kLoopStaged>(W, X, n0, m0, K, lds, acc);
@@ -47,6 +50,43 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
   const int wave_m = wave / S::WN;
   const int n_run = n0 + wave_n * 16 * S::TN + (lane >> 4) * S::kRun;  // first feature of this lane's run
   const int m_lane = m0 + wave_m * 16 * S::TM + (lane & 15);
+
+  if constexpr (LOOP == kLoopPingPongKMajor) {
+    // No run permutation on this path: MFMA tile jn holds features jn*16 + (lane>>4)*4 + q.
+    const int n_tile = n0 + wave_n * 16 * S::TN + (lane >> 4) * 4;
+#pragma unroll
+    for (int jm = 0; jm < S::TM; ++jm) {
+      const int m = m_lane + jm * 16;
+      if (m >= M) continue;
+#pragma unroll
+      for (int jn = 0; jn < S::TN; ++jn) {
+        const int n = n_tile + jn * 16;
+        if (OUT_F32) {
+          float* dst = reinterpret_cast<float*>(C) + (int64_t)m * ldc + n;
+          if (n + 4 <= N && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+            *reinterpret_cast<f32x4_t*>(dst) = acc[jn][jm];
+          } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              if (n + q < N) dst[q] = acc[jn][jm][q];
+          }
+        } else {
+          bf16_bits* dst = reinterpret_cast<bf16_bits*>(C) + (int64_t)m * ldc + n;
+          const uint32_t lo = pack_bf16x2(acc[jn][jm][0], acc[jn][jm][1]);
+          const uint32_t hi = pack_bf16x2(acc[jn][jm][2], acc[jn][jm][3]);
+          if (n + 4 <= N && (reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
+            *reinterpret_cast<u32x2_t*>(dst) = u32x2_t{lo, hi};
+          } else {
+            const uint32_t packed[2] = {lo, hi};
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              if (n + q < N) dst[q] = (bf16_bits)((packed[q >> 1] >> ((q & 1) * 16)) & 0xffffu);
+          }
+        }
+      }
+    }
+    return;
+  }
 
 #pragma unroll
   for (int jm = 0; jm < S::TM; ++jm) {
@@ -125,7 +165,13 @@ static hipError_t launch_tile(const MatView& W, const MatView& X, void* C, int64
 
 template <class S>
 static hipError_t launch_shape(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
-                               bool vec, bool allow_pingpong, bool out_f32, hipStream_t stream) {
+                               bool vec, bool w_kmajor, bool allow_pingpong, bool out_f32, hipStream_t stream) {
+  if constexpr (pingpong_supported<S>() && S::TN == 4) {
+    if (w_kmajor && allow_pingpong) {
+      return out_f32 ? launch_tile<S, kLoopPingPongKMajor, true>(W, X, C, ldc, M, N, K, stream)
+                     : launch_tile<S, kLoopPingPongKMajor, false>(W, X, C, ldc, M, N, K, stream);
+    }
+  }
   if constexpr (pingpong_supported<S>()) {
     if (vec && allow_pingpong && K % kTileK == 0) {
       return out_f32 ? launch_tile<S, kLoopPingPong, true>(W, X, C, ldc, M, N, K, stream)
@@ -143,6 +189,7 @@ static hipError_t launch_shape(const MatView& W, const MatView& X, void* C, int6
 // Tile shapes. Which one runs is a pure performance choice (see det_gemm_tile.h).
 using Shape256x256 = TileShape<256, 256, 4, 2>;
 using Shape256x128 = TileShape<256, 128, 4, 2>;
+using Shape256x64 = TileShape<256, 64, 4, 2>;
 using Shape128x128 = TileShape<128, 128, 4, 2>;
 using Shape128x64 = TileShape<128, 64, 4, 2>;
 using Shape64x64 = TileShape<64, 64, 4, 2>;
@@ -172,6 +219,7 @@ int pick_det_gemm_config(int M, int N, int K) {
   };
   static const Candidate kCandidates[] = {
       {RLK_GEMM_CFG_256x256, 256, 256, 1.00}, {RLK_GEMM_CFG_256x128, 256, 128, 0.95},
+      {RLK_GEMM_CFG_256x64, 256, 64, 0.75},
       {RLK_GEMM_CFG_128x128, 128, 128, 0.90}, {RLK_GEMM_CFG_128x64, 128, 64, 0.70},
       {RLK_GEMM_CFG_64x64, 64, 64, 0.55},
   };
@@ -189,15 +237,37 @@ int pick_det_gemm_config(int M, int N, int K) {
   return best;
 }
 
+// A K-major weight view (B[K,N] with N contiguous) that the transposing ping-pong loop can take.
+static bool weight_is_kmajor_fast(const MatView& W, const MatView& X, int N, int K) {
+  return W.row_stride == 1 && W.k_stride >= N && (W.k_stride % kChunkElems) == 0 &&
+         (reinterpret_cast<uintptr_t>(W.ptr) & 15) == 0 && (N % kChunkElems) == 0 && view_is_vectorizable(X) &&
+         (K % kTileK) == 0;
+}
+
 hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
                            bool out_f32, int config, hipStream_t stream) {
   const bool vec = view_is_vectorizable(W) && view_is_vectorizable(X) && (K % kChunkElems) == 0;
   const bool allow_pingpong = (config & RLK_GEMM_CFG_FORCE_STAGED) == 0;
   config &= ~RLK_GEMM_CFG_FORCE_STAGED;
+  const bool w_kmajor = !vec && allow_pingpong && weight_is_kmajor_fast(W, X, N, K);
+  if (w_kmajor) {
+    // Only the shapes with 64-feature wave columns have the transposing loop.
+    if (config == RLK_GEMM_CFG_AUTO) {
+      const int64_t t256 = tile_count(M, N, 256, 256), t128 = tile_count(M, N, 128, 256);
+      config = M <= 64 ? RLK_GEMM_CFG_256x64 : (M > 128 && t256 >= 256) ? RLK_GEMM_CFG_256x256 : t128 >= 128 ? RLK_GEMM_CFG_256x128 : RLK_GEMM_CFG_256x64;
+    }
+    switch (config) {
+      case RLK_GEMM_CFG_256x256:
+        return launch_shape<Shape256x256>(W, X, C, ldc, M, N, K, false, true, true, out_f32, stream);
+      case RLK_GEMM_CFG_256x128:
+        return launch_shape<Shape256x128>(W, X, C, ldc, M, N, K, false, true, true, out_f32, stream);
+      case RLK_GEMM_CFG_256x64:
+        return launch_shape<Shape256x64>(W, X, C, ldc, M, N, K, false, true, true, out_f32, stream);
+      default:
+        break;  // an explicitly requested other shape runs the element-wise loader below
+    }
+  }
   if (config == RLK_GEMM_CFG_AUTO) config = pick_det_gemm_config(M, N, K);
-  // The element-wise loader of the generic path keeps eight values per chunk in
-  // flight; the two largest shapes would spill registers with it.
-  if (!vec && (config == RLK_GEMM_CFG_256x256 || config == RLK_GEMM_CFG_256x128)) config = RLK_GEMM_CFG_128x128;
   if (config == RLK_GEMM_CFG_STREAM16_DEEP || config == RLK_GEMM_CFG_STREAM16) {
     // The streaming kernel serves one 16-token tile and needs the fast layout; otherwise the
     // 16x16 tile kernel computes the same bits.
@@ -206,21 +276,27 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
     }
     config = M <= 16 ? RLK_GEMM_CFG_16x16 : pick_det_gemm_config(M, N, K);
   }
+  // The element-wise loader of the generic path keeps eight values per chunk in
+  // flight; the largest shapes would spill registers with it.
+  if (!vec && (config == RLK_GEMM_CFG_256x256 || config == RLK_GEMM_CFG_256x128 || config == RLK_GEMM_CFG_256x64))
+    config = RLK_GEMM_CFG_128x128;
   switch (config) {
     case RLK_GEMM_CFG_256x256:
-      return launch_shape<Shape256x256>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape256x256>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
     case RLK_GEMM_CFG_256x128:
-      return launch_shape<Shape256x128>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape256x128>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
+    case RLK_GEMM_CFG_256x64:
+      return launch_shape<Shape256x64>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
     case RLK_GEMM_CFG_128x128:
-      return launch_shape<Shape128x128>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape128x128>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
     case RLK_GEMM_CFG_128x64:
-      return launch_shape<Shape128x64>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape128x64>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
     case RLK_GEMM_CFG_64x64:
-      return launch_shape<Shape64x64>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape64x64>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
     case RLK_GEMM_CFG_64x16:
-      return launch_shape<Shape64x16>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape64x16>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
     case RLK_GEMM_CFG_16x16:
-      return launch_shape<Shape16x16>(W, X, C, ldc, M, N, K, vec, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape16x16>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
     default:
       return hipErrorInvalidValue;
   }

@@ -260,9 +260,21 @@ __device__ __forceinline__ void wg_barrier() {
 // 32-bit lane offsets instead of one pointer per block; a block that crosses the
 // last row takes a slower path with per-lane clamping (rows past the edge are
 // computed and never stored).
-template <class S>
+//
+// WK = true serves a weight operand stored K-major (B[K,N] with N contiguous, the
+// `a @ b` and prepared-weight form). Its stage keeps, per 64-feature wave column,
+// 64 K rows of 128 bytes (64 features); a block is 8 K rows of one column, so the
+// ownership rule above is unchanged. Fragments come from ds_read_b64_tr_b16, which
+// hands lane i of a 16-lane group the four K values of feature i out of 4 K rows x
+// 16 features. The 16-byte chunk (8 features) at K row k sits at chunk position
+// c ^ kmajor_swizzle(k), which keeps both the loads and the transposing reads
+// free of bank conflicts. Needs TN == 4 (64-feature columns) and N % 8 == 0.
+__device__ __forceinline__ int kmajor_swizzle(int k_row) { return 2 * (((k_row >> 1) & 1) ^ ((k_row >> 3) & 3)); }
+
+template <class S, bool WK = false>
 struct DmaLoader {
   static constexpr int kWaveRows = 16 * S::TN;
+  static_assert(!WK || S::TN == 4, "K-major weights need 64-feature wave columns");
   static constexpr int kWBlocksPerWave = kWaveRows / 8;     // late waves only
   static constexpr int kXBlocksPerWave = (S::BM / 16) / 4;  // every wave
   static constexpr int kLateLoads = kWBlocksPerWave + kXBlocksPerWave;
@@ -291,18 +303,38 @@ struct DmaLoader {
     m0 = m0_;
     n_rows = W.rows;
     m_rows = X.rows;
-    ldw = W.row_stride;
+    ldw = WK ? W.k_stride : W.row_stride;  // K-major: elements between consecutive K rows
     ldx = X.row_stride;
-    w_base = W.ptr + (int64_t)n0 * ldw;
+    w_base = WK ? W.ptr + n0 : W.ptr + (int64_t)n0 * ldw;
     x_base = X.ptr + (int64_t)m0 * ldx;
     rib = lane >> 3;
     chunk_elems = ((lane & 7) ^ rib) * kChunkElems;
-    w_lane_off[0] = (uint32_t)(w_lane_row(0, rib) * ldw) + chunk_elems;
-    w_lane_off[1] = (uint32_t)(w_lane_row(1, rib) * ldw) + chunk_elems;
+    if (WK) {
+      // lane -> (K row rib of the block, chunk position lane & 7); the K-row part of the
+      // swizzle that does not depend on the block is folded in here.
+      w_lane_off[0] = (uint32_t)(rib * ldw);
+      w_lane_off[1] = (uint32_t)((lane & 7) ^ (2 * ((rib >> 1) & 1)));  // chunk before the block part of the swizzle
+    } else {
+      w_lane_off[0] = (uint32_t)(w_lane_row(0, rib) * ldw) + chunk_elems;
+      w_lane_off[1] = (uint32_t)(w_lane_row(1, rib) * ldw) + chunk_elems;
+    }
     x_lane_off = (uint32_t)(rib * ldx) + chunk_elems;
   }
 
   __device__ __forceinline__ void load_w_block(char* stage, int k0, int b) const {
+    if constexpr (WK) {
+      const int col = b >> 3;   // 64-feature wave column
+      const int kblk = b & 7;   // K rows 8 kblk .. 8 kblk + 7 of the tile
+      const int chunk = (int)w_lane_off[1] ^ (2 * (kblk & 3));
+      int n = col * 64 + chunk * kChunkElems;  // feature offset inside the tile
+      if (n0 + col * 64 + 64 > n_rows) {        // column crosses the last feature (N % 8 == 0 here)
+        const int last = n_rows - kChunkElems - n0;
+        n = n < last ? n : last;
+      }
+      const bf16_bits* src = w_base + (int64_t)(k0 + kblk * 8) * ldw + w_lane_off[0] + n;
+      __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + b * 1024), 16, 0, 0);
+      return;
+    }
     const int r0 = b * 8;
     const int row0 = (r0 / kWaveRows) * kWaveRows + ((r0 % kWaveRows) / 16) * 4;  // block-uniform feature offset
     const int parity = b & 1;
@@ -349,11 +381,13 @@ constexpr bool pingpong_supported() {
   return S::WN == 4 && S::WM == 2 && S::BM % 64 == 0;
 }
 
-template <class S>
+// With WK the accumulator of MFMA tile jn holds features wave_n*64 + jn*16 + (lane>>4)*4 + q
+// (no run permutation: a K-major chunk is eight consecutive features).
+template <class S, bool WK = false>
 __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const MatView& X, int n0, int m0, int K,
                                                        char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
   static_assert(pingpong_supported<S>(), "two groups of four waves, 4 x 2 wave layout");
-  using Loader = DmaLoader<S>;
+  using Loader = DmaLoader<S, WK>;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -382,6 +416,23 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
   auto tile_k = [&](int t) { return (t < nk ? t : nk - 1) * kTileK; };
   auto stage = [&](int t) { return lds + (t & 1) * S::kStageBytes; };
 
+  // K-major weight fragments: the transposing read takes, from lane r of a 16-lane group, the
+  // address of 4 features at K row (r >> 2), features 4 (r & 3) .. +3 of the MFMA tile.
+  typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+  typedef __attribute__((address_space(3))) bf16x4_t* lds_bf16x4_ptr_t;
+  auto read_w_kmajor = [&](const char* st, int jn, int step) -> u32x4_t {
+    const char* col = st + wave_n * (64 * kRowBytes);
+    u32x2_t half[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int k_row = step * 32 + grp * 8 + h * 4 + (l16 >> 2);
+      const int chunk = (2 * jn + ((l16 & 3) >> 1)) ^ kmajor_swizzle(k_row);
+      const char* p = col + k_row * kRowBytes + chunk * 16 + (l16 & 1) * 8;
+      half[h] = __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr_t)p));
+    }
+    return u32x4_t{half[0].x, half[0].y, half[1].x, half[1].y};
+  };
+
   u32x4_t w0[S::TN], x0[S::TM], w1[S::TN], x1[S::TM];
   auto read_tile = [&](int t) {
     const char* st = stage(t);
@@ -389,14 +440,24 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
     for (int jm = 0; jm < S::TM; ++jm)
       x0[jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + frag_lo);
 #pragma unroll
-    for (int jn = 0; jn < S::TN; ++jn)
-      w0[jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + frag_lo);
+    for (int jn = 0; jn < S::TN; ++jn) {
+      if constexpr (WK) {
+        w0[jn] = read_w_kmajor(st, jn, 0);
+      } else {
+        w0[jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + frag_lo);
+      }
+    }
 #pragma unroll
     for (int jm = 0; jm < S::TM; ++jm)
       x1[jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + (frag_lo ^ 64));
 #pragma unroll
-    for (int jn = 0; jn < S::TN; ++jn)
-      w1[jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + (frag_lo ^ 64));
+    for (int jn = 0; jn < S::TN; ++jn) {
+      if constexpr (WK) {
+        w1[jn] = read_w_kmajor(st, jn, 1);
+      } else {
+        w1[jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + (frag_lo ^ 64));
+      }
+    }
   };
   auto compute = [&]() {
     __builtin_amdgcn_s_setprio(2);

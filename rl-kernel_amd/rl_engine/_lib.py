@@ -32,6 +32,7 @@ GEMM_CONFIGS = {
     "16x16": 7,
     "stream16_deep": 8,
     "stream16": 9,
+    "256x64": 10,
 }
 # OR-ed into a GEMM or LogP configuration: register-staged main loop (bit-neutral).
 FORCE_STAGED = 0x100

@@ -261,6 +261,34 @@ def test_operand_layouts_give_the_same_bits(gemm, native, shape):
     assert _same_bits(native.det_gemm_fwd_rhs_transposed(a, unaligned), expected)
 
 
+@pytest.mark.parametrize("shape", [(512, 1024, 4096), (300, 1000, 192), (1000, 2056, 320), (64, 8, 64), (7, 1024, 1024), (2048, 4096, 1024)])
+def test_kmajor_weight_fast_path_gives_the_same_bits(gemm, native, shape):
+    """B[K,N] with N contiguous (the `a @ b`, prepared-weight and input-gradient
+    form) is read through transposing LDS loads in three tile shapes. Each must
+    equal the [N,K] path bit for bit, including N edges inside a 256-wide tile, a
+    row-padded weight and a weight view whose base is not 16-byte aligned (which
+    has to fall back to the element loader)."""
+    m, n, k = shape
+    a = inputs.randn_bf16(53, m, k).to(DEV)
+    bt = inputs.randn_bf16(54, n, k, 0.02).to(DEV)  # [N,K]
+    b = bt.t().contiguous()  # [K,N]
+    expected = gemm.mfma_gemm(a, bt.t(), config="16x16")
+    for name in ("auto", "256x256", "256x128", "256x64", "128x128"):
+        for _ in range(2):
+            assert _same_bits(gemm.mfma_gemm(a, b, config=name), expected), name
+    padded = torch.zeros((k, n + 24), dtype=torch.bfloat16, device=DEV)
+    padded[:, 8 : 8 + n] = b
+    assert _same_bits(gemm.mfma_gemm(a, padded[:, 8 : 8 + n]), expected)
+    shifted = torch.zeros((k, n + 8), dtype=torch.bfloat16, device=DEV)
+    shifted[:, 1 : 1 + n] = b
+    assert _same_bits(gemm.mfma_gemm(a, shifted[:, 1 : 1 + n]), expected)
+    # fp32 output: same accumulator from both layouts, and it rounds to the bf16 result
+    acc_kn = native.det_gemm_fwd_out_fp32(a, b)
+    acc_nk = native.det_gemm_fwd_out_fp32(a, bt.t())
+    assert torch.equal(acc_kn.view(torch.int32), acc_nk.view(torch.int32))
+    assert _same_bits(acc_kn.to(torch.bfloat16), expected)
+
+
 @pytest.mark.parametrize("k", (1, 8, 31, 32, 33, 65, 100, 1000))
 def test_ragged_k_equals_zero_padded_k(gemm, k):
     a = inputs.randn_bf16(61, 9, k).to(DEV)
