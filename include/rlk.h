@@ -70,9 +70,12 @@ const char* rlk_last_error(void);
  *
  * A is addressed as a[m*a_row_stride + k*a_k_stride], B as
  * b[k*b_k_stride + n*b_n_stride], C as c[m*ldc + n]. Any non-negative strides
- * are accepted; the fast path needs a_k_stride == 1 and b_k_stride == 1 (the
- * native [N,K] linear weight), 16-byte aligned bases, K % 8 == 0 and row
- * strides % 8 == 0. Other layouts run a slower loader with identical results.
+ * are accepted. Fast paths, per operand: reduction axis contiguous (a_k_stride == 1;
+ * b_k_stride == 1, the native [N,K] linear weight) with K % 8 == 0 and row strides
+ * % 8 == 0; or, when K % 64 == 0, the other axis contiguous (a_row_stride == 1 with
+ * M % 8 == 0, the transposed operand of a weight gradient; b_n_stride == 1 with
+ * N % 8 == 0, a plain B[K,N]) with k strides % 8 == 0. Bases 16-byte aligned. Other
+ * layouts run a slower element loader with identical results.
  * C must not alias A or B.
  *
  * One entry point serves rl_engine._C.det_gemm_fwd, det_gemm_fwd_rhs_transposed,

@@ -12,8 +12,19 @@ namespace rlk {
 // LOOP selects the main loop: kLoopGeneric (any strides, element loads),
 // kLoopStaged (16-byte loads through registers) or kLoopPingPong (direct-to-LDS
 // loads, two wave groups half an iteration apart). All three run the same MFMA chain.
-// kLoopPingPongKMajor is the ping-pong loop for a K-major weight operand (B[K,N], N contiguous).
-enum : int { kLoopGeneric = 0, kLoopStaged = 1, kLoopPingPong = 2, kLoopPingPongKMajor = 3 };
+// The K-major variants are the ping-pong loop with the weight operand (B[K,N], N contiguous),
+// the activation operand (x[k * ld + m], tokens contiguous) or both read through transposing
+// LDS loads.
+enum : int {
+  kLoopGeneric = 0,
+  kLoopStaged = 1,
+  kLoopPingPong = 2,
+  kLoopPingPongKMajor = 3,   // weight K-major
+  kLoopPingPongXKMajor = 4,  // activation K-major
+  kLoopPingPongBothKMajor = 5
+};
+constexpr bool loop_weight_kmajor(int loop) { return loop == kLoopPingPongKMajor || loop == kLoopPingPongBothKMajor; }
+constexpr bool loop_act_kmajor(int loop) { return loop == kLoopPingPongXKMajor || loop == kLoopPingPongBothKMajor; }
 
 template <class S, int LOOP, bool OUT_F32>
 __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatView X, void* __restrict__ C,
@@ -36,8 +47,8 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
   const int m0 = tile_m * S::BM;
 
   f32x4_t acc[S::TN][S::TM];
-  if constexpr (LOOP == kLoopPingPongKMajor) {
-    tile_mainloop_pingpong<S, true>(W, X, n0, m0, K, lds, acc);
+  if constexpr (LOOP >= kLoopPingPongKMajor) {
+    tile_mainloop_pingpong<S, loop_weight_kmajor(LOOP), loop_act_kmajor(LOOP)>(W, X, n0, m0, K, lds, acc);
   } else if constexpr (LOOP == kLoopPingPong) {
     tile_mainloop_pingpong<S>(W, X, n0, m0, K, lds, acc);
   } else {
@@ -51,7 +62,7 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
   const int n_run = n0 + wave_n * 16 * S::TN + (lane >> 4) * S::kRun;  // first feature of this lane's run
   const int m_lane = m0 + wave_m * 16 * S::TM + (lane & 15);
 
-  if constexpr (LOOP == kLoopPingPongKMajor) {
+  if constexpr (loop_weight_kmajor(LOOP)) {
     // No run permutation on this path: MFMA tile jn holds features jn*16 + (lane>>4)*4 + q.
     const int n_tile = n0 + wave_n * 16 * S::TN + (lane >> 4) * 4;
 #pragma unroll
@@ -163,27 +174,33 @@ static hipError_t launch_tile(const MatView& W, const MatView& X, void* C, int64
   return hipGetLastError();
 }
 
+template <class S, int LOOP>
+static hipError_t launch_loop(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
+                              bool out_f32, hipStream_t stream) {
+  return out_f32 ? launch_tile<S, LOOP, true>(W, X, C, ldc, M, N, K, stream)
+                 : launch_tile<S, LOOP, false>(W, X, C, ldc, M, N, K, stream);
+}
+
+// kmajor_loop: 0, or the K-major ping-pong variant the operand layouts call for.
 template <class S>
 static hipError_t launch_shape(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
-                               bool vec, bool w_kmajor, bool allow_pingpong, bool out_f32, hipStream_t stream) {
+                               bool vec, int kmajor_loop, bool allow_pingpong, bool out_f32, hipStream_t stream) {
   if constexpr (pingpong_supported<S>() && S::TN == 4) {
-    if (w_kmajor && allow_pingpong) {
-      return out_f32 ? launch_tile<S, kLoopPingPongKMajor, true>(W, X, C, ldc, M, N, K, stream)
-                     : launch_tile<S, kLoopPingPongKMajor, false>(W, X, C, ldc, M, N, K, stream);
+    if (kmajor_loop == kLoopPingPongKMajor)
+      return launch_loop<S, kLoopPingPongKMajor>(W, X, C, ldc, M, N, K, out_f32, stream);
+    if constexpr (S::BM % 128 == 0) {
+      if (kmajor_loop == kLoopPingPongXKMajor)
+        return launch_loop<S, kLoopPingPongXKMajor>(W, X, C, ldc, M, N, K, out_f32, stream);
+      if (kmajor_loop == kLoopPingPongBothKMajor)
+        return launch_loop<S, kLoopPingPongBothKMajor>(W, X, C, ldc, M, N, K, out_f32, stream);
     }
   }
+  if (kmajor_loop != 0) return hipErrorInvalidValue;
   if constexpr (pingpong_supported<S>()) {
-    if (vec && allow_pingpong && K % kTileK == 0) {
-      return out_f32 ? launch_tile<S, kLoopPingPong, true>(W, X, C, ldc, M, N, K, stream)
-                     : launch_tile<S, kLoopPingPong, false>(W, X, C, ldc, M, N, K, stream);
-    }
+    if (vec && allow_pingpong && K % kTileK == 0) return launch_loop<S, kLoopPingPong>(W, X, C, ldc, M, N, K, out_f32, stream);
   }
-  if (vec) {
-    return out_f32 ? launch_tile<S, kLoopStaged, true>(W, X, C, ldc, M, N, K, stream)
-                   : launch_tile<S, kLoopStaged, false>(W, X, C, ldc, M, N, K, stream);
-  }
-  return out_f32 ? launch_tile<S, kLoopGeneric, true>(W, X, C, ldc, M, N, K, stream)
-                 : launch_tile<S, kLoopGeneric, false>(W, X, C, ldc, M, N, K, stream);
+  if (vec) return launch_loop<S, kLoopStaged>(W, X, C, ldc, M, N, K, out_f32, stream);
+  return launch_loop<S, kLoopGeneric>(W, X, C, ldc, M, N, K, out_f32, stream);
 }
 
 // Tile shapes. Which one runs is a pure performance choice (see det_gemm_tile.h).
@@ -237,32 +254,40 @@ int pick_det_gemm_config(int M, int N, int K) {
   return best;
 }
 
-// A K-major weight view (B[K,N] with N contiguous) that the transposing ping-pong loop can take.
-static bool weight_is_kmajor_fast(const MatView& W, const MatView& X, int N, int K) {
-  return W.row_stride == 1 && W.k_stride >= N && (W.k_stride % kChunkElems) == 0 &&
-         (reinterpret_cast<uintptr_t>(W.ptr) & 15) == 0 && (N % kChunkElems) == 0 && view_is_vectorizable(X) &&
-         (K % kTileK) == 0;
+// A K-major view (element [row, k] at ptr[k * k_stride + row], rows contiguous: B[K,N] as the
+// weight operand, or the transposed operands of a weight gradient) that the transposing
+// ping-pong loop can take.
+static bool view_is_kmajor_fast(const MatView& v) {
+  return v.row_stride == 1 && v.k_stride >= v.rows && (v.k_stride % kChunkElems) == 0 &&
+         (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0 && (v.rows % kChunkElems) == 0;
 }
 
 hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
                            bool out_f32, int config, hipStream_t stream) {
-  const bool vec = view_is_vectorizable(W) && view_is_vectorizable(X) && (K % kChunkElems) == 0;
+  const bool w_native = view_is_vectorizable(W), x_native = view_is_vectorizable(X);
+  const bool vec = w_native && x_native && (K % kChunkElems) == 0;
   const bool allow_pingpong = (config & RLK_GEMM_CFG_FORCE_STAGED) == 0;
   config &= ~RLK_GEMM_CFG_FORCE_STAGED;
-  const bool w_kmajor = !vec && allow_pingpong && weight_is_kmajor_fast(W, X, N, K);
-  if (w_kmajor) {
-    // Only the shapes with 64-feature wave columns have the transposing loop.
+  const bool w_kmajor = !w_native && view_is_kmajor_fast(W), x_kmajor = !x_native && view_is_kmajor_fast(X);
+  if (allow_pingpong && (K % kTileK) == 0 && (w_kmajor || x_kmajor) && (w_native || w_kmajor) &&
+      (x_native || x_kmajor)) {
+    const int loop = w_kmajor ? (x_kmajor ? kLoopPingPongBothKMajor : kLoopPingPongKMajor) : kLoopPingPongXKMajor;
+    // Only the shapes with 64-feature wave columns have the transposing loop, and a K-major
+    // activation needs at least 128 tokens per tile.
     if (config == RLK_GEMM_CFG_AUTO) {
       const int64_t t256 = tile_count(M, N, 256, 256), t128 = tile_count(M, N, 128, 256);
-      config = M <= 64 ? RLK_GEMM_CFG_256x64 : (M > 128 && t256 >= 256) ? RLK_GEMM_CFG_256x256 : t128 >= 128 ? RLK_GEMM_CFG_256x128 : RLK_GEMM_CFG_256x64;
+      config = (M > 128 && t256 >= 256) ? RLK_GEMM_CFG_256x256
+               : (t128 >= 128 || M > 64 || x_kmajor) ? RLK_GEMM_CFG_256x128
+                                                     : RLK_GEMM_CFG_256x64;
     }
     switch (config) {
       case RLK_GEMM_CFG_256x256:
-        return launch_shape<Shape256x256>(W, X, C, ldc, M, N, K, false, true, true, out_f32, stream);
+        return launch_shape<Shape256x256>(W, X, C, ldc, M, N, K, false, loop, true, out_f32, stream);
       case RLK_GEMM_CFG_256x128:
-        return launch_shape<Shape256x128>(W, X, C, ldc, M, N, K, false, true, true, out_f32, stream);
+        return launch_shape<Shape256x128>(W, X, C, ldc, M, N, K, false, loop, true, out_f32, stream);
       case RLK_GEMM_CFG_256x64:
-        return launch_shape<Shape256x64>(W, X, C, ldc, M, N, K, false, true, true, out_f32, stream);
+        if (!x_kmajor) return launch_shape<Shape256x64>(W, X, C, ldc, M, N, K, false, loop, true, out_f32, stream);
+        break;
       default:
         break;  // an explicitly requested other shape runs the element-wise loader below
     }
@@ -282,21 +307,21 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
     config = RLK_GEMM_CFG_128x128;
   switch (config) {
     case RLK_GEMM_CFG_256x256:
-      return launch_shape<Shape256x256>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape256x256>(W, X, C, ldc, M, N, K, vec, 0, allow_pingpong, out_f32, stream);
     case RLK_GEMM_CFG_256x128:
-      return launch_shape<Shape256x128>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape256x128>(W, X, C, ldc, M, N, K, vec, 0, allow_pingpong, out_f32, stream);
     case RLK_GEMM_CFG_256x64:
-      return launch_shape<Shape256x64>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape256x64>(W, X, C, ldc, M, N, K, vec, 0, allow_pingpong, out_f32, stream);
     case RLK_GEMM_CFG_128x128:
-      return launch_shape<Shape128x128>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape128x128>(W, X, C, ldc, M, N, K, vec, 0, allow_pingpong, out_f32, stream);
     case RLK_GEMM_CFG_128x64:
-      return launch_shape<Shape128x64>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape128x64>(W, X, C, ldc, M, N, K, vec, 0, allow_pingpong, out_f32, stream);
     case RLK_GEMM_CFG_64x64:
-      return launch_shape<Shape64x64>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape64x64>(W, X, C, ldc, M, N, K, vec, 0, allow_pingpong, out_f32, stream);
     case RLK_GEMM_CFG_64x16:
-      return launch_shape<Shape64x16>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape64x16>(W, X, C, ldc, M, N, K, vec, 0, allow_pingpong, out_f32, stream);
     case RLK_GEMM_CFG_16x16:
-      return launch_shape<Shape16x16>(W, X, C, ldc, M, N, K, vec, false, allow_pingpong, out_f32, stream);
+      return launch_shape<Shape16x16>(W, X, C, ldc, M, N, K, vec, 0, allow_pingpong, out_f32, stream);
     default:
       return hipErrorInvalidValue;
   }

@@ -269,12 +269,18 @@ __device__ __forceinline__ void wg_barrier() {
 // 16 features. The 16-byte chunk (8 features) at K row k sits at chunk position
 // c ^ kmajor_swizzle(k), which keeps both the loads and the transposing reads
 // free of bank conflicts. Needs TN == 4 (64-feature columns) and N % 8 == 0.
+//
+// XK = true is the same for the activation operand (X addressed as x[k * ldx + m],
+// tokens contiguous: the transposed operands of a weight gradient). Its stage keeps
+// 64-token columns of 64 K rows; a wave group must own whole columns, so BM % 128 == 0,
+// and M % 8 == 0.
 __device__ __forceinline__ int kmajor_swizzle(int k_row) { return 2 * (((k_row >> 1) & 1) ^ ((k_row >> 3) & 3)); }
 
-template <class S, bool WK = false>
+template <class S, bool WK = false, bool XK = false>
 struct DmaLoader {
   static constexpr int kWaveRows = 16 * S::TN;
   static_assert(!WK || S::TN == 4, "K-major weights need 64-feature wave columns");
+  static_assert(!XK || S::BM % 128 == 0, "K-major activations need whole 64-token columns per wave group");
   static constexpr int kWBlocksPerWave = kWaveRows / 8;     // late waves only
   static constexpr int kXBlocksPerWave = (S::BM / 16) / 4;  // every wave
   static constexpr int kLateLoads = kWBlocksPerWave + kXBlocksPerWave;
@@ -289,6 +295,7 @@ struct DmaLoader {
   int chunk_elems;         // element offset of this lane's 16-byte chunk inside a 64-wide K tile
   uint32_t w_lane_off[2];  // by block parity: (feature offset of the lane) * ldw + chunk_elems
   uint32_t x_lane_off;     // rib * ldx + chunk_elems
+  int kmajor_chunk;        // K-major operands: chunk position of this lane before the block part of the swizzle
 
   // Feature offset of lane row `rib` inside a weight block of parity p: LDS row
   // r = 8 b + rib holds feature weight_row_of_lds_row(r), which is a block-uniform
@@ -304,34 +311,42 @@ struct DmaLoader {
     n_rows = W.rows;
     m_rows = X.rows;
     ldw = WK ? W.k_stride : W.row_stride;  // K-major: elements between consecutive K rows
-    ldx = X.row_stride;
+    ldx = XK ? X.k_stride : X.row_stride;
     w_base = WK ? W.ptr + n0 : W.ptr + (int64_t)n0 * ldw;
-    x_base = X.ptr + (int64_t)m0 * ldx;
+    x_base = XK ? X.ptr + m0 : X.ptr + (int64_t)m0 * ldx;
     rib = lane >> 3;
     chunk_elems = ((lane & 7) ^ rib) * kChunkElems;
+    // K-major: lane -> (K row rib of the block, chunk position lane & 7); the K-row part
+    // of the swizzle that does not depend on the block is folded in here.
+    kmajor_chunk = (lane & 7) ^ (2 * ((rib >> 1) & 1));
     if (WK) {
-      // lane -> (K row rib of the block, chunk position lane & 7); the K-row part of the
-      // swizzle that does not depend on the block is folded in here.
       w_lane_off[0] = (uint32_t)(rib * ldw);
-      w_lane_off[1] = (uint32_t)((lane & 7) ^ (2 * ((rib >> 1) & 1)));  // chunk before the block part of the swizzle
+      w_lane_off[1] = 0;
     } else {
       w_lane_off[0] = (uint32_t)(w_lane_row(0, rib) * ldw) + chunk_elems;
       w_lane_off[1] = (uint32_t)(w_lane_row(1, rib) * ldw) + chunk_elems;
     }
-    x_lane_off = (uint32_t)(rib * ldx) + chunk_elems;
+    x_lane_off = XK ? (uint32_t)(rib * ldx) : (uint32_t)(rib * ldx) + chunk_elems;
+  }
+
+  // Source of this lane's 16 bytes of K-major block `b` (8 K rows of one 64-wide column).
+  static __device__ __forceinline__ const bf16_bits* kmajor_src(const bf16_bits* base, int64_t ld, uint32_t lane_off,
+                                                                int kmajor_chunk, int first, int rows, int k0,
+                                                                int b) {
+    const int col = b >> 3;  // 64-wide column of the tile
+    const int kblk = b & 7;  // K rows 8 kblk .. 8 kblk + 7 of the tile
+    const int chunk = kmajor_chunk ^ (2 * (kblk & 3));
+    int at = col * 64 + chunk * kChunkElems;  // offset inside the tile along the contiguous axis
+    if (first + col * 64 + 64 > rows) {       // column crosses the edge (rows % 8 == 0 here)
+      const int last = rows - kChunkElems - first;
+      at = at < last ? at : last;
+    }
+    return base + (int64_t)(k0 + kblk * 8) * ld + lane_off + at;
   }
 
   __device__ __forceinline__ void load_w_block(char* stage, int k0, int b) const {
     if constexpr (WK) {
-      const int col = b >> 3;   // 64-feature wave column
-      const int kblk = b & 7;   // K rows 8 kblk .. 8 kblk + 7 of the tile
-      const int chunk = (int)w_lane_off[1] ^ (2 * (kblk & 3));
-      int n = col * 64 + chunk * kChunkElems;  // feature offset inside the tile
-      if (n0 + col * 64 + 64 > n_rows) {        // column crosses the last feature (N % 8 == 0 here)
-        const int last = n_rows - kChunkElems - n0;
-        n = n < last ? n : last;
-      }
-      const bf16_bits* src = w_base + (int64_t)(k0 + kblk * 8) * ldw + w_lane_off[0] + n;
+      const bf16_bits* src = kmajor_src(w_base, ldw, w_lane_off[0], kmajor_chunk, n0, n_rows, k0, b);
       __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + b * 1024), 16, 0, 0);
       return;
     }
@@ -350,6 +365,11 @@ struct DmaLoader {
   }
 
   __device__ __forceinline__ void load_x_block(char* stage, int k0, int xb) const {
+    if constexpr (XK) {
+      const bf16_bits* src = kmajor_src(x_base, ldx, x_lane_off, kmajor_chunk, m0, m_rows, k0, xb);
+      __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + (kBlocksW + xb) * 1024), 16, 0, 0);
+      return;
+    }
     const int row0 = xb * 8;
     const bf16_bits* src;
     if (m0 + row0 + 7 < m_rows) {
@@ -383,11 +403,11 @@ constexpr bool pingpong_supported() {
 
 // With WK the accumulator of MFMA tile jn holds features wave_n*64 + jn*16 + (lane>>4)*4 + q
 // (no run permutation: a K-major chunk is eight consecutive features).
-template <class S, bool WK = false>
+template <class S, bool WK = false, bool XK = false>
 __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const MatView& X, int n0, int m0, int K,
                                                        char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
   static_assert(pingpong_supported<S>(), "two groups of four waves, 4 x 2 wave layout");
-  using Loader = DmaLoader<S, WK>;
+  using Loader = DmaLoader<S, WK, XK>;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -416,29 +436,41 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
   auto tile_k = [&](int t) { return (t < nk ? t : nk - 1) * kTileK; };
   auto stage = [&](int t) { return lds + (t & 1) * S::kStageBytes; };
 
-  // K-major weight fragments: the transposing read takes, from lane r of a 16-lane group, the
-  // address of 4 features at K row (r >> 2), features 4 (r & 3) .. +3 of the MFMA tile.
+  // K-major fragments: the transposing read takes, from lane r of a 16-lane group, the address
+  // of 4 features (tokens) at K row (r >> 2), positions 4 (r & 3) .. +3 of MFMA tile `j16` of a
+  // 64-wide column.
   typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
   typedef __attribute__((address_space(3))) bf16x4_t* lds_bf16x4_ptr_t;
-  auto read_w_kmajor = [&](const char* st, int jn, int step) -> u32x4_t {
-    const char* col = st + wave_n * (64 * kRowBytes);
+  auto read_kmajor = [&](const char* col, int j16, int step) -> u32x4_t {
     u32x2_t half[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int k_row = step * 32 + grp * 8 + h * 4 + (l16 >> 2);
-      const int chunk = (2 * jn + ((l16 & 3) >> 1)) ^ kmajor_swizzle(k_row);
+      const int chunk = (2 * j16 + ((l16 & 3) >> 1)) ^ kmajor_swizzle(k_row);
       const char* p = col + k_row * kRowBytes + chunk * 16 + (l16 & 1) * 8;
       half[h] = __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr_t)p));
     }
     return u32x4_t{half[0].x, half[0].y, half[1].x, half[1].y};
+  };
+  auto read_w_kmajor = [&](const char* st, int jn, int step) -> u32x4_t {
+    return read_kmajor(st + wave_n * (64 * kRowBytes), jn, step);
+  };
+  auto read_x_kmajor = [&](const char* st, int jm, int step) -> u32x4_t {
+    const int col = wave_m * (S::TM / 4) + (jm >> 2);
+    return read_kmajor(st + S::BN * kRowBytes + col * (64 * kRowBytes), jm & 3, step);
   };
 
   u32x4_t w0[S::TN], x0[S::TM], w1[S::TN], x1[S::TM];
   auto read_tile = [&](int t) {
     const char* st = stage(t);
 #pragma unroll
-    for (int jm = 0; jm < S::TM; ++jm)
-      x0[jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + frag_lo);
+    for (int jm = 0; jm < S::TM; ++jm) {
+      if constexpr (XK) {
+        x0[jm] = read_x_kmajor(st, jm, 0);
+      } else {
+        x0[jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + frag_lo);
+      }
+    }
 #pragma unroll
     for (int jn = 0; jn < S::TN; ++jn) {
       if constexpr (WK) {
@@ -448,8 +480,13 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
       }
     }
 #pragma unroll
-    for (int jm = 0; jm < S::TM; ++jm)
-      x1[jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + (frag_lo ^ 64));
+    for (int jm = 0; jm < S::TM; ++jm) {
+      if constexpr (XK) {
+        x1[jm] = read_x_kmajor(st, jm, 1);
+      } else {
+        x1[jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + (frag_lo ^ 64));
+      }
+    }
 #pragma unroll
     for (int jn = 0; jn < S::TN; ++jn) {
       if constexpr (WK) {

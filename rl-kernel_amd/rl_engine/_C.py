@@ -126,9 +126,25 @@ def det_gemm_fwd_out_fp32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
 
 
 def _reduction_major(t: torch.Tensor) -> torch.Tensor:
-    """``t.t()`` with the (new) last axis contiguous; a plain copy when needed."""
+    """``t.t()`` ready for a GEMM whose reduction runs over ``t``'s rows.
+
+    A row-major ``t[M, C]`` with ``C % 8 == 0``, ``M % 64 == 0`` and 16-byte aligned
+    rows is passed as the plain view ``t.t()``: the library reads such a K-major
+    operand through transposing LDS loads. Anything else gets a value-preserving
+    copy with the reduction axis contiguous.
+    """
     tt = t.t()
-    return tt if tt.stride(1) == 1 else tt.contiguous()
+    if tt.stride(1) == 1:
+        return tt
+    if (
+        t.stride(1) == 1
+        and t.size(1) % 8 == 0
+        and t.size(0) % 64 == 0
+        and t.stride(0) % 8 == 0
+        and t.data_ptr() % 16 == 0
+    ):
+        return tt
+    return tt.contiguous()
 
 
 def det_gemm_da(dc: torch.Tensor, b: torch.Tensor) -> torch.Tensor:

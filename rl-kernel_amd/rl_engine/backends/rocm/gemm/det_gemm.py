@@ -131,10 +131,10 @@ def mfma_gemm(
     return out
 
 
-def _reduction_major_copy(tensor: torch.Tensor) -> torch.Tensor:
-    """``tensor.t()`` with the reduction axis contiguous (a value-preserving copy)."""
-    transposed = tensor.t()
-    return transposed if transposed.stride(1) == 1 else transposed.contiguous()
+def _reduction_major(tensor: torch.Tensor) -> torch.Tensor:
+    """``tensor.t()`` for a GEMM that reduces over ``tensor``'s rows: the plain view when
+    the library's K-major loader can take it, else a value-preserving copy."""
+    return _C._reduction_major(tensor)
 
 
 def mfma_linear(a: torch.Tensor, weight: torch.Tensor, *, out: torch.Tensor | None = None) -> torch.Tensor:
@@ -144,13 +144,13 @@ def mfma_linear(a: torch.Tensor, weight: torch.Tensor, *, out: torch.Tensor | No
 
 def mfma_linear_input_gradient(grad_output: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """``dX = dY @ W`` with ``W`` in native ``[N,K]`` layout."""
-    # The reduction runs over N, the slow axis of W: stage a reduction-major copy.
-    return mfma_gemm(grad_output, _reduction_major_copy(weight).t())
+    # The reduction runs over N, the slow axis of W: a K-major operand of the kernel.
+    return mfma_gemm(grad_output, _reduction_major(weight).t())
 
 
 def mfma_linear_weight_gradient(a: torch.Tensor, grad_output: torch.Tensor) -> torch.Tensor:
     """``dW = dY.T @ X`` returned in native ``[N,K]`` layout."""
-    return mfma_gemm(_reduction_major_copy(grad_output), _reduction_major_copy(a).t())
+    return mfma_gemm(_reduction_major(grad_output), _reduction_major(a).t())
 
 
 # ---------------------------------------------------------------------------
@@ -342,7 +342,7 @@ class MfmaGemmFn(torch.autograd.Function):
         a, b = ctx.saved_tensors
         grad_out = _as_bf16_grad(grad_out)
         da = mfma_gemm(grad_out, b.t()) if ctx.needs_input_grad[0] else None
-        db = mfma_gemm(_reduction_major_copy(a), _reduction_major_copy(grad_out).t()) if ctx.needs_input_grad[1] else None
+        db = mfma_gemm(_reduction_major(a), _reduction_major(grad_out).t()) if ctx.needs_input_grad[1] else None
         return da, db
 
 

@@ -264,7 +264,7 @@ def test_operand_layouts_give_the_same_bits(gemm, native, shape):
 @pytest.mark.parametrize("shape", [(512, 1024, 4096), (300, 1000, 192), (1000, 2056, 320), (64, 8, 64), (7, 1024, 1024), (2048, 4096, 1024)])
 def test_kmajor_weight_fast_path_gives_the_same_bits(gemm, native, shape):
     """B[K,N] with N contiguous (the `a @ b`, prepared-weight and input-gradient
-    form) is read through transposing LDS loads in three tile shapes. Each must
+    form) and token-contiguous activations are read through transposing LDS loads. Each must
     equal the [N,K] path bit for bit, including N edges inside a 256-wide tile, a
     row-padded weight and a weight view whose base is not 16-byte aligned (which
     has to fall back to the element loader)."""
@@ -276,6 +276,12 @@ def test_kmajor_weight_fast_path_gives_the_same_bits(gemm, native, shape):
     for name in ("auto", "256x256", "256x128", "256x64", "128x128"):
         for _ in range(2):
             assert _same_bits(gemm.mfma_gemm(a, b, config=name), expected), name
+    # the activation as a K-major view (tokens contiguous: the operands of a weight gradient),
+    # alone and together with the K-major weight; M % 8 != 0 falls back to the element loader
+    a_kmajor = a.t().contiguous().t()
+    for name in ("auto", "256x256", "256x128", "256x64"):
+        assert _same_bits(gemm.mfma_gemm(a_kmajor, bt.t(), config=name), expected), f"x k-major {name}"
+        assert _same_bits(gemm.mfma_gemm(a_kmajor, b, config=name), expected), f"both k-major {name}"
     padded = torch.zeros((k, n + 24), dtype=torch.bfloat16, device=DEV)
     padded[:, 8 : 8 + n] = b
     assert _same_bits(gemm.mfma_gemm(a, padded[:, 8 : 8 + n]), expected)
