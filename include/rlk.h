@@ -143,6 +143,37 @@ int rlk_linear_logp_fwd(const void* hidden, int64_t h_row_stride, const void* we
                         float* lse, void* workspace, size_t workspace_bytes, int T, int D, int V,
                         int64_t vocab_start, int real_vocab_end, int config, void* stream);
 
+/* Bytes of workspace rlk_linear_logp_bwd needs: the bf16 d(logits) [T, V rounded up to 64]
+ * plus, when a bias gradient is wanted, fp32 block sums [ceil(T / 256), V]. */
+size_t rlk_linear_logp_bwd_workspace_bytes(int T, int V, int with_bias);
+
+/*
+ * Backward of rlk_linear_logp_fwd. Inputs as in the forward, plus
+ *   lse        [T] fp32: the forward's result for the same inputs
+ *   grad_logp  [T] fp32 or NULL (zero);  grad_lse [T] fp32 or NULL (zero)
+ * Outputs (each may be NULL when not wanted):
+ *   grad_hidden [T, D] bf16, row stride gh_row_stride
+ *   grad_weight [V, D] bf16, row stride gw_row_stride
+ *   grad_bias   [V] fp32
+ * With p = exp(y - lse) on the forward's scaled logits y (0 on padded lanes),
+ *   d(logits) = (p * (grad_lse - grad_logp) + [column == target] * grad_logp) / temperature,
+ * rounded once to bf16; grad_hidden = d(logits) @ weight over the vocabulary ascending,
+ * grad_weight = d(logits)^T @ hidden over tokens ascending (both under the det_gemm
+ * contract), grad_bias = column sums of d(logits) in fixed 256-token blocks. The clamp
+ * logp = min(., 0) of the forward is not differentiated (gradient 1), as in the reference.
+ * workspace must be 256-byte aligned.
+ *
+ * Stands in for _DetTritonLinearLogpAutograd.backward and _det_reference_dlogits
+ * (rl_engine/backends/shared/triton/logprob/linear_logp.py:522-570, 600-628) and for
+ * chunked_linear_logp_backward (rl_engine/reference/logprob/linear_logp.py:642-715).
+ */
+int rlk_linear_logp_bwd(const void* hidden, int64_t h_row_stride, const void* weight, int64_t w_row_stride,
+                        const int64_t* target, const float* bias, const float* temperature, const float* lse,
+                        const float* grad_logp, const float* grad_lse, void* grad_hidden, int64_t gh_row_stride,
+                        void* grad_weight, int64_t gw_row_stride, float* grad_bias, void* workspace,
+                        size_t workspace_bytes, int T, int D, int V, int64_t vocab_start, int real_vocab_end,
+                        int config, void* stream);
+
 /* Bytes of workspace rlk_grpo_ratio_kl_loss needs. */
 size_t rlk_grpo_workspace_bytes(int rollouts);
 

@@ -26,6 +26,9 @@ Pinning (which check fixes which function; see tests/test_oracle.py):
 * ``linear_logp_chunked`` / ``linear_logp_dense``: uniform logits (logp = -log V),
   probabilities summing to one, the fp64 brute force, agreement between the
   chunked and the dense form, chunk-size independence.
+* ``linear_logp_dlogits`` / ``linear_logp_backward``: central finite differences of
+  ``linear_logp_f64`` in hidden, weight and bias; rows of d(logits) summing to
+  ``grad_lse / temperature``; zero hidden gradient when every weight row is the same.
 * ``grpo_ratio_kl_loss`` / ``group_advantages`` / ``masked_mean``: the reference's
   hand examples (tests/reference/test_reference_ops.py:77-98,
   tests/ops/loss/test_grpo_loss.py:112-119) and closed forms (old == logp gives
@@ -326,6 +329,90 @@ def linear_logp_f64(h_bits, w_bits, target, bias=None, *, temperature=None, real
     lse = m + np.log(np.exp(logits - m[:, None]).sum(axis=-1))
     zt = logits[np.arange(h.shape[0]), target]
     return zt - lse, lse
+
+
+def linear_logp_dlogits(
+    h_bits,
+    w_bits,
+    target,
+    lse,
+    grad_logp=None,
+    grad_lse=None,
+    bias=None,
+    *,
+    temperature=None,
+    real_vocab_size=-1,
+    dtype=np.float32,
+):
+    """d(logits) of the strict linear-LogP, recomputed from a saved ``lse``.
+
+    Restates _det_reference_dlogits
+    (rl_engine/backends/shared/triton/logprob/linear_logp.py:522-570): logits from the
+    fp32-upcast operands, divided by the temperature, padded lanes -inf;
+    ``probs = exp(logits - lse)``; ``dlogits = probs * (grad_lse - grad_logp)``, plus
+    ``grad_logp`` at the target column, divided by the temperature once more.
+    ``dtype`` float64 turns the same formula into the exact anchor.
+    """
+    h = bf16_to_f32(np.ascontiguousarray(h_bits, dtype=np.uint16)).astype(dtype)
+    w = bf16_to_f32(np.ascontiguousarray(w_bits, dtype=np.uint16)).astype(dtype)
+    target = np.asarray(target, dtype=np.int64).reshape(-1)
+    n = h.shape[0]
+    logits = h @ w.T
+    if bias is not None:
+        logits = logits + np.asarray(bias, dtype=np.float32).astype(dtype)
+    temp = None
+    if temperature is not None:
+        temp = np.broadcast_to(np.asarray(temperature, dtype=np.float32), (n,)).astype(dtype)
+        logits = logits / temp[:, None]
+    if real_vocab_size is not None and 0 <= real_vocab_size < logits.shape[1]:
+        logits[:, real_vocab_size:] = -np.inf
+    probs = np.exp(logits - np.asarray(lse, dtype=dtype).reshape(-1, 1))
+    g_logp = np.zeros((n,), dtype=dtype) if grad_logp is None else np.asarray(grad_logp, dtype=np.float32).astype(dtype)
+    g_lse = np.zeros((n,), dtype=dtype) if grad_lse is None else np.asarray(grad_lse, dtype=np.float32).astype(dtype)
+    dlogits = probs * (g_lse - g_logp)[:, None]
+    dlogits[np.arange(n), target] += g_logp
+    if temp is not None:
+        dlogits = dlogits / temp[:, None]
+    return dlogits.astype(dtype)
+
+
+def linear_logp_backward(
+    h_bits,
+    w_bits,
+    target,
+    lse,
+    grad_logp=None,
+    grad_lse=None,
+    bias=None,
+    *,
+    temperature=None,
+    real_vocab_size=-1,
+    round_dlogits_to_bf16: bool = True,
+):
+    """``(grad_hidden, grad_weight, grad_bias, dlogits)`` of the strict linear-LogP.
+
+    ``grad_hidden = dlogits @ W``, ``grad_weight = dlogits.T @ H``,
+    ``grad_bias = dlogits.sum(0)``
+    (_DetTritonLinearLogpAutograd.backward,
+    rl_engine/backends/shared/triton/logprob/linear_logp.py:600-628). With
+    ``round_dlogits_to_bf16`` the d(logits) are rounded to the weight dtype before the
+    two products, which is the bf16 branch of chunked_linear_logp_backward
+    (rl_engine/reference/logprob/linear_logp.py:698-703; its bias gradient sums the
+    unrounded values, :704-705). Products accumulate in fp64 here, so what is left to
+    the implementation under test is its summation order and the final rounding.
+    Gradients are returned as float64 arrays, dlogits as float32.
+    """
+    dz = linear_logp_dlogits(
+        h_bits, w_bits, target, lse, grad_logp, grad_lse, bias, temperature=temperature, real_vocab_size=real_vocab_size
+    )
+    h = bf16_to_f32(np.ascontiguousarray(h_bits, dtype=np.uint16)).astype(np.float64)
+    w = bf16_to_f32(np.ascontiguousarray(w_bits, dtype=np.uint16)).astype(np.float64)
+    used = bf16_to_f32(f32_to_bf16(dz)) if round_dlogits_to_bf16 else dz
+    used = used.astype(np.float64)
+    grad_hidden = used @ w
+    grad_weight = used.T @ h
+    grad_bias = dz.astype(np.float64).sum(axis=0)
+    return grad_hidden, grad_weight, grad_bias, dz
 
 
 # ---------------------------------------------------------------------------

@@ -26,20 +26,10 @@
 //   final merge over splits ascending with the same formula;
 //   lse = M + log(S);  zt = y_target;  logp = min(zt - lse, 0)
 //   e(x) = v_exp_f32(x * log2(e)) with an unfused fp32 multiply.
-#include "det_gemm_tile.h"
+#include "linear_logp_common.h"
 #include "rlk_host.h"
 
 namespace rlk {
-
-constexpr int kLogpTileCols = 256;
-constexpr int kLogpStreams = 16;
-constexpr int kLogpSplitTiles = 4;
-constexpr int kLogpSplitCols = kLogpTileCols * kLogpSplitTiles;
-constexpr float kNegInf = -__builtin_huge_valf();
-
-__device__ __forceinline__ float pinned_exp(float x) {
-  return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
-}
 
 struct LogpArgs {
   MatView W;  // [V, D] lm_head weight, rows = vocabulary
@@ -121,10 +111,8 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_partial_kernel(LogpAr
       float tmax = kNegInf;
 #pragma unroll
       for (int c = 0; c < 16; ++c) {
-        float z = acc[c >> 2][jm][c & 3];
-        if (a.bias) z = z + bias_run[c];
-        z = (col0 + c < a.vocab_limit) ? z : kNegInf;
-        if (a.temperature) z = z * inv_t[jm];
+        const float z = scaled_logit(acc[c >> 2][jm][c & 3], a.bias != nullptr, bias_run[c], col0 + c, a.vocab_limit,
+                                     a.temperature != nullptr, inv_t[jm]);
         y[c] = z;
         tmax = fmaxf(tmax, z);
       }

@@ -1,0 +1,286 @@
+// Backward of the fused linear-LogP for gfx950.
+//
+// Stands in for _DetTritonLinearLogpAutograd.backward + _det_reference_dlogits
+// (reference rl_engine/backends/shared/triton/logprob/linear_logp.py:522-570, 600-628)
+// and for the bf16 branch of chunked_linear_logp_backward
+// (rl_engine/reference/logprob/linear_logp.py:642-715): the logits are recomputed,
+// d(logits) is rounded to bf16 once and feeds two GEMMs.
+//
+// Three steps, all in fixed order:
+//   1. dlogits kernel. The same MFMA chain as the forward gives z; with y the scaled
+//      logit of the forward contract and lse the forward's saved value,
+//          p  = e(y - lse)                          (0 on padded lanes)
+//          dz = p * (g_lse - g_logp)                (+ g_logp at the target column)
+//          dz = dz * (1 / temperature)              when a temperature is given
+//      rounded once to bf16 and written to dz[T, ld] (the only [T, V]-sized buffer;
+//      2 bytes per logit).
+//   2. grad_hidden[T, D] = dz[T, V] @ W[V, D]: det_gemm over the vocabulary, ascending,
+//      with W read as a K-major operand. A row depends on that token's dz row only, so
+//      it is batch invariant like the forward.
+//   3. grad_weight[V, D] = dz^T[V, T] @ H[T, D]: det_gemm over tokens, ascending, both
+//      operands read K-major (no transposed copies).
+//      grad_bias[V] = column sums of the bf16 dz in fp32: 256-token blocks summed
+//      ascending inside a block, block sums added ascending.
+#include "linear_logp_common.h"
+#include "rlk_host.h"
+
+namespace rlk {
+
+struct LogpBwdArgs {
+  MatView W;  // [V, D] lm_head weight
+  MatView H;  // [T, D] hidden states
+  const int64_t* target;
+  const float* bias;         // [V] or null
+  const float* temperature;  // [T] or null
+  const float* lse;          // [T] forward result
+  const float* grad_logp;    // [T] or null (= 0)
+  const float* grad_lse;     // [T] or null (= 0)
+  bf16_bits* dz;             // [T, ld_dz]
+  int64_t ld_dz;
+  int T, V, D;
+  int vocab_limit;
+  int64_t vocab_start;
+  int tiles_m, tiles_v, group_m;
+};
+
+// LOOP: 0 generic element loader, 1 register-staged 16-byte loads, 2 direct-to-LDS ping-pong.
+template <class S, int LOOP>
+__global__ __launch_bounds__(S::kThreads) void linear_logp_dlogits_kernel(LogpBwdArgs a) {
+  static_assert(S::BN == kLogpTileCols && S::kRun == 16 && S::WN == 4, "a lane owns 16 consecutive columns");
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int total = a.tiles_m * a.tiles_v;
+  const int id = xcd_compact_id(blockIdx.x, total);
+  const int per_group = a.group_m * a.tiles_v;
+  const int group = id / per_group;
+  const int first_m = group * a.group_m;
+  const int width = (a.tiles_m - first_m) < a.group_m ? (a.tiles_m - first_m) : a.group_m;
+  const int within = id - group * per_group;
+  const int tile_m = first_m + within % width;
+  const int tile_v = within / width;
+  const int m0 = tile_m * S::BM;
+  const int v0 = tile_v * kLogpTileCols;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wave_n = wave % S::WN;
+  const int wave_m = wave / S::WN;
+  const int l16 = lane & 15;
+  const int grp = lane >> 4;
+  const int tok_local = wave_m * 16 * S::TM + l16;
+  const int col0 = v0 + (wave_n * 4 + grp) * 16;  // first column of this lane's run
+
+  f32x4_t acc[S::TN][S::TM];
+  if constexpr (LOOP == 2) {
+    tile_mainloop_pingpong<S>(a.W, a.H, v0, m0, a.D, lds, acc);
+  } else {
+    tile_mainloop_staged<S, LOOP == 1>(a.W, a.H, v0, m0, a.D, lds, acc);
+  }
+
+  float bias_run[16];
+#pragma unroll
+  for (int c = 0; c < 16; ++c) bias_run[c] = 0.f;
+  if (a.bias) {
+#pragma unroll
+    for (int c = 0; c < 16; ++c) bias_run[c] = (col0 + c < a.V) ? a.bias[col0 + c] : 0.f;
+  }
+
+#pragma unroll
+  for (int jm = 0; jm < S::TM; ++jm) {
+    const int m = m0 + tok_local + jm * 16;
+    if (m >= a.T) continue;
+    const int64_t local = a.target[m] - a.vocab_start;
+    const int tl = (local >= 0 && local < a.vocab_limit) ? (int)local - col0 : -1;
+    const float inv_t = a.temperature ? 1.0f / a.temperature[m] : 1.0f;
+    const float row_lse = a.lse[m];
+    const float g_logp = a.grad_logp ? a.grad_logp[m] : 0.f;
+    const float g_lse = a.grad_lse ? a.grad_lse[m] : 0.f;
+    const float coeff = g_lse - g_logp;
+    uint32_t packed[8];
+#pragma unroll
+    for (int c = 0; c < 16; c += 2) {
+      float d[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int cc = c + e;
+        const float y = scaled_logit(acc[cc >> 2][jm][cc & 3], a.bias != nullptr, bias_run[cc], col0 + cc,
+                                     a.vocab_limit, a.temperature != nullptr, inv_t);
+        float v = pinned_exp(y - row_lse) * coeff;
+        if (tl == cc) v = v + g_logp;
+        if (a.temperature) v = v * inv_t;
+        d[e] = v;
+      }
+      packed[c >> 1] = pack_bf16x2(d[0], d[1]);
+    }
+    bf16_bits* dst = a.dz + (int64_t)m * a.ld_dz + col0;
+    if (col0 + 16 <= a.V) {
+      *reinterpret_cast<u32x4_t*>(dst) = u32x4_t{packed[0], packed[1], packed[2], packed[3]};
+      *reinterpret_cast<u32x4_t*>(dst + 8) = u32x4_t{packed[4], packed[5], packed[6], packed[7]};
+    } else {
+#pragma unroll
+      for (int c = 0; c < 16; ++c)
+        if (col0 + c < a.V) dst[c] = (bf16_bits)((packed[c >> 1] >> ((c & 1) * 16)) & 0xffffu);
+    }
+  }
+}
+
+// grad_bias, step 1: fp32 sums of 256-token blocks, tokens ascending. One thread per column pair.
+constexpr int kBiasBlockTokens = 256;
+
+__global__ void logp_bias_block_sums_kernel(const bf16_bits* __restrict__ dz, int64_t ld, float* __restrict__ part,
+                                            int T, int V) {
+  const int pair = blockIdx.x * blockDim.x + threadIdx.x;
+  const int col = pair * 2;
+  if (col >= V) return;
+  const int t0 = blockIdx.y * kBiasBlockTokens;
+  const int t1 = (t0 + kBiasBlockTokens < T) ? t0 + kBiasBlockTokens : T;
+  const bool two = col + 1 < V;
+  float s0 = 0.f, s1 = 0.f;
+  for (int t = t0; t < t1; ++t) {
+    const bf16_bits* row = dz + (int64_t)t * ld + col;
+    s0 = s0 + __uint_as_float((uint32_t)row[0] << 16);
+    if (two) s1 = s1 + __uint_as_float((uint32_t)row[1] << 16);
+  }
+  float* out = part + (int64_t)blockIdx.y * V + col;
+  out[0] = s0;
+  if (two) out[1] = s1;
+}
+
+// grad_bias, step 2: block sums added ascending.
+__global__ void logp_bias_merge_kernel(const float* __restrict__ part, float* __restrict__ grad_bias, int blocks,
+                                       int V) {
+  const int col = blockIdx.x * blockDim.x + threadIdx.x;
+  if (col >= V) return;
+  float s = 0.f;
+  for (int b = 0; b < blocks; ++b) s = s + part[(int64_t)b * V + col];
+  grad_bias[col] = s;
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+
+using LogpShape256 = TileShape<256, 256, 4, 2>;
+using LogpShape128 = TileShape<256, 128, 4, 2>;
+using LogpShape64 = TileShape<256, 64, 4, 2>;
+using LogpShape16 = TileShape<256, 16, 4, 1>;
+
+int64_t linear_logp_dz_row_stride(int V) { return ((int64_t)V + 63) / 64 * 64; }
+
+static size_t dz_bytes(int T, int V) {
+  // 256-byte multiple so the fp32 block sums behind it stay aligned
+  const size_t raw = (size_t)(T > 0 ? T : 0) * (size_t)linear_logp_dz_row_stride(V) * sizeof(bf16_bits);
+  return (raw + 255) / 256 * 256;
+}
+
+size_t linear_logp_bwd_workspace_bytes(int T, int V, bool with_bias) {
+  size_t bytes = dz_bytes(T, V);
+  if (with_bias && T > 0) bytes += (size_t)((T + kBiasBlockTokens - 1) / kBiasBlockTokens) * (size_t)V * sizeof(float);
+  return bytes;
+}
+
+template <class S, int LOOP>
+static hipError_t launch_dlogits(LogpBwdArgs a, hipStream_t stream) {
+  auto kernel = linear_logp_dlogits_kernel<S, LOOP>;
+  static bool configured[kMaxDevices] = {};
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev >= 0 && dev < kMaxDevices && !configured[dev]) {
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              S::kLdsBytes);
+    if (err != hipSuccess) return err;
+    configured[dev] = true;
+  }
+  a.tiles_m = (a.T + S::BM - 1) / S::BM;
+  a.tiles_v = (a.V + kLogpTileCols - 1) / kLogpTileCols;
+  a.group_m = a.tiles_m < 8 ? a.tiles_m : 8;
+  hipLaunchKernelGGL(kernel, dim3(a.tiles_m * a.tiles_v), dim3(S::kThreads), S::kLdsBytes, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t linear_logp_bwd_launch(const MatView& H, const MatView& W, const int64_t* target, const float* bias,
+                                  const float* temperature, const float* lse, const float* grad_logp,
+                                  const float* grad_lse, void* grad_hidden, int64_t gh_row_stride, void* grad_weight,
+                                  int64_t gw_row_stride, float* grad_bias, void* workspace, int T, int D, int V,
+                                  int64_t vocab_start, int vocab_limit, int config, hipStream_t stream) {
+  LogpBwdArgs a;
+  a.W = W;
+  a.H = H;
+  a.target = target;
+  a.bias = bias;
+  a.temperature = temperature;
+  a.lse = lse;
+  a.grad_logp = grad_logp;
+  a.grad_lse = grad_lse;
+  a.dz = reinterpret_cast<bf16_bits*>(workspace);
+  a.ld_dz = linear_logp_dz_row_stride(V);
+  a.T = T;
+  a.V = V;
+  a.D = D;
+  a.vocab_limit = vocab_limit;
+  a.vocab_start = vocab_start;
+  a.tiles_m = a.tiles_v = 0;
+  a.group_m = 1;
+
+  const bool vec = W.k_stride == 1 && H.k_stride == 1 && (W.row_stride % kChunkElems) == 0 &&
+                   (H.row_stride % kChunkElems) == 0 && (reinterpret_cast<uintptr_t>(W.ptr) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(H.ptr) & 15) == 0 && (D % kChunkElems) == 0;
+  const bool force_staged = (config & RLK_LOGP_CFG_FORCE_STAGED) != 0;
+  config &= ~RLK_LOGP_CFG_FORCE_STAGED;
+  if (config == RLK_LOGP_CFG_AUTO) config = pick_linear_logp_config(T, V);
+  if (!vec && config == RLK_LOGP_CFG_256) config = RLK_LOGP_CFG_128;
+  const int loop = !vec ? 0 : (D % kTileK == 0 && !force_staged) ? 2 : 1;
+  hipError_t err;
+  switch (config) {
+    case RLK_LOGP_CFG_256:
+      err = loop == 2 ? launch_dlogits<LogpShape256, 2>(a, stream) : launch_dlogits<LogpShape256, 1>(a, stream);
+      break;
+    case RLK_LOGP_CFG_128:
+      err = loop == 2   ? launch_dlogits<LogpShape128, 2>(a, stream)
+            : loop == 1 ? launch_dlogits<LogpShape128, 1>(a, stream)
+                        : launch_dlogits<LogpShape128, 0>(a, stream);
+      break;
+    case RLK_LOGP_CFG_64:
+      err = loop == 2   ? launch_dlogits<LogpShape64, 2>(a, stream)
+            : loop == 1 ? launch_dlogits<LogpShape64, 1>(a, stream)
+                        : launch_dlogits<LogpShape64, 0>(a, stream);
+      break;
+    case RLK_LOGP_CFG_16:
+      err = loop >= 1 ? launch_dlogits<LogpShape16, 1>(a, stream) : launch_dlogits<LogpShape16, 0>(a, stream);
+      break;
+    default:
+      return hipErrorInvalidValue;
+  }
+  if (err != hipSuccess) return err;
+
+  const int gemm_config = force_staged ? (RLK_GEMM_CFG_AUTO | RLK_GEMM_CFG_FORCE_STAGED) : RLK_GEMM_CFG_AUTO;
+  if (grad_hidden) {
+    // grad_hidden[t, d] = sum over v ascending of dz[t, v] * W[v, d]
+    const MatView w_by_feature{W.ptr, 1, W.row_stride, D};  // rows = d, reduction index = v
+    const MatView dz_by_token{a.dz, a.ld_dz, 1, T};
+    err = det_gemm_launch(w_by_feature, dz_by_token, grad_hidden, gh_row_stride, T, D, V, false, gemm_config, stream);
+    if (err != hipSuccess) return err;
+  }
+  if (grad_weight) {
+    // grad_weight[v, d] = sum over t ascending of dz[t, v] * H[t, d]
+    const MatView h_by_feature{H.ptr, 1, H.row_stride, D};  // rows = d, reduction index = t
+    const MatView dz_by_column{a.dz, 1, a.ld_dz, V};        // rows = v, reduction index = t
+    err = det_gemm_launch(h_by_feature, dz_by_column, grad_weight, gw_row_stride, V, D, T, false, gemm_config, stream);
+    if (err != hipSuccess) return err;
+  }
+  if (grad_bias) {
+    float* part = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + dz_bytes(T, V));
+    const int blocks = (T + kBiasBlockTokens - 1) / kBiasBlockTokens;
+    const int pairs = (V + 1) / 2;
+    hipLaunchKernelGGL(logp_bias_block_sums_kernel, dim3((pairs + 255) / 256, blocks), dim3(256), 0, stream, a.dz,
+                       a.ld_dz, part, T, V);
+    err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    hipLaunchKernelGGL(logp_bias_merge_kernel, dim3((V + 255) / 256), dim3(256), 0, stream, part, grad_bias, blocks, V);
+    err = hipGetLastError();
+  }
+  return err;
+}
+
+}  // namespace rlk

@@ -136,6 +136,59 @@ int rlk_linear_logp_fwd(const void* hidden, int64_t h_row_stride, const void* we
   return err == hipSuccess ? RLK_OK : device_error("rlk_linear_logp_fwd", err);
 }
 
+size_t rlk_linear_logp_bwd_workspace_bytes(int T, int V, int with_bias) {
+  if (T <= 0 || V <= 0) return 0;
+  return linear_logp_bwd_workspace_bytes(T, V, with_bias != 0);
+}
+
+int rlk_linear_logp_bwd(const void* hidden, int64_t h_row_stride, const void* weight, int64_t w_row_stride,
+                        const int64_t* target, const float* bias, const float* temperature, const float* lse,
+                        const float* grad_logp, const float* grad_lse, void* grad_hidden, int64_t gh_row_stride,
+                        void* grad_weight, int64_t gw_row_stride, float* grad_bias, void* workspace,
+                        size_t workspace_bytes, int T, int D, int V, int64_t vocab_start, int real_vocab_end,
+                        int config, void* stream) {
+  if (T < 0 || D <= 0 || V <= 0) {
+    set_last_error("rlk_linear_logp_bwd: bad sizes T=%d D=%d V=%d", T, D, V);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (real_vocab_end <= 0 || real_vocab_end > V) {
+    set_last_error("rlk_linear_logp_bwd: real_vocab_end must be in [1, %d], got %d", V, real_vocab_end);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (config < 0 || (config & ~RLK_LOGP_CFG_FORCE_STAGED) >= RLK_LOGP_CFG_COUNT) {
+    set_last_error("rlk_linear_logp_bwd: unknown config %d", config);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (hidden == nullptr || weight == nullptr || (T > 0 && (target == nullptr || lse == nullptr))) {
+    set_last_error("rlk_linear_logp_bwd: null hidden / weight / target / lse");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (h_row_stride < D || w_row_stride < D || (grad_hidden && gh_row_stride < D) || (grad_weight && gw_row_stride < D)) {
+    set_last_error("rlk_linear_logp_bwd: row strides must be >= D");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (T == 0) {
+    // No tokens: the token-summed gradients are zero.
+    hipError_t err = hipSuccess;
+    if (grad_weight) err = fill_zero_launch(grad_weight, V, D, gw_row_stride, 2, s);
+    if (err == hipSuccess && grad_bias) err = fill_zero_launch(grad_bias, 1, V, V, 4, s);
+    return err == hipSuccess ? RLK_OK : device_error("rlk_linear_logp_bwd", err);
+  }
+  const size_t need = linear_logp_bwd_workspace_bytes(T, V, grad_bias != nullptr);
+  if (workspace == nullptr || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0) {
+    set_last_error("rlk_linear_logp_bwd: 256-byte aligned workspace of %zu bytes needed, %zu given", need,
+                   workspace_bytes);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  MatView H{reinterpret_cast<const bf16_bits*>(hidden), h_row_stride, 1, T};
+  MatView W{reinterpret_cast<const bf16_bits*>(weight), w_row_stride, 1, V};
+  hipError_t err = linear_logp_bwd_launch(H, W, target, bias, temperature, lse, grad_logp, grad_lse, grad_hidden,
+                                          gh_row_stride, grad_weight, gw_row_stride, grad_bias, workspace, T, D, V,
+                                          vocab_start, real_vocab_end, config, s);
+  return err == hipSuccess ? RLK_OK : device_error("rlk_linear_logp_bwd", err);
+}
+
 size_t rlk_grpo_workspace_bytes(int rollouts) { return rollouts > 0 ? (size_t)3 * rollouts * sizeof(float) : 0; }
 
 int rlk_grpo_ratio_kl_loss(const float* logp, const float* old_logp, const float* ref_logp,

@@ -35,6 +35,17 @@ hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t*
                               const float* temperature, float* logp, float* lse, float* workspace, int T, int D,
                               int V, int64_t vocab_start, int vocab_limit, int config, hipStream_t stream);
 
+// Backward of the fused linear-LogP. workspace holds linear_logp_bwd_workspace_bytes() bytes
+// (the bf16 d(logits) with row stride linear_logp_dz_row_stride(V), then the bias block sums).
+// grad_hidden / grad_weight / grad_bias may each be null.
+int64_t linear_logp_dz_row_stride(int V);
+size_t linear_logp_bwd_workspace_bytes(int T, int V, bool with_bias);
+hipError_t linear_logp_bwd_launch(const MatView& H, const MatView& W, const int64_t* target, const float* bias,
+                                  const float* temperature, const float* lse, const float* grad_logp,
+                                  const float* grad_lse, void* grad_hidden, int64_t gh_row_stride, void* grad_weight,
+                                  int64_t gw_row_stride, float* grad_bias, void* workspace, int T, int D, int V,
+                                  int64_t vocab_start, int vocab_limit, int config, hipStream_t stream);
+
 // workspace: 3 * rollouts floats.
 hipError_t grpo_launch(const float* logp, const float* old_logp, const float* ref_logp, const float* advantages,
                        const uint8_t* mask, int rollouts, int tokens, float clip_eps, float beta, float* ratio,

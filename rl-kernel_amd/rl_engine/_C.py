@@ -286,6 +286,116 @@ def fused_linear_logp(
     return outputs
 
 
+def fused_linear_logp_bwd(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    target: torch.Tensor,
+    lse: torch.Tensor,
+    grad_logp: Optional[torch.Tensor],
+    grad_lse: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor] = None,
+    temperature: Optional[torch.Tensor] = None,
+    real_vocab_size: int = -1,
+    *,
+    vocab_start_index: int = 0,
+    need_grad_hidden: bool = True,
+    need_grad_weight: bool = True,
+    need_grad_bias: bool = False,
+    config: int = 0,
+) -> List[Optional[torch.Tensor]]:
+    """Backward of :func:`fused_linear_logp` -> ``[grad_hidden, grad_weight, grad_bias]``.
+
+    ``lse`` is the forward's result; ``grad_logp`` / ``grad_lse`` are fp32 ``[N]`` or
+    ``None``. ``grad_hidden`` / ``grad_weight`` are bf16, ``grad_bias`` fp32; an entry
+    that was not asked for is ``None``. Stands in for
+    ``_DetTritonLinearLogpAutograd.backward``
+    (rl_engine/backends/shared/triton/logprob/linear_logp.py:600-628) and
+    ``chunked_linear_logp_backward`` (rl_engine/reference/logprob/linear_logp.py:642-715).
+    """
+    if not hidden.is_cuda or not weight.is_cuda or not target.is_cuda or not lse.is_cuda:
+        raise RuntimeError("fused_linear_logp_bwd: hidden, weight, target and lse must be CUDA tensors")
+    if hidden.dtype != _BF16 or weight.dtype != _BF16:
+        raise RuntimeError("fused_linear_logp_bwd: hidden and weight must be bf16")
+    if hidden.dim() != 2 or weight.dim() != 2:
+        raise RuntimeError("fused_linear_logp_bwd: expect hidden [N,D] and weight [V,D]")
+    if not hidden.is_contiguous() or not weight.is_contiguous():
+        raise RuntimeError("fused_linear_logp_bwd: hidden and weight must be contiguous")
+    n, d = hidden.shape
+    v = weight.size(0)
+    if weight.size(1) != d:
+        raise RuntimeError("fused_linear_logp_bwd: hidden dim must match weight dim")
+    if target.numel() != n or lse.numel() != n:
+        raise RuntimeError("fused_linear_logp_bwd: target and lse must have one value per row")
+    real_vocab = v if int(real_vocab_size) < 0 else int(real_vocab_size)
+    if not 0 < real_vocab <= v:
+        raise RuntimeError(f"fused_linear_logp_bwd: real_vocab_size must be in [1, {v}]")
+
+    def _per_row(t: Optional[torch.Tensor], name: str) -> Optional[torch.Tensor]:
+        if t is None:
+            return None
+        if t.numel() != n:
+            raise RuntimeError(f"fused_linear_logp_bwd: {name} must have one value per row")
+        return t.reshape(-1).to(device=hidden.device, dtype=torch.float32).contiguous()
+
+    target_i64 = target.reshape(-1).to(torch.int64).contiguous()
+    lse_f32 = _per_row(lse, "lse")
+    g_logp = _per_row(grad_logp, "grad_logp")
+    g_lse = _per_row(grad_lse, "grad_lse")
+    temp_f32 = _per_row(temperature, "temperature")
+    bias_f32 = None
+    if bias is not None:
+        if bias.numel() != v:
+            raise RuntimeError("fused_linear_logp_bwd: bias must have V elements")
+        bias_f32 = bias.to(device=hidden.device, dtype=torch.float32).contiguous()
+
+    lib = _lib.load()
+    grad_hidden = torch.empty((n, d), dtype=_BF16, device=hidden.device) if need_grad_hidden else None
+    grad_weight = torch.empty((v, d), dtype=_BF16, device=hidden.device) if need_grad_weight else None
+    grad_bias = torch.empty((v,), dtype=torch.float32, device=hidden.device) if need_grad_bias else None
+    ws_bytes = int(lib.rlk_linear_logp_bwd_workspace_bytes(n, v, 1 if need_grad_bias else 0))
+    # torch's allocator hands out 512-byte aligned blocks, which covers the 256 the library asks for
+    workspace = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=hidden.device)
+
+    def _ptr(t: Optional[torch.Tensor]):
+        return t.data_ptr() if t is not None else None
+
+    if n == 0:  # no tokens: the token-summed gradients are zero
+        if grad_weight is not None:
+            grad_weight.zero_()
+        if grad_bias is not None:
+            grad_bias.zero_()
+        return [grad_hidden, grad_weight, grad_bias]
+    with torch.cuda.device(hidden.device):
+        status = lib.rlk_linear_logp_bwd(
+            hidden.data_ptr(),
+            hidden.stride(0),
+            weight.data_ptr(),
+            weight.stride(0),
+            target_i64.data_ptr(),
+            _ptr(bias_f32),
+            _ptr(temp_f32),
+            lse_f32.data_ptr(),
+            _ptr(g_logp),
+            _ptr(g_lse),
+            _ptr(grad_hidden),
+            d,
+            _ptr(grad_weight),
+            d,
+            _ptr(grad_bias),
+            workspace.data_ptr(),
+            ws_bytes,
+            n,
+            d,
+            v,
+            int(vocab_start_index),
+            real_vocab,
+            int(config),
+            _stream_handle(hidden.device),
+        )
+    _lib.check(status, "rlk_linear_logp_bwd failed")
+    return [grad_hidden, grad_weight, grad_bias]
+
+
 def grpo_ratio_kl_loss(
     logp: torch.Tensor,
     old_logp: torch.Tensor,

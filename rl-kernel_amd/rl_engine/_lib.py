@@ -49,6 +49,8 @@ EXPORTED_SYMBOLS = (
     "rlk_linear_logp_split_count",
     "rlk_linear_logp_workspace_bytes",
     "rlk_linear_logp_fwd",
+    "rlk_linear_logp_bwd_workspace_bytes",
+    "rlk_linear_logp_bwd",
     "rlk_grpo_workspace_bytes",
     "rlk_grpo_ratio_kl_loss",
 )
@@ -101,6 +103,13 @@ def load() -> ctypes.CDLL:
     lib.rlk_linear_logp_workspace_bytes.argtypes = [i32, i32]
     lib.rlk_linear_logp_fwd.restype = i32
     lib.rlk_linear_logp_fwd.argtypes = [vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, sz, i32, i32, i32, i64, i32, i32, vp]
+
+    lib.rlk_linear_logp_bwd_workspace_bytes.restype = sz
+    lib.rlk_linear_logp_bwd_workspace_bytes.argtypes = [i32, i32, i32]
+    lib.rlk_linear_logp_bwd.restype = i32
+    lib.rlk_linear_logp_bwd.argtypes = [
+        vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, vp, i64, vp, i64, vp, vp, sz, i32, i32, i32, i64, i32, i32, vp,
+    ]  # fmt: skip
 
     lib.rlk_grpo_workspace_bytes.restype = sz
     lib.rlk_grpo_workspace_bytes.argtypes = [i32]

@@ -63,6 +63,67 @@ def _requires_grad(*tensors: Optional[torch.Tensor]) -> bool:
     return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
 
 
+class _HipLinearLogpAutograd(torch.autograd.Function):
+    """Differentiable ``(logp, lse)``: forward and backward both on the HIP library.
+
+    Mirrors ``_DetTritonLinearLogpAutograd``
+    (rl_engine/backends/shared/triton/logprob/linear_logp.py:573-628): the backward
+    recomputes the logits from the saved ``lse`` and returns gradients in the dtypes
+    of ``hidden``, ``lm_head_weight`` and ``bias``; the clamp ``logp = min(., 0)`` is
+    not differentiated.
+    """
+
+    @staticmethod
+    def forward(ctx, hidden_2d, weight, bias, target_1d, temp_arg, real_vocab, vocab_start, config):
+        bias_c = bias.contiguous() if bias is not None else None
+        logp, lse = _C.fused_linear_logp(
+            hidden_2d, weight, target_1d, bias_c, temp_arg, False, real_vocab,
+            vocab_start_index=vocab_start, config=config,
+        )  # fmt: skip
+        ctx.save_for_backward(
+            hidden_2d,
+            weight,
+            bias_c if bias_c is not None else hidden_2d.new_empty(0),
+            target_1d,
+            lse,
+            temp_arg if temp_arg is not None else hidden_2d.new_empty(0),
+        )
+        ctx.has_bias = bias is not None
+        ctx.bias_dtype = bias.dtype if bias is not None else None
+        ctx.real_vocab = real_vocab
+        ctx.vocab_start = vocab_start
+        ctx.config = config
+        ctx.mark_non_differentiable(target_1d)
+        return logp, lse
+
+    @staticmethod
+    def backward(ctx, grad_logp, grad_lse):
+        if grad_logp is None and grad_lse is None:
+            return (None,) * 8
+        hidden_2d, weight, bias, target_1d, lse, temp = ctx.saved_tensors
+        need_h, need_w, need_b = ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.needs_input_grad[2]
+        with torch.no_grad():
+            grad_hidden, grad_weight, grad_bias = _C.fused_linear_logp_bwd(
+                hidden_2d,
+                weight,
+                target_1d,
+                lse,
+                grad_logp,
+                grad_lse,
+                bias if ctx.has_bias else None,
+                temp if temp.numel() else None,
+                ctx.real_vocab,
+                vocab_start_index=ctx.vocab_start,
+                need_grad_hidden=need_h,
+                need_grad_weight=need_w,
+                need_grad_bias=bool(ctx.has_bias and need_b),
+                config=ctx.config,
+            )
+        if grad_bias is not None:
+            grad_bias = grad_bias.to(ctx.bias_dtype)
+        return grad_hidden, grad_weight, grad_bias, None, None, None, None, None
+
+
 def hip_deterministic_linear_logp(
     hidden: torch.Tensor,
     lm_head_weight: torch.Tensor,
@@ -75,7 +136,8 @@ def hip_deterministic_linear_logp(
     vocab_start_index: int = 0,
     config: str | int = 0,
 ):
-    """Strict forward entry: returns fp32 ``(logp, lse)`` (plus logits on request).
+    """Strict entry: returns fp32 ``(logp, lse)`` (plus logits on request); differentiable
+    with respect to ``hidden``, ``lm_head_weight`` and ``bias``.
 
     Two callers with byte-identical ``hidden`` rows, ``lm_head_weight``,
     ``target_ids`` and ``temperature`` receive bitwise-identical results for a
@@ -95,13 +157,15 @@ def hip_deterministic_linear_logp(
                 f"target_ids must be in the real vocabulary [{lo}, {lo + real_vocab}), "
                 f"got [{int(target_1d.min().item())}, {int(target_1d.max().item())}]"
             )
-    if _requires_grad(hidden, lm_head_weight, bias):
-        raise RuntimeError(
-            "the gfx950 fused linear_logp is forward-only; call it under torch.no_grad() "
-            "(the backward of this op is not part of this build)"
-        )
     if isinstance(config, str):
         config = _lib.LOGP_CONFIGS[config]
+    if _requires_grad(hidden, lm_head_weight, bias):
+        if return_logits:
+            raise RuntimeError("return_logits=True is inference-only: call it under torch.no_grad()")
+        logp, lse = _HipLinearLogpAutograd.apply(
+            hidden_2d, weight, bias, target_1d, temp_arg, real_vocab, int(vocab_start_index), int(config)
+        )
+        return logp.reshape(lead_shape), lse.reshape(lead_shape)
     outputs = _C.fused_linear_logp(
         hidden_2d,
         weight,

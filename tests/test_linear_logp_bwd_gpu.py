@@ -1,0 +1,225 @@
+"""Backward of the fused linear-LogP on a real MI355X, through the C ABI.
+
+Parity bar: grad_hidden / grad_weight are bf16 results of a bf16 GEMM over d(logits)
+that were themselves rounded to bf16 once, so against the exact (fp64) gradient of the
+oracle every element must lie within
+    half a bf16 ulp of itself  +  (2^-8 + K 2^-24 + 2e-5) * sum_k |dz_k| |operand_k|
+(the second term: dz rounding, fp32 accumulation over K terms, fp32 exp / lse).
+grad_bias is fp32 and sums the bf16 dz: within 2^-8 * sum_t |dz| + fp32 accumulation.
+Determinism, batch invariance of grad_hidden rows and configuration neutrality are
+bit-exact."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+import inputs
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def logp_mod():
+    from rl_engine.ops import logprob
+
+    return logprob
+
+
+@pytest.fixture(scope="module")
+def native():
+    from rl_engine import _C
+
+    return _C
+
+
+def _bits16(x: torch.Tensor) -> torch.Tensor:
+    return x.contiguous().view(torch.int16)
+
+
+def _case(t, v, d, seed, *, bias=False, temperature=False, real=None):
+    h, w, target = inputs.logp_inputs(t, vocab=v, hidden=d, seed=seed, rms_norm=False)
+    w = (w.float() * 2.5).to(torch.bfloat16)
+    gen = torch.Generator().manual_seed(seed + 1)
+    real = v if real is None else real
+    target = target % real
+    out = {
+        "h": h,
+        "w": w,
+        "target": target,
+        "g_logp": torch.randn(t, generator=gen),
+        "g_lse": torch.randn(t, generator=gen) * 0.5,
+        "bias": torch.randn(v, generator=gen) * 0.3 if bias else None,
+        "temp": torch.rand(t, generator=gen) * 1.5 + 0.5 if temperature else None,
+        "real": real,
+    }
+    return out
+
+
+def _gpu_backward(native, c, *, config=0, need_bias=None, g_lse=True):
+    dev = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+    logp, lse = native.fused_linear_logp(dev["h"], dev["w"], dev["target"], dev["bias"], dev["temp"], False, c["real"])
+    need_bias = (c["bias"] is not None) if need_bias is None else need_bias
+    grads = native.fused_linear_logp_bwd(
+        dev["h"], dev["w"], dev["target"], lse, dev["g_logp"], dev["g_lse"] if g_lse else None, dev["bias"], dev["temp"],
+        c["real"], need_grad_bias=need_bias, config=config,
+    )  # fmt: skip
+    return lse, grads
+
+
+def _assert_grad_parity(oracle, c, lse, grads, *, g_lse=True):
+    gh, gw, gb = grads
+    hb, wb = inputs.bits(c["h"]), inputs.bits(c["w"])
+    args = dict(
+        grad_logp=c["g_logp"].numpy(),
+        grad_lse=c["g_lse"].numpy() if g_lse else None,
+        bias=None if c["bias"] is None else c["bias"].numpy(),
+        temperature=None if c["temp"] is None else c["temp"].numpy(),
+        real_vocab_size=c["real"],
+    )
+    lse64 = lse.double().cpu().numpy()
+    dz = oracle.linear_logp_dlogits(hb, wb, c["target"].numpy(), lse64, dtype=np.float64, **args)
+    hf = oracle.bf16_to_f32(hb).astype(np.float64)
+    wf = oracle.bf16_to_f32(wb).astype(np.float64)
+    t, v = dz.shape
+    slack = 2.0**-8 + 2e-5
+
+    def check(got_bits, exact, abs_sum, k, tag):
+        got = oracle.bf16_to_f32(got_bits).astype(np.float64)
+        bound = 2.0**-8 * np.abs(got) + (slack + k * 2.0**-24) * abs_sum + 1e-30
+        worst = float((np.abs(got - exact) / bound).max())
+        assert worst <= 1.0, f"{tag}: error is {worst:.3f}x the rounding + accumulation bound"
+
+    check(inputs.bits(gh), dz @ wf, np.abs(dz) @ np.abs(wf), v, "grad_hidden")
+    check(inputs.bits(gw), dz.T @ hf, np.abs(dz).T @ np.abs(hf), t, "grad_weight")
+    if gb is not None:
+        exact = dz.sum(axis=0)
+        bound = (slack + t * 2.0**-24) * np.abs(dz).sum(axis=0) + 1e-30
+        worst = float((np.abs(gb.double().cpu().numpy() - exact) / bound).max())
+        assert worst <= 1.0, f"grad_bias: error is {worst:.3f}x the bound"
+    # the reference's own bf16-dz formulation as a second, looser witness (its ws1 bf16 tolerance)
+    ref = oracle.linear_logp_backward(hb, wb, c["target"].numpy(), lse64, **args)
+    assert np.allclose(gh.double().cpu().numpy(), ref[0], atol=5e-2, rtol=2e-2)
+    assert np.allclose(gw.double().cpu().numpy(), ref[1], atol=5e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize(
+    "shape,opts",
+    [
+        ((64, 1024, 128), {}),
+        ((192, 2048, 256), dict(bias=True, temperature=True, real=1900)),
+        ((40, 3000, 264), dict(bias=True)),  # D % 64 != 0 and V % 64 != 0: staged / element loaders
+        ((130, 5000, 512), dict(temperature=True)),  # T % 64 != 0: weight gradient on the element loader
+        ((256, 4096, 320), dict(bias=True, temperature=True, real=4000)),
+    ],
+)
+def test_backward_parity_with_oracle(native, oracle, shape, opts):
+    t, v, d = shape
+    c = _case(t, v, d, 5100 + t, **opts)
+    lse, grads = _gpu_backward(native, c)
+    assert grads[0].dtype == torch.bfloat16 and tuple(grads[0].shape) == (t, d)
+    assert grads[1].dtype == torch.bfloat16 and tuple(grads[1].shape) == (v, d)
+    _assert_grad_parity(oracle, c, lse, grads)
+    if c["real"] < v:  # padded vocabulary rows get exactly zero
+        assert not bool(grads[1][c["real"] :].any())
+        assert not bool(grads[2][c["real"] :].any())
+
+
+def test_backward_is_bitwise_deterministic_and_config_neutral(native):
+    from rl_engine import _lib
+
+    c = _case(320, 3072, 256, 5200, bias=True, temperature=True, real=3000)
+    _, base = _gpu_backward(native, c)
+    for _ in range(3):
+        _, again = _gpu_backward(native, c)
+        for x, y in zip(base, again):
+            assert torch.equal(x.view(torch.uint8), y.view(torch.uint8))
+    for name, value in _lib.LOGP_CONFIGS.items():
+        for flag in (0, _lib.FORCE_STAGED):
+            _, other = _gpu_backward(native, c, config=value | flag)
+            for x, y in zip(base, other):
+                assert torch.equal(x.view(torch.uint8), y.view(torch.uint8)), (name, flag)
+
+
+def test_grad_hidden_rows_are_batch_invariant(native):
+    c = _case(384, 4096, 256, 5300, temperature=True)
+    _, (gh_full, _, _) = _gpu_backward(native, c)
+    for start, rows in ((0, 1), (37, 1), (100, 17), (128, 256), (383, 1)):
+        part = {k: (v[start : start + rows] if isinstance(v, torch.Tensor) and k in ("h", "target", "g_logp", "g_lse", "temp") else v) for k, v in c.items()}
+        _, (gh, _, _) = _gpu_backward(native, part)
+        assert torch.equal(_bits16(gh), _bits16(gh_full[start : start + rows])), (start, rows)
+
+
+def test_closed_forms_on_the_gpu(native):
+    # grad_lse only: d(logits) = softmax * g / T, so grad_bias sums to sum_t g_t / T_t
+    c = _case(128, 2048, 128, 5400, bias=True, temperature=True)
+    dev = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+    _, lse = native.fused_linear_logp(dev["h"], dev["w"], dev["target"], dev["bias"], dev["temp"], False, c["real"])
+    _, _, gb = native.fused_linear_logp_bwd(
+        dev["h"], dev["w"], dev["target"], lse, None, dev["g_lse"], dev["bias"], dev["temp"], c["real"], need_grad_bias=True
+    )
+    expect = float((c["g_lse"].double() / c["temp"].double()).sum())
+    assert abs(float(gb.double().sum()) - expect) < 2e-2 * float((c["g_lse"].abs().double() / c["temp"].double()).sum())
+    # zero upstream gradients give exactly zero everywhere
+    zero = torch.zeros(128, device=DEV)
+    gh, gw, gb = native.fused_linear_logp_bwd(
+        dev["h"], dev["w"], dev["target"], lse, zero, zero, dev["bias"], dev["temp"], c["real"], need_grad_bias=True
+    )
+    assert not bool(gh.any()) and not bool(gw.any()) and not bool(gb.any())
+    # identical weight rows: logp = -log V for any hidden, so grad_hidden of logp is ~0
+    same = dev["w"][:1].expand(2048, -1).contiguous()
+    _, lse_same = native.fused_linear_logp(dev["h"], same, dev["target"])
+    gh, _, _ = native.fused_linear_logp_bwd(dev["h"], same, dev["target"], lse_same, dev["g_logp"], None)
+    scale = float(dev["g_logp"].abs().max() * same.float().abs().max())
+    assert float(gh.float().abs().max()) <= 2.0**-7 * scale
+
+
+def test_autograd_entry_matches_the_native_backward(logp_mod, native):
+    c = _case(96, 2048, 128, 5500, bias=True, temperature=True, real=2000)
+    dev = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+    h = dev["h"].clone().requires_grad_(True)
+    w = dev["w"].clone().requires_grad_(True)
+    b = dev["bias"].clone().requires_grad_(True)
+    logp, lse = logp_mod.deterministic_linear_logp(
+        h.view(8, 12, 128), w, dev["target"].view(8, 12), b, temperature=dev["temp"], real_vocab_size=2000
+    )
+    assert logp.shape == (8, 12) and logp.requires_grad and lse.requires_grad
+    loss = (logp * dev["g_logp"].view(8, 12)).sum() + (lse * dev["g_lse"].view(8, 12)).sum()
+    loss.backward()
+    assert h.grad.dtype == torch.bfloat16 and h.grad.shape == h.shape
+    assert w.grad.dtype == torch.bfloat16 and b.grad.dtype == b.dtype
+    _, (gh, gw, gb) = _gpu_backward(native, c)
+    assert torch.equal(_bits16(h.grad), _bits16(gh))
+    assert torch.equal(_bits16(w.grad), _bits16(gw))
+    assert torch.equal(b.grad, gb)
+    # forward values under autograd are the inference values, bit for bit
+    with torch.no_grad():
+        logp2, lse2 = logp_mod.deterministic_linear_logp(
+            dev["h"], dev["w"], dev["target"], dev["bias"], temperature=dev["temp"], real_vocab_size=2000
+        )
+    assert torch.equal(logp.detach().reshape(-1).view(torch.int32), logp2.view(torch.int32))
+    # only hidden needs a gradient: the weight-sized outputs are skipped
+    h2 = dev["h"].clone().requires_grad_(True)
+    out, _ = logp_mod.deterministic_linear_logp(h2, dev["w"], dev["target"])
+    out.sum().backward()
+    assert h2.grad is not None and dev["w"].grad is None
+
+
+def test_backward_argument_errors(native):
+    c = _case(16, 256, 64, 5600)
+    dev = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+    _, lse = native.fused_linear_logp(dev["h"], dev["w"], dev["target"])
+    with pytest.raises(RuntimeError, match="must be bf16"):
+        native.fused_linear_logp_bwd(dev["h"].float(), dev["w"], dev["target"], lse, dev["g_logp"], None)
+    with pytest.raises(RuntimeError, match="one value per row"):
+        native.fused_linear_logp_bwd(dev["h"], dev["w"], dev["target"], lse[:3], dev["g_logp"], None)
+    with pytest.raises(RuntimeError, match="real_vocab_size"):
+        native.fused_linear_logp_bwd(dev["h"], dev["w"], dev["target"], lse, dev["g_logp"], None, None, None, 9999)
+    # empty batch: token-summed gradients are zero, grad_hidden is empty
+    empty = native.fused_linear_logp_bwd(
+        dev["h"][:0], dev["w"], dev["target"][:0], lse[:0], dev["g_logp"][:0], None, need_grad_bias=False
+    )
+    assert tuple(empty[0].shape) == (0, 64) and not bool(empty[1].any())

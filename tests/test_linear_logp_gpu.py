@@ -147,8 +147,8 @@ def test_uniform_logits_and_target_checks(logp_mod):
     with pytest.raises(ValueError, match="one id per hidden row"):
         logp_mod.deterministic_linear_logp(h, w, t[:3])
     hg = h.clone().requires_grad_(True)
-    with pytest.raises(RuntimeError, match="forward-only"):
-        logp_mod.deterministic_linear_logp(hg, w, t)
+    with pytest.raises(RuntimeError, match="inference-only"):
+        logp_mod.deterministic_linear_logp(hg, w, t, return_logits=True)
 
 
 def test_vocab_start_index_offsets_targets(logp_mod):

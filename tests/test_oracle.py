@@ -290,6 +290,123 @@ def test_logp_temperature_and_padding_follow_the_strict_contract(oracle):
 
 
 # ---------------------------------------------------------------------------
+# linear-LogP backward
+# ---------------------------------------------------------------------------
+
+
+def _objective(h, w, b, target, temp, real, g_logp, g_lse):
+    """sum_t g_logp[t] * logp[t] + g_lse[t] * lse[t] in fp64 from real-valued operands,
+    through scipy's logsumexp (an independent routine, not the oracle's formula)."""
+    from scipy.special import logsumexp
+
+    z = (h @ w.T + b) / temp[:, None]
+    z = z[:, :real]
+    lse = logsumexp(z, axis=-1)
+    logp = z[np.arange(h.shape[0]), target] - lse
+    return float((g_logp * logp + g_lse * lse).sum()), lse
+
+
+def test_logp_backward_matches_central_finite_differences(oracle):
+    rng = np.random.default_rng(21)
+    n, d, v, real = 3, 8, 12, 10
+    h_bits = oracle.randn_bf16(rng, (n, d))
+    w_bits = oracle.randn_bf16(rng, (v, d), 0.5)
+    bias = rng.standard_normal(v).astype(np.float32)
+    temp = np.array([0.5, 1.0, 1.75], np.float32)
+    target = np.array([0, 9, 4])
+    g_logp = rng.standard_normal(n).astype(np.float32)
+    g_lse = rng.standard_normal(n).astype(np.float32)
+    h = oracle.bf16_to_f32(h_bits).astype(np.float64)
+    w = oracle.bf16_to_f32(w_bits).astype(np.float64)
+    b = bias.astype(np.float64)
+    t64, gl, gs = temp.astype(np.float64), g_logp.astype(np.float64), g_lse.astype(np.float64)
+    _, lse = _objective(h, w, b, target, t64, real, gl, gs)
+    dz = oracle.linear_logp_dlogits(
+        h_bits, w_bits, target, lse, g_logp, g_lse, bias, temperature=temp, real_vocab_size=real, dtype=np.float64
+    )
+    grad_h, grad_w, grad_b = dz @ w, dz.T @ h, dz.sum(axis=0)
+    eps = 1e-6
+
+    def fd(arr, index):
+        saved = arr[index]
+        arr[index] = saved + eps
+        up, _ = _objective(h, w, b, target, t64, real, gl, gs)
+        arr[index] = saved - eps
+        down, _ = _objective(h, w, b, target, t64, real, gl, gs)
+        arr[index] = saved
+        return (up - down) / (2 * eps)
+
+    for i in range(n):
+        for j in range(d):
+            assert abs(fd(h, (i, j)) - grad_h[i, j]) < 1e-7, ("hidden", i, j)
+    for i in range(v):
+        for j in range(d):
+            assert abs(fd(w, (i, j)) - grad_w[i, j]) < 1e-7, ("weight", i, j)
+        assert abs(fd(b, i) - grad_b[i]) < 1e-7, ("bias", i)
+    # padded vocabulary rows receive no gradient at all
+    assert np.all(grad_w[real:] == 0) and np.all(grad_b[real:] == 0)
+    # the fp32 restatement and the packaged backward agree with the fp64 anchor
+    gh32, gw32, gb32, dz32 = oracle.linear_logp_backward(
+        h_bits, w_bits, target, lse, g_logp, g_lse, bias, temperature=temp, real_vocab_size=real,
+        round_dlogits_to_bf16=False,
+    )  # fmt: skip
+    assert np.abs(dz32 - dz).max() < 1e-5
+    assert np.abs(gh32 - grad_h).max() < 1e-4 and np.abs(gw32 - grad_w).max() < 1e-4 and np.abs(gb32 - grad_b).max() < 1e-4
+
+
+def test_logp_backward_closed_forms(oracle):
+    rng = np.random.default_rng(22)
+    n, d, v = 5, 16, 64
+    h_bits = oracle.randn_bf16(rng, (n, d))
+    w_bits = oracle.randn_bf16(rng, (v, d), 0.3)
+    target = rng.integers(0, v, n)
+    temp = np.array([0.5, 1.0, 2.0, 0.7, 1.3], np.float32)
+    g_logp = rng.standard_normal(n).astype(np.float32)
+    g_lse = rng.standard_normal(n).astype(np.float32)
+    _, lse = oracle.linear_logp_f64(h_bits, w_bits, target, temperature=temp)
+    dz = oracle.linear_logp_dlogits(h_bits, w_bits, target, lse, g_logp, g_lse, temperature=temp, dtype=np.float64)
+    # probabilities sum to one: a row of d(logits) sums to grad_lse / temperature
+    assert np.allclose(dz.sum(axis=-1), g_lse.astype(np.float64) / temp.astype(np.float64), atol=1e-12)
+    # grad_logp only: the target column gets g * (1 - p_t) / T, every other column -g * p / T
+    dz_lp = oracle.linear_logp_dlogits(h_bits, w_bits, target, lse, g_logp, None, temperature=temp, dtype=np.float64)
+    rows = np.arange(n)
+    assert np.all(np.sign(dz_lp[rows, target]) == np.sign(g_logp))
+    others = dz_lp.copy()
+    others[rows, target] = 0
+    assert np.all(others * g_logp[:, None] <= 0)
+    # identical weight rows: logits are constant per token, so logp = -log V whatever hidden is
+    same = np.repeat(w_bits[:1], v, axis=0)
+    lse_same = oracle.linear_logp_f64(h_bits, same, target)[1]
+    gh, gw, gb, _ = oracle.linear_logp_backward(h_bits, same, target, lse_same, g_logp, None, round_dlogits_to_bf16=False)
+    assert np.abs(gh).max() < 1e-5
+    # ... and the weight gradient of row v is (onehot - 1/V) g h summed over tokens
+    hf = oracle.bf16_to_f32(h_bits).astype(np.float64)
+    expect = -(g_logp[:, None] * hf).sum(axis=0) / v
+    expect_rows = np.tile(expect, (v, 1))
+    for t in range(n):
+        expect_rows[target[t]] += g_logp[t] * hf[t]
+    assert np.abs(gw - expect_rows).max() < 1e-5
+
+
+def test_logp_backward_bf16_dlogits_stay_within_their_rounding(oracle):
+    rng = np.random.default_rng(23)
+    n, d, v = 8, 32, 256
+    h_bits = oracle.randn_bf16(rng, (n, d))
+    w_bits = oracle.randn_bf16(rng, (v, d), 0.3)
+    target = rng.integers(0, v, n)
+    g = rng.standard_normal(n).astype(np.float32)
+    lse = oracle.linear_logp_f64(h_bits, w_bits, target)[1]
+    exact = oracle.linear_logp_backward(h_bits, w_bits, target, lse, g, None, round_dlogits_to_bf16=False)
+    rounded = oracle.linear_logp_backward(h_bits, w_bits, target, lse, g, None, round_dlogits_to_bf16=True)
+    dz = np.abs(exact[3].astype(np.float64))
+    w = np.abs(oracle.bf16_to_f32(w_bits).astype(np.float64))
+    h = np.abs(oracle.bf16_to_f32(h_bits).astype(np.float64))
+    assert np.all(np.abs(rounded[0] - exact[0]) <= 2.0**-8 * (dz @ w) + 1e-12)
+    assert np.all(np.abs(rounded[1] - exact[1]) <= 2.0**-8 * (dz.T @ h) + 1e-12)
+    assert np.array_equal(rounded[2], exact[2])  # the bias gradient sums the unrounded values
+
+
+# ---------------------------------------------------------------------------
 # GRPO
 # ---------------------------------------------------------------------------
 
