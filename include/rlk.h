@@ -174,6 +174,62 @@ int rlk_linear_logp_bwd(const void* hidden, int64_t h_row_stride, const void* we
                         size_t workspace_bytes, int T, int D, int V, int64_t vocab_start, int real_vocab_end,
                         int config, void* stream);
 
+/* Element types of materialised logits. */
+typedef enum rlk_dtype { RLK_DTYPE_BF16 = 0, RLK_DTYPE_FP16 = 1, RLK_DTYPE_FP32 = 2 } rlk_dtype;
+
+/*
+ * Per-row, per-tile statistics of materialised logits [T, V] (row stride in elements):
+ * tile t covers columns [t * V / num_tiles, (t + 1) * V / num_tiles), cut at the real
+ * vocabulary (global column vocab_start + c counts only while it is < real_vocab).
+ *   tile_max [T, num_tiles] fp32: max of the tile (-inf for an all-padding tile)
+ *   tile_sum [T, num_tiles] fp32: sum of exp(z - tile_max) (0 when tile_max is not finite)
+ * temperature [T] fp32 or NULL scales the logits by 1 / temperature in registers first
+ * (the scaling of rlk_linear_logp_fwd). V % num_tiles == 0.
+ * A row's result depends on that row only.
+ *
+ * Stands in for rl_engine._C.hip_deterministic_logp_tile_stats
+ * (csrc/bindings/ops.cpp:122-126; csrc/rocm/logprob/hip_deterministic_logp_kernel.hip:389-467, 550-588).
+ */
+int rlk_logits_tile_stats(const void* logits, int dtype, int64_t row_stride, const float* temperature, int T,
+                          int64_t V, int64_t vocab_start, int64_t real_vocab, int num_tiles, float* tile_max,
+                          float* tile_sum, void* stream);
+
+/* Bytes of workspace rlk_logp_from_logits needs. */
+size_t rlk_logp_from_logits_workspace_bytes(int T, int num_tiles);
+
+/*
+ * Selected-token log-probabilities from materialised logits, without another GEMM:
+ * tile statistics as above, tiles merged ascending (M = max_t m_t,
+ * S = sum_t s_t * exp(m_t - M), lse = M + log S), target logit gathered in fp32,
+ * logp = target * (1 / temperature) - lse. target holds GLOBAL ids; one outside
+ * [vocab_start, vocab_start + V) or in the padding contributes a target logit of 0.
+ *
+ * Stands in for the ROCm branch of LinearLogpWrapper.from_local_logits
+ * (rl_engine/integrations/common/linear_logp.py:750-815, 817-923), i.e.
+ * _RocmVocabParallelLogprobFunction.forward + _merge_tile_partials
+ * (rl_engine/backends/rocm/logprob/vocab_parallel_logp.py:308-352;
+ * rl_engine/reference/logprob/vocab_parallel_logp.py:355-363) on one GPU.
+ */
+int rlk_logp_from_logits(const void* logits, int dtype, int64_t row_stride, const int64_t* target,
+                         const float* temperature, int T, int64_t V, int64_t vocab_start, int64_t real_vocab,
+                         int num_tiles, float* logp, float* lse, void* workspace, size_t workspace_bytes,
+                         void* stream);
+
+/*
+ * d(logits) for logp / lse computed from materialised logits, in the dtype of the logits:
+ *   grad[c] = coef_logp * ([c == target_local] - p_c) + coef_lse * p_c,  p_c = exp(y_c - lse)
+ * with y = z * (1 / temperature) (and the result scaled by it once more), 0 on
+ * padded columns, p = 0 on a row whose lse is not finite. coef_lse and temperature may be
+ * NULL; target_local is the LOCAL column or -1.
+ *
+ * Stands in for rl_engine._C.hip_deterministic_logp_backward
+ * (csrc/bindings/ops.cpp:127-135; hip_deterministic_logp_kernel.hip:472-540, 590-640).
+ */
+int rlk_logits_logp_backward(const void* logits, int dtype, int64_t row_stride, const float* lse,
+                             const float* coef_logp, const float* coef_lse, const int64_t* target_local,
+                             const float* temperature, void* grad, int64_t grad_row_stride, int T, int64_t V,
+                             int64_t vocab_start, int64_t real_vocab, void* stream);
+
 /* Bytes of workspace rlk_grpo_ratio_kl_loss needs. */
 size_t rlk_grpo_workspace_bytes(int rollouts);
 

@@ -29,6 +29,10 @@ Pinning (which check fixes which function; see tests/test_oracle.py):
 * ``linear_logp_dlogits`` / ``linear_logp_backward``: central finite differences of
   ``linear_logp_f64`` in hidden, weight and bias; rows of d(logits) summing to
   ``grad_lse / temperature``; zero hidden gradient when every weight row is the same.
+* ``logits_tile_stats`` / ``merge_tile_partials`` / ``logp_from_logits`` /
+  ``logits_logp_backward``: scipy's logsumexp on the real columns, tile-count
+  independence of the merged lse, the all-padding tile identity, central finite
+  differences of logsumexp and the gathered logit.
 * ``grpo_ratio_kl_loss`` / ``group_advantages`` / ``masked_mean``: the reference's
   hand examples (tests/reference/test_reference_ops.py:77-98,
   tests/ops/loss/test_grpo_loss.py:112-119) and closed forms (old == logp gives
@@ -413,6 +417,107 @@ def linear_logp_backward(
     grad_weight = used.T @ h
     grad_bias = dz.astype(np.float64).sum(axis=0)
     return grad_hidden, grad_weight, grad_bias, dz
+
+
+# ---------------------------------------------------------------------------
+# log-probabilities from materialised logits (the stage that reuses LM-head logits)
+# ---------------------------------------------------------------------------
+
+
+def logits_tile_stats(logits, vocab_start: int, real_vocab: int, num_tiles: int, *, temperature=None):
+    """Per-row, per-tile ``(max, sum of exp(z - max))`` over the real-vocabulary part of a tile.
+
+    Restates hip_tile_stats_kernel
+    (csrc/rocm/logprob/hip_deterministic_logp_kernel.hip:389-467): tile ``t`` covers
+    columns ``[t * V / tiles, (t + 1) * V / tiles)`` cut at ``real_vocab - vocab_start``;
+    an all-padding tile reports ``(-inf, 0)``. ``logits`` is a float array (already
+    upcast); ``temperature`` divides it first, as the wrapper does
+    (rl_engine/integrations/common/linear_logp.py:777-785). fp32 throughout.
+    """
+    z = np.asarray(logits, dtype=np.float32)
+    rows, v = z.shape
+    if v % num_tiles:
+        raise ValueError("local_vocab must be divisible by num_tiles")
+    if temperature is not None:
+        z = (z / np.broadcast_to(np.asarray(temperature, dtype=np.float32), (rows,))[:, None]).astype(np.float32)
+    tile = v // num_tiles
+    real_cols = max(int(real_vocab) - int(vocab_start), 0)
+    tile_max = np.full((rows, num_tiles), -np.inf, dtype=np.float32)
+    tile_sum = np.zeros((rows, num_tiles), dtype=np.float32)
+    for t in range(num_tiles):
+        lo, hi = t * tile, min((t + 1) * tile, real_cols)
+        if hi <= lo:
+            continue
+        part = z[:, lo:hi]
+        m = part.max(axis=1)
+        tile_max[:, t] = m
+        with np.errstate(invalid="ignore"):
+            s = np.exp(part - m[:, None]).sum(axis=1, dtype=np.float32)
+        tile_sum[:, t] = np.where(np.isfinite(m), s, 0.0)
+    return tile_max, tile_sum
+
+
+def merge_tile_partials(m_all, s_all):
+    """``lse = M + log(sum_t s_t * exp(m_t - M))`` with ``M = max_t m_t``.
+
+    _merge_tile_partials, rl_engine/reference/logprob/vocab_parallel_logp.py:355-363.
+    """
+    m_all = np.asarray(m_all, dtype=np.float32)
+    s_all = np.asarray(s_all, dtype=np.float32)
+    big = m_all.max(axis=1)
+    safe = np.where(big > -np.inf, big, 0.0).astype(np.float32)
+    with np.errstate(divide="ignore"):
+        terms = s_all * np.exp(m_all - safe[:, None])
+        return (big + np.log(terms.sum(axis=1, dtype=np.float32))).astype(np.float32)
+
+
+def logp_from_logits(logits, target, vocab_start: int, real_vocab: int, num_tiles: int, *, temperature=None):
+    """``(logp, lse)`` of materialised logits: tile statistics, merge, target gather
+    (_RocmVocabParallelLogprobFunction.forward,
+    rl_engine/backends/rocm/logprob/vocab_parallel_logp.py:311-352, single rank)."""
+    z = np.asarray(logits, dtype=np.float32)
+    rows = z.shape[0]
+    m_all, s_all = logits_tile_stats(z, vocab_start, real_vocab, num_tiles, temperature=temperature)
+    lse = merge_tile_partials(m_all, s_all)
+    local = np.asarray(target, dtype=np.int64).reshape(-1) - int(vocab_start)
+    zt = z[np.arange(rows), np.clip(local, 0, z.shape[1] - 1)]
+    if temperature is not None:
+        zt = (zt / np.broadcast_to(np.asarray(temperature, dtype=np.float32), (rows,))).astype(np.float32)
+    owned = (local >= 0) & (local < min(z.shape[1], max(int(real_vocab) - int(vocab_start), 0)))
+    zt = np.where(owned, zt, np.float32(0.0)).astype(np.float32)
+    return (zt - lse).astype(np.float32), lse
+
+
+def logits_logp_backward(
+    logits, lse, coef_logp, coef_lse, target_local, vocab_start: int, real_vocab: int, *, temperature=None,
+    dtype=np.float32,
+):  # fmt: skip
+    """``grad = coef_logp * (onehot - p) + coef_lse * p`` with ``p = exp(z - lse)`` on finite
+    rows, 0 on padded columns (hip_backward_kernel,
+    csrc/rocm/logprob/hip_deterministic_logp_kernel.hip:472-540). With a temperature the
+    logits are divided by it first and the gradient once more (chain rule)."""
+    z = np.asarray(logits, dtype=dtype)
+    rows, v = z.shape
+    temp = None
+    if temperature is not None:
+        temp = np.broadcast_to(np.asarray(temperature, dtype=np.float32), (rows,)).astype(dtype)
+        z = z / temp[:, None]
+    lse = np.asarray(lse, dtype=dtype).reshape(-1)
+    finite = np.isfinite(lse)
+    with np.errstate(over="ignore", invalid="ignore"):
+        p = np.where(finite[:, None], np.exp(z - np.where(finite, lse, 0.0)[:, None]), 0.0)
+    g_logp = np.asarray(coef_logp, dtype=dtype).reshape(-1)
+    g_lse = np.zeros((rows,), dtype=dtype) if coef_lse is None else np.asarray(coef_lse, dtype=dtype).reshape(-1)
+    onehot = np.zeros((rows, v), dtype=dtype)
+    hit = np.asarray(target_local, dtype=np.int64).reshape(-1)
+    ok = hit >= 0
+    onehot[np.arange(rows)[ok], hit[ok]] = 1.0
+    grad = g_logp[:, None] * (onehot - p) + g_lse[:, None] * p
+    real_end = min(v, max(int(real_vocab) - int(vocab_start), 0))
+    grad[:, real_end:] = 0.0
+    if temp is not None:
+        grad = grad / temp[:, None]
+    return grad.astype(dtype)
 
 
 # ---------------------------------------------------------------------------

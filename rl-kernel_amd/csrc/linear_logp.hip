@@ -170,23 +170,81 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_partial_kernel(LogpAr
   }
 }
 
-__global__ void linear_logp_merge_kernel(const float* __restrict__ part, float* __restrict__ logp,
-                                         float* __restrict__ lse, int T, int n_split) {
-  const int m = blockIdx.x * blockDim.x + threadIdx.x;
-  if (m >= T) return;
+// Final merge over splits. 16 tokens per workgroup, 16 threads per token: the maximum and
+// the rescaled terms s_p * e(m_p - M) are computed by all threads (neither depends on an
+// order), then one thread per token adds the terms of a chunk in ascending split order,
+// chunk after chunk. The target logit has a single non-zero contribution, so its sum is
+// exact in any order.
+constexpr int kMergeTokens = 16;
+constexpr int kMergeLanes = 16;                           // threads per token
+constexpr int kMergeChunk = 8 * kMergeLanes;              // splits staged per round
+constexpr int kMergeThreads = kMergeTokens * kMergeLanes;  // 256
+
+__global__ __launch_bounds__(kMergeThreads) void linear_logp_merge_kernel(const float* __restrict__ part,
+                                                                          float* __restrict__ logp,
+                                                                          float* __restrict__ lse, int T,
+                                                                          int n_split, bool clamp) {
+  __shared__ float red[kMergeLanes][kMergeTokens];
+  __shared__ float terms[kMergeChunk][kMergeTokens];
+  const int tk = threadIdx.x % kMergeTokens;
+  const int sp = threadIdx.x / kMergeTokens;
+  const int m = blockIdx.x * kMergeTokens + tk;
+  const bool live = m < T;
   const int64_t plane = (int64_t)n_split * T;
-  float big = kNegInf;
-  for (int p = 0; p < n_split; ++p) big = fmaxf(big, part[(int64_t)p * T + m]);
-  float sum = 0.f, zt = 0.f;
-  for (int p = 0; p < n_split; ++p) {
-    const float pm = part[(int64_t)p * T + m];
-    const float term = part[plane + (int64_t)p * T + m] * pinned_exp(pm - big);
-    sum = sum + ((pm > kNegInf) ? term : 0.f);
-    zt = zt + part[2 * plane + (int64_t)p * T + m];
+
+  float big = kNegInf, zt = 0.f;
+  if (live) {
+    for (int p = sp; p < n_split; p += kMergeLanes) {
+      big = fmaxf(big, part[(int64_t)p * T + m]);
+      zt = zt + part[2 * plane + (int64_t)p * T + m];
+    }
   }
-  const float l = big + logf(sum);
-  if (lse) lse[m] = l;
-  if (logp) logp[m] = fminf(zt - l, 0.f);
+  red[sp][tk] = big;
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kMergeLanes; ++j) big = fmaxf(big, red[j][tk]);
+  __syncthreads();
+  red[sp][tk] = zt;
+  __syncthreads();
+  if (sp == 0) {
+    zt = 0.f;
+#pragma unroll
+    for (int j = 0; j < kMergeLanes; ++j) zt = zt + red[j][tk];
+  }
+
+  float sum = 0.f;
+  for (int c0 = 0; c0 < n_split; c0 += kMergeChunk) {
+#pragma unroll
+    for (int i = 0; i < kMergeChunk / kMergeLanes; ++i) {
+      const int local = i * kMergeLanes + sp;
+      const int p = c0 + local;
+      float term = 0.f;
+      if (live && p < n_split) {
+        const float pm = part[(int64_t)p * T + m];
+        const float scaled = part[plane + (int64_t)p * T + m] * pinned_exp(pm - big);
+        term = (pm > kNegInf) ? scaled : 0.f;
+      }
+      terms[local][tk] = term;
+    }
+    __syncthreads();
+    if (sp == 0) {
+      const int count = (n_split - c0) < kMergeChunk ? (n_split - c0) : kMergeChunk;
+      for (int j = 0; j < count; ++j) sum = sum + terms[j][tk];
+    }
+    __syncthreads();
+  }
+  if (sp == 0 && live) {
+    const float l = big + logf(sum);
+    if (lse) lse[m] = l;
+    if (logp) logp[m] = clamp ? fminf(zt - l, 0.f) : zt - l;
+  }
+}
+
+hipError_t linear_logp_merge_launch(const float* part, float* logp, float* lse, int T, int n_split, bool clamp,
+                                    hipStream_t stream) {
+  hipLaunchKernelGGL(linear_logp_merge_kernel, dim3((T + kMergeTokens - 1) / kMergeTokens), dim3(kMergeThreads), 0,
+                     stream, part, logp, lse, T, n_split, clamp);
+  return hipGetLastError();
 }
 
 // ---------------------------------------------------------------------------
@@ -281,9 +339,7 @@ hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t*
       return hipErrorInvalidValue;
   }
   if (err != hipSuccess) return err;
-  hipLaunchKernelGGL(linear_logp_merge_kernel, dim3((T + 255) / 256), dim3(256), 0, stream, workspace, logp, lse, T,
-                     a.n_split);
-  return hipGetLastError();
+  return linear_logp_merge_launch(workspace, logp, lse, T, a.n_split, true, stream);
 }
 
 }  // namespace rlk

@@ -189,6 +189,98 @@ int rlk_linear_logp_bwd(const void* hidden, int64_t h_row_stride, const void* we
   return err == hipSuccess ? RLK_OK : device_error("rlk_linear_logp_bwd", err);
 }
 
+static int check_logits_args(const char* what, const void* logits, int dtype, int64_t row_stride, int T, int64_t V,
+                             int64_t vocab_start, int64_t real_vocab) {
+  if (T < 0 || V <= 0 || V > 0x7fffffff) {
+    set_last_error("%s: bad sizes T=%d V=%lld", what, T, (long long)V);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (dtype != RLK_DTYPE_BF16 && dtype != RLK_DTYPE_FP16 && dtype != RLK_DTYPE_FP32) {
+    set_last_error("%s: logits must be float16, bfloat16, or float32", what);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (vocab_start < 0 || real_vocab <= 0) {
+    set_last_error("%s: invalid vocabulary metadata", what);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (T > 0 && (logits == nullptr || row_stride < V)) {
+    set_last_error("%s: null logits or row stride < V", what);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  return RLK_OK;
+}
+
+int rlk_logits_tile_stats(const void* logits, int dtype, int64_t row_stride, const float* temperature, int T,
+                          int64_t V, int64_t vocab_start, int64_t real_vocab, int num_tiles, float* tile_max,
+                          float* tile_sum, void* stream) {
+  int rc = check_logits_args("rlk_logits_tile_stats", logits, dtype, row_stride, T, V, vocab_start, real_vocab);
+  if (rc != RLK_OK) return rc;
+  if (num_tiles <= 0 || num_tiles > 65535 || V % num_tiles != 0) {
+    set_last_error("rlk_logits_tile_stats: local_vocab must be divisible by num_tiles (1..65535)");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (T == 0) return RLK_OK;
+  if (tile_max == nullptr || tile_sum == nullptr) {
+    set_last_error("rlk_logits_tile_stats: null output");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  hipError_t err = logits_tile_stats_launch(logits, dtype, row_stride, nullptr, temperature, T, V, vocab_start,
+                                            real_vocab, num_tiles, tile_max, tile_sum, nullptr, num_tiles, 1,
+                                            reinterpret_cast<hipStream_t>(stream));
+  return err == hipSuccess ? RLK_OK : device_error("rlk_logits_tile_stats", err);
+}
+
+size_t rlk_logp_from_logits_workspace_bytes(int T, int num_tiles) {
+  if (T <= 0 || num_tiles <= 0) return 0;
+  return (size_t)3 * (size_t)num_tiles * (size_t)T * sizeof(float);
+}
+
+int rlk_logp_from_logits(const void* logits, int dtype, int64_t row_stride, const int64_t* target,
+                         const float* temperature, int T, int64_t V, int64_t vocab_start, int64_t real_vocab,
+                         int num_tiles, float* logp, float* lse, void* workspace, size_t workspace_bytes,
+                         void* stream) {
+  int rc = check_logits_args("rlk_logp_from_logits", logits, dtype, row_stride, T, V, vocab_start, real_vocab);
+  if (rc != RLK_OK) return rc;
+  if (num_tiles <= 0 || num_tiles > 65535 || V % num_tiles != 0) {
+    set_last_error("rlk_logp_from_logits: local_vocab must be divisible by num_tiles (1..65535)");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (T == 0) return RLK_OK;
+  if (target == nullptr) {
+    set_last_error("rlk_logp_from_logits: null target");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  const size_t need = rlk_logp_from_logits_workspace_bytes(T, num_tiles);
+  if (workspace == nullptr || workspace_bytes < need) {
+    set_last_error("rlk_logp_from_logits: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  float* part = reinterpret_cast<float*>(workspace);
+  const int64_t plane = (int64_t)num_tiles * T;
+  hipError_t err = logits_tile_stats_launch(logits, dtype, row_stride, target, temperature, T, V, vocab_start,
+                                            real_vocab, num_tiles, part, part + plane, part + 2 * plane, 1, T, s);
+  if (err == hipSuccess) err = linear_logp_merge_launch(part, logp, lse, T, num_tiles, false, s);
+  return err == hipSuccess ? RLK_OK : device_error("rlk_logp_from_logits", err);
+}
+
+int rlk_logits_logp_backward(const void* logits, int dtype, int64_t row_stride, const float* lse,
+                             const float* coef_logp, const float* coef_lse, const int64_t* target_local,
+                             const float* temperature, void* grad, int64_t grad_row_stride, int T, int64_t V,
+                             int64_t vocab_start, int64_t real_vocab, void* stream) {
+  int rc = check_logits_args("rlk_logits_logp_backward", logits, dtype, row_stride, T, V, vocab_start, real_vocab);
+  if (rc != RLK_OK) return rc;
+  if (T == 0) return RLK_OK;
+  if (lse == nullptr || coef_logp == nullptr || target_local == nullptr || grad == nullptr || grad_row_stride < V) {
+    set_last_error("rlk_logits_logp_backward: null lse / coef_logp / target_local / grad, or grad row stride < V");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  hipError_t err = logits_backward_launch(logits, dtype, row_stride, lse, coef_logp, coef_lse, target_local,
+                                          temperature, grad, grad_row_stride, T, V, vocab_start, real_vocab,
+                                          reinterpret_cast<hipStream_t>(stream));
+  return err == hipSuccess ? RLK_OK : device_error("rlk_logits_logp_backward", err);
+}
+
 size_t rlk_grpo_workspace_bytes(int rollouts) { return rollouts > 0 ? (size_t)3 * rollouts * sizeof(float) : 0; }
 
 int rlk_grpo_ratio_kl_loss(const float* logp, const float* old_logp, const float* ref_logp,

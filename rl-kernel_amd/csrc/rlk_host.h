@@ -35,6 +35,26 @@ hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t*
                               const float* temperature, float* logp, float* lse, float* workspace, int T, int D,
                               int V, int64_t vocab_start, int vocab_limit, int config, hipStream_t stream);
 
+// Ascending merge of (max, sum, target logit) partials laid out [3][n_split][T] into
+// lse = M + log(S) and logp = target - lse (clamped at 0 when `clamp`).
+hipError_t linear_logp_merge_launch(const float* part, float* logp, float* lse, int T, int n_split, bool clamp,
+                                    hipStream_t stream);
+
+// Per-row, per-tile (max, sum of exp relative to it[, target logit]) of materialised logits
+// of element type `dtype` (rlk_dtype); element (row, tile) of each output sits at
+// out[row * out_row_stride + tile * out_tile_stride]. V % num_tiles == 0.
+hipError_t logits_tile_stats_launch(const void* logits, int dtype, int64_t row_stride, const int64_t* target,
+                                    const float* temperature, int T, int64_t V, int64_t vocab_start,
+                                    int64_t real_vocab, int num_tiles, float* out_max, float* out_sum,
+                                    float* out_target, int64_t out_row_stride, int64_t out_tile_stride,
+                                    hipStream_t stream);
+
+// d(logits) of logp / lse computed from materialised logits, in the dtype of the logits.
+hipError_t logits_backward_launch(const void* logits, int dtype, int64_t row_stride, const float* lse,
+                                  const float* coef_logp, const float* coef_lse, const int64_t* target_local,
+                                  const float* temperature, void* grad, int64_t grad_row_stride, int T, int64_t V,
+                                  int64_t vocab_start, int64_t real_vocab, hipStream_t stream);
+
 // Backward of the fused linear-LogP. workspace holds linear_logp_bwd_workspace_bytes() bytes
 // (the bf16 d(logits) with row stride linear_logp_dz_row_stride(V), then the bias block sums).
 // grad_hidden / grad_weight / grad_bias may each be null.

@@ -396,6 +396,162 @@ def fused_linear_logp_bwd(
     return [grad_hidden, grad_weight, grad_bias]
 
 
+def _logits_dtype_code(logits: torch.Tensor) -> int:
+    if not logits.is_cuda:
+        raise RuntimeError("logits must be a ROCm tensor")
+    if logits.dim() != 2:
+        raise RuntimeError("logits must be 2D [tokens, local_vocab]")
+    codes = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16, torch.float32: _lib.DTYPE_FP32}
+    if logits.dtype not in codes:
+        raise RuntimeError("logits must be float16, bfloat16, or float32")
+    return codes[logits.dtype]
+
+
+def _row_contiguous(logits: torch.Tensor) -> torch.Tensor:
+    return logits if logits.stride(1) == 1 and logits.stride(0) >= logits.size(1) else logits.contiguous()
+
+
+def hip_deterministic_logp_tile_stats(
+    logits: torch.Tensor,
+    vocab_start: int,
+    real_vocab: int,
+    num_tiles: int,
+    *,
+    temperature: Optional[torch.Tensor] = None,
+) -> List[torch.Tensor]:
+    """``[tile_max, tile_sum]``, each fp32 ``[rows, num_tiles]``, of materialised logits.
+
+    Same signature, checks and messages as ``_C.hip_deterministic_logp_tile_stats``
+    (csrc/bindings/ops.cpp:122-126; csrc/rocm/logprob/hip_deterministic_logp_kernel.hip:550-588).
+    ``temperature`` (fp32, one value per row) scales the logits by its reciprocal in registers.
+    """
+    code = _logits_dtype_code(logits)
+    if not (int(vocab_start) >= 0 and int(real_vocab) > 0 and int(num_tiles) > 0):
+        raise RuntimeError("invalid vocabulary metadata")
+    rows, local_vocab = logits.shape
+    if not (local_vocab > 0 and local_vocab % int(num_tiles) == 0):
+        raise RuntimeError("local_vocab must be divisible by num_tiles")
+    if int(num_tiles) > 65535:
+        raise RuntimeError("num_tiles must fit the launch grid")
+    src = _row_contiguous(logits)
+    tile_max = torch.empty((rows, int(num_tiles)), dtype=torch.float32, device=logits.device)
+    tile_sum = torch.empty((rows, int(num_tiles)), dtype=torch.float32, device=logits.device)
+    if rows == 0:
+        return [tile_max, tile_sum]
+    temp = None
+    if temperature is not None:
+        if temperature.numel() != rows:
+            raise RuntimeError("temperature must have one value per row")
+        temp = temperature.reshape(-1).to(device=logits.device, dtype=torch.float32).contiguous()
+    with torch.cuda.device(logits.device):
+        status = _lib.load().rlk_logits_tile_stats(
+            src.data_ptr(), code, src.stride(0), temp.data_ptr() if temp is not None else None, rows, local_vocab,
+            int(vocab_start), int(real_vocab), int(num_tiles), tile_max.data_ptr(), tile_sum.data_ptr(),
+            _stream_handle(logits.device),
+        )  # fmt: skip
+    _lib.check(status, "rlk_logits_tile_stats failed")
+    return [tile_max, tile_sum]
+
+
+def hip_deterministic_logp_from_logits(
+    logits: torch.Tensor,
+    target: torch.Tensor,
+    vocab_start: int,
+    real_vocab: int,
+    num_tiles: int,
+    *,
+    temperature: Optional[torch.Tensor] = None,
+) -> List[torch.Tensor]:
+    """``[logp, lse]`` (fp32 ``[rows]``) from materialised logits: tile statistics, ascending
+    tile merge and target gather in one pass over the logits. ``target`` holds global ids."""
+    code = _logits_dtype_code(logits)
+    if not (int(vocab_start) >= 0 and int(real_vocab) > 0 and int(num_tiles) > 0):
+        raise RuntimeError("invalid vocabulary metadata")
+    rows, local_vocab = logits.shape
+    if not (local_vocab > 0 and local_vocab % int(num_tiles) == 0):
+        raise RuntimeError("local_vocab must be divisible by num_tiles")
+    if target.numel() != rows:
+        raise RuntimeError("target must have one id per row")
+    src = _row_contiguous(logits)
+    logp = torch.empty((rows,), dtype=torch.float32, device=logits.device)
+    lse = torch.empty((rows,), dtype=torch.float32, device=logits.device)
+    if rows == 0:
+        return [logp, lse]
+    target_i64 = target.reshape(-1).to(device=logits.device, dtype=torch.int64).contiguous()
+    temp = None
+    if temperature is not None:
+        if temperature.numel() != rows:
+            raise RuntimeError("temperature must have one value per row")
+        temp = temperature.reshape(-1).to(device=logits.device, dtype=torch.float32).contiguous()
+    lib = _lib.load()
+    ws_bytes = int(lib.rlk_logp_from_logits_workspace_bytes(rows, int(num_tiles)))
+    workspace = torch.empty((ws_bytes // 4,), dtype=torch.float32, device=logits.device)
+    with torch.cuda.device(logits.device):
+        status = lib.rlk_logp_from_logits(
+            src.data_ptr(), code, src.stride(0), target_i64.data_ptr(), temp.data_ptr() if temp is not None else None,
+            rows, local_vocab, int(vocab_start), int(real_vocab), int(num_tiles), logp.data_ptr(), lse.data_ptr(),
+            workspace.data_ptr(), ws_bytes, _stream_handle(logits.device),
+        )  # fmt: skip
+    _lib.check(status, "rlk_logp_from_logits failed")
+    return [logp, lse]
+
+
+def hip_deterministic_logp_backward(
+    logits: torch.Tensor,
+    lse: torch.Tensor,
+    coef_logp: torch.Tensor,
+    coef_lse: torch.Tensor,
+    target_local: torch.Tensor,
+    vocab_start: int,
+    real_vocab: int,
+    has_lse_grad: bool,
+    *,
+    temperature: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """``grad = coef_logp * (onehot - p) + coef_lse * p`` in the dtype of ``logits``.
+
+    Same signature, checks and messages as ``_C.hip_deterministic_logp_backward``
+    (csrc/bindings/ops.cpp:127-135; hip_deterministic_logp_kernel.hip:590-640).
+    """
+    code = _logits_dtype_code(logits)
+    if not (int(vocab_start) >= 0 and int(real_vocab) > 0):
+        raise RuntimeError("invalid vocabulary metadata")
+    src = _row_contiguous(logits)
+    rows, local_vocab = src.shape
+
+    def _check_row_vector(t: torch.Tensor, dtype: torch.dtype, name: str) -> None:
+        if not t.is_cuda or t.device != src.device:
+            raise RuntimeError(f"{name} must live on the logits device")
+        if t.dtype != dtype:
+            raise RuntimeError(f"{name} has the wrong dtype")
+        if t.dim() != 1 or t.size(0) != rows:
+            raise RuntimeError(f"{name} must have one entry per token")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+
+    _check_row_vector(lse, torch.float32, "lse")
+    _check_row_vector(coef_logp, torch.float32, "coef_logp")
+    _check_row_vector(coef_lse, torch.float32, "coef_lse")
+    _check_row_vector(target_local, torch.int64, "target_local")
+    grad = torch.empty((rows, local_vocab), dtype=src.dtype, device=src.device)
+    if rows == 0 or local_vocab == 0:
+        return grad
+    temp = None
+    if temperature is not None:
+        if temperature.numel() != rows:
+            raise RuntimeError("temperature must have one value per row")
+        temp = temperature.reshape(-1).to(device=src.device, dtype=torch.float32).contiguous()
+    with torch.cuda.device(src.device):
+        status = _lib.load().rlk_logits_logp_backward(
+            src.data_ptr(), code, src.stride(0), lse.data_ptr(), coef_logp.data_ptr(),
+            coef_lse.data_ptr() if has_lse_grad else None, target_local.data_ptr(),
+            temp.data_ptr() if temp is not None else None, grad.data_ptr(), grad.stride(0), rows, local_vocab,
+            int(vocab_start), int(real_vocab), _stream_handle(src.device),
+        )  # fmt: skip
+    _lib.check(status, "rlk_logits_logp_backward failed")
+    return grad
+
+
 def grpo_ratio_kl_loss(
     logp: torch.Tensor,
     old_logp: torch.Tensor,

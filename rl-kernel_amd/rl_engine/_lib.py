@@ -36,6 +36,8 @@ GEMM_CONFIGS = {
 }
 # OR-ed into a GEMM or LogP configuration: register-staged main loop (bit-neutral).
 FORCE_STAGED = 0x100
+# rlk_dtype (element types of materialised logits)
+DTYPE_BF16, DTYPE_FP16, DTYPE_FP32 = 0, 1, 2
 # rlk_logp_config
 LOGP_CONFIGS = {"auto": 0, "256": 1, "128": 2, "64": 3, "16": 4}
 
@@ -51,6 +53,10 @@ EXPORTED_SYMBOLS = (
     "rlk_linear_logp_fwd",
     "rlk_linear_logp_bwd_workspace_bytes",
     "rlk_linear_logp_bwd",
+    "rlk_logits_tile_stats",
+    "rlk_logp_from_logits_workspace_bytes",
+    "rlk_logp_from_logits",
+    "rlk_logits_logp_backward",
     "rlk_grpo_workspace_bytes",
     "rlk_grpo_ratio_kl_loss",
 )
@@ -110,6 +116,15 @@ def load() -> ctypes.CDLL:
     lib.rlk_linear_logp_bwd.argtypes = [
         vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, vp, i64, vp, i64, vp, vp, sz, i32, i32, i32, i64, i32, i32, vp,
     ]  # fmt: skip
+
+    lib.rlk_logits_tile_stats.restype = i32
+    lib.rlk_logits_tile_stats.argtypes = [vp, i32, i64, vp, i32, i64, i64, i64, i32, vp, vp, vp]
+    lib.rlk_logp_from_logits_workspace_bytes.restype = sz
+    lib.rlk_logp_from_logits_workspace_bytes.argtypes = [i32, i32]
+    lib.rlk_logp_from_logits.restype = i32
+    lib.rlk_logp_from_logits.argtypes = [vp, i32, i64, vp, vp, i32, i64, i64, i64, i32, vp, vp, vp, sz, vp]
+    lib.rlk_logits_logp_backward.restype = i32
+    lib.rlk_logits_logp_backward.argtypes = [vp, i32, i64, vp, vp, vp, vp, vp, vp, i64, i32, i64, i64, i64, vp]
 
     lib.rlk_grpo_workspace_bytes.restype = sz
     lib.rlk_grpo_workspace_bytes.argtypes = [i32]

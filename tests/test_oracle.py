@@ -407,6 +407,75 @@ def test_logp_backward_bf16_dlogits_stay_within_their_rounding(oracle):
 
 
 # ---------------------------------------------------------------------------
+# log-probabilities from materialised logits
+# ---------------------------------------------------------------------------
+
+
+def test_logits_tile_stats_and_merge_against_scipy(oracle):
+    from scipy.special import logsumexp
+
+    rng = np.random.default_rng(31)
+    rows, v, start, real = 6, 96, 32, 32 + 70  # global columns 32..127, the last 26 are padding
+    z = (rng.standard_normal((rows, v)) * 3).astype(np.float32)
+    temp = np.array([0.5, 1.0, 2.0, 0.7, 1.0, 1.3], np.float32)
+    target = start + rng.integers(0, 70, rows)
+    exact = logsumexp(z[:, :70].astype(np.float64) / temp[:, None], axis=1)
+    for tiles in (1, 2, 8, 96):
+        m, s = oracle.logits_tile_stats(z, start, real, tiles, temperature=temp)
+        assert m.shape == (rows, tiles)
+        width = v // tiles
+        for t in range(tiles):
+            lo, hi = t * width, min((t + 1) * width, 70)
+            if hi <= lo:  # all padding: the identity of the merge
+                assert np.all(m[:, t] == -np.inf) and np.all(s[:, t] == 0)
+            else:
+                assert np.array_equal(m[:, t], (z[:, lo:hi] / temp[:, None]).astype(np.float32).max(axis=1))
+                assert np.all(s[:, t] >= 1.0) and np.all(s[:, t] <= hi - lo)
+        assert np.abs(oracle.merge_tile_partials(m, s) - exact).max() < 2e-6
+        logp, lse = oracle.logp_from_logits(z, target, start, real, tiles, temperature=temp)
+        zt = z[np.arange(rows), target - start].astype(np.float64) / temp
+        assert np.abs(logp - (zt - exact)).max() < 3e-6 and np.abs(lse - exact).max() < 2e-6
+    # a target owned by another shard contributes a zero logit
+    logp, lse = oracle.logp_from_logits(z, np.full(rows, 5), start, real, 8)
+    assert np.array_equal(logp, -lse)
+
+
+def test_logits_backward_matches_finite_differences(oracle):
+    from scipy.special import logsumexp
+
+    rng = np.random.default_rng(32)
+    rows, v, real = 3, 10, 8
+    z = rng.standard_normal((rows, v))
+    temp = np.array([0.5, 1.0, 1.75])
+    target = np.array([0, 7, 3])
+    g_logp = rng.standard_normal(rows)
+    g_lse = rng.standard_normal(rows)
+
+    def objective(arr):
+        y = arr[:, :real] / temp[:, None]
+        lse = logsumexp(y, axis=1)
+        return float((g_logp * (y[np.arange(rows), target] - lse) + g_lse * lse).sum()), lse
+
+    _, lse = objective(z)
+    grad = oracle.logits_logp_backward(z, lse, g_logp, g_lse, target, 0, real, temperature=temp, dtype=np.float64)
+    eps = 1e-6
+    for i in range(rows):
+        for j in range(v):
+            up, down = z.copy(), z.copy()
+            up[i, j] += eps
+            down[i, j] -= eps
+            fd = (objective(up)[0] - objective(down)[0]) / (2 * eps)
+            assert abs(fd - grad[i, j]) < 1e-7, (i, j)
+    assert np.all(grad[:, real:] == 0)
+    # rows of the gradient sum to coef_lse / temperature; a non-finite lse row gives onehot * coef only
+    assert np.allclose(grad.sum(axis=1), g_lse / temp, atol=1e-12)
+    dead = oracle.logits_logp_backward(z, np.full(rows, -np.inf), g_logp, None, target, 0, real, dtype=np.float64)
+    expect = np.zeros_like(z)
+    expect[np.arange(rows), target] = g_logp
+    assert np.array_equal(dead, expect)
+
+
+# ---------------------------------------------------------------------------
 # GRPO
 # ---------------------------------------------------------------------------
 
