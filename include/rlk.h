@@ -230,6 +230,48 @@ int rlk_logits_logp_backward(const void* logits, int dtype, int64_t row_stride, 
                              const float* temperature, void* grad, int64_t grad_row_stride, int T, int64_t V,
                              int64_t vocab_start, int64_t real_vocab, void* stream);
 
+/*
+ * SwiGLU on bf16 rows: y[m, c] = bf16((g * sigmoid(g)) * u) with g = gate[m * ld_gate + c],
+ * u = up[m * ld_up + c] widened to fp32 and sigmoid(g) = 1 / (1 + exp(-g)) (hardware
+ * reciprocal and exponential, each within 1 ulp). A packed
+ * [rows, 2 * cols] projection is the case up = gate + cols, ld_gate = ld_up = 2 * cols.
+ *
+ * Stands in for rl_engine._C.swiglu_forward / swiglu_packed_forward
+ * (csrc/bindings/ops.cpp:400-413; csrc/cuda/activation/activation.cu:62-75, 97-112).
+ */
+int rlk_swiglu_fwd(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, void* y, int64_t ld_y, int rows,
+                   int cols, void* stream);
+
+/*
+ * Backward of rlk_swiglu_fwd: d_up = bf16(dy * silu(g)), d_gate = bf16(dy * u * silu'(g)),
+ * silu'(g) = s * (1 + g * (1 - s)), s = sigmoid(g).
+ *
+ * Stands in for rl_engine._C.swiglu_backward / swiglu_packed_backward
+ * (csrc/bindings/ops.cpp:404-419; activation.cu:77-95, 114-135).
+ */
+int rlk_swiglu_bwd(const void* dy, int64_t ld_dy, const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                   void* d_gate, int64_t ld_d_gate, void* d_up, int64_t ld_d_up, int rows, int cols, void* stream);
+
+/* Bytes of workspace rlk_det_gemm_swiglu_bf16 needs for these operands: 0 when the fused
+ * kernel applies (unit K strides, 16-byte aligned rows, K % 64 == 0, M > 16), else the
+ * bf16 [M, 2 I] projection. */
+size_t rlk_det_gemm_swiglu_workspace_bytes(const void* a, int64_t a_row_stride, const void* w_packed,
+                                           int64_t w_row_stride, int M, int I, int K);
+
+/*
+ * y[M, I] = swiglu(a @ w_packed[0:I]^T, a @ w_packed[I:2I]^T): the packed gate/up projection
+ * of a gated FFN (weight rows [0, I) gate, [I, 2 I) up, unit stride along K) under the
+ * det_gemm contract, each projection rounded to bf16 before the activation, so the result
+ * equals rlk_det_gemm_bf16 followed by rlk_swiglu_fwd bit for bit. When the fused kernel
+ * applies the [M, 2 I] projection is never written.
+ *
+ * Stands in for rl_engine/backends/rocm/gemm/swiglu_gemm.py:36-86 (forward) and for
+ * _packed_gate_up_inference (rl_engine/backends/rocm/ffn/ffn.py:69-83).
+ */
+int rlk_det_gemm_swiglu_bf16(const void* a, int64_t a_row_stride, const void* w_packed, int64_t w_row_stride,
+                             void* y, int64_t ldy, void* workspace, size_t workspace_bytes, int M, int I, int K,
+                             void* stream);
+
 /* Bytes of workspace rlk_grpo_ratio_kl_loss needs. */
 size_t rlk_grpo_workspace_bytes(int rollouts);
 

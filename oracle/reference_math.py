@@ -33,6 +33,9 @@ Pinning (which check fixes which function; see tests/test_oracle.py):
   ``logits_logp_backward``: scipy's logsumexp on the real columns, tile-count
   independence of the merged lse, the all-padding tile identity, central finite
   differences of logsumexp and the gathered logit.
+* ``swiglu`` / ``swiglu_backward`` / ``swiglu_packed`` / ``gated_ffn``: silu(0) = 0,
+  silu(x) -> x and -> 0 in the tails, linearity in ``up``, central finite differences of
+  the fp64 formula, and ``gated_ffn`` against an fp64 evaluation.
 * ``grpo_ratio_kl_loss`` / ``group_advantages`` / ``masked_mean``: the reference's
   hand examples (tests/reference/test_reference_ops.py:77-98,
   tests/ops/loss/test_grpo_loss.py:112-119) and closed forms (old == logp gives
@@ -518,6 +521,54 @@ def logits_logp_backward(
     if temp is not None:
         grad = grad / temp[:, None]
     return grad.astype(dtype)
+
+
+# ---------------------------------------------------------------------------
+# SwiGLU and the gated FFN
+# ---------------------------------------------------------------------------
+
+
+def _sigmoid_f32(x: np.ndarray) -> np.ndarray:
+    with np.errstate(over="ignore"):
+        return (np.float32(1.0) / (np.float32(1.0) + np.exp(-x, dtype=np.float32))).astype(np.float32)
+
+
+def swiglu(gate_bits, up_bits) -> np.ndarray:
+    """``silu(gate) * up`` with fp32 math on the bf16 inputs, rounded once to bf16.
+
+    swiglu_forward_kernel / silu_f32, csrc/cuda/activation/activation.cu:20-24, 62-75:
+    ``s = 1 / (1 + expf(-g))``, ``y = (g * s) * u``.
+    """
+    g = bf16_to_f32(np.ascontiguousarray(gate_bits, dtype=np.uint16))
+    u = bf16_to_f32(np.ascontiguousarray(up_bits, dtype=np.uint16))
+    return f32_to_bf16(((g * _sigmoid_f32(g)).astype(np.float32) * u).astype(np.float32))
+
+
+def swiglu_backward(dy_bits, gate_bits, up_bits):
+    """``(d_gate, d_up)`` as bf16 bits: ``d_up = dy * silu(g)``,
+    ``d_gate = dy * u * s * (1 + g * (1 - s))`` (activation.cu:26-31, 77-95)."""
+    dy = bf16_to_f32(np.ascontiguousarray(dy_bits, dtype=np.uint16))
+    g = bf16_to_f32(np.ascontiguousarray(gate_bits, dtype=np.uint16))
+    u = bf16_to_f32(np.ascontiguousarray(up_bits, dtype=np.uint16))
+    s = _sigmoid_f32(g)
+    d_up = (dy * (g * s)).astype(np.float32)
+    d_gate = ((dy * u) * (s * (np.float32(1.0) + g * (np.float32(1.0) - s)))).astype(np.float32)
+    return f32_to_bf16(d_gate), f32_to_bf16(d_up)
+
+
+def swiglu_packed(gate_up_bits) -> np.ndarray:
+    """SwiGLU of a packed ``[rows, 2 I]`` projection: columns ``[0, I)`` gate, ``[I, 2 I)`` up
+    (swiglu_packed_forward_kernel, activation.cu:97-112)."""
+    gu = np.ascontiguousarray(gate_up_bits, dtype=np.uint16)
+    width = gu.shape[1] // 2
+    return swiglu(gu[:, :width], gu[:, width:])
+
+
+def gated_ffn(x_bits, gate_up_weight_bits, down_weight_bits) -> np.ndarray:
+    """``down(swiglu(x @ W_gu^T))`` with every projection rounded once to bf16
+    (_packed_gate_up_inference + det_gemm_linear, rl_engine/backends/rocm/ffn/ffn.py:69-104)."""
+    gate_up = det_gemm_ref(x_bits, gate_up_weight_bits)
+    return det_gemm_ref(swiglu_packed(gate_up), down_weight_bits)
 
 
 # ---------------------------------------------------------------------------

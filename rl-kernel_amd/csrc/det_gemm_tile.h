@@ -276,8 +276,46 @@ __device__ __forceinline__ void wg_barrier() {
 // and M % 8 == 0.
 __device__ __forceinline__ int kmajor_swizzle(int k_row) { return 2 * (((k_row >> 1) & 1) ^ ((k_row >> 3) & 3)); }
 
-template <class S, bool WK = false, bool XK = false>
+// Which weight row an LDS row of the native (reduction-contiguous) weight stage holds, split
+// into a block-uniform part and a part that depends on the lane's row inside the block.
+// PlainRowMap is weight_row_of_lds_row(). GatedRowMap serves a packed gate/up weight
+// [2 * I, K] (rows [0, I) gate, [I, 2 I) up): a tile covers BN / 2 features of both halves,
+// MFMA tiles jn = 0, 1 of a wave hold gate features wave_n * 32 + (lane>>4) * 8 + jn * 4 + q
+// and tiles jn = 2, 3 the up projection of the same features, so gate and up of one output
+// element meet in one lane.
+template <class S>
+struct PlainRowMap {
+  static constexpr bool kGated = false;
+  static __device__ __forceinline__ int block_offset(int b) {
+    constexpr int kWaveRows = 16 * S::TN;
+    const int r0 = b * 8;
+    return (r0 / kWaveRows) * kWaveRows + ((r0 % kWaveRows) / 16) * 4;
+  }
+  static __device__ __forceinline__ int block_half(int) { return 0; }
+  static __device__ __forceinline__ int lane_offset(int parity, int rib) {
+    const int i = parity * 8 + rib;
+    return (i >> 2) * S::kRun + (i & 3);
+  }
+};
+
+template <class S>
+struct GatedRowMap {
+  static_assert(S::TN == 4, "two gate and two up MFMA tiles per wave");
+  static constexpr bool kGated = true;
+  static __device__ __forceinline__ int block_offset(int b) {
+    const int r0 = b * 8;
+    return (r0 / 64) * 32 + (((r0 % 64) / 16) & 1) * 4;
+  }
+  static __device__ __forceinline__ int block_half(int b) { return ((b * 8 % 64) / 16) >> 1; }
+  static __device__ __forceinline__ int lane_offset(int parity, int rib) {
+    const int i = parity * 8 + rib;
+    return (i >> 2) * 8 + (i & 3);
+  }
+};
+
+template <class S, bool WK = false, bool XK = false, class Map = PlainRowMap<S>>
 struct DmaLoader {
+  static_assert(!(WK && Map::kGated), "the gated row map is for the native weight layout");
   static constexpr int kWaveRows = 16 * S::TN;
   static_assert(!WK || S::TN == 4, "K-major weights need 64-feature wave columns");
   static_assert(!XK || S::BM % 128 == 0, "K-major activations need whole 64-token columns per wave group");
@@ -298,17 +336,13 @@ struct DmaLoader {
   int kmajor_chunk;        // K-major operands: chunk position of this lane before the block part of the swizzle
 
   // Feature offset of lane row `rib` inside a weight block of parity p: LDS row
-  // r = 8 b + rib holds feature weight_row_of_lds_row(r), which is a block-uniform
-  // part plus (i >> 2) * kRun + (i & 3) with i = 8 p + rib.
-  static __device__ __forceinline__ int w_lane_row(int parity, int rib) {
-    const int i = parity * 8 + rib;
-    return (i >> 2) * S::kRun + (i & 3);
-  }
+  // r = 8 b + rib holds a block-uniform feature plus Map::lane_offset(p, rib).
+  static __device__ __forceinline__ int w_lane_row(int parity, int rib) { return Map::lane_offset(parity, rib); }
 
   __device__ __forceinline__ void init(const MatView& W, const MatView& X, int n0_, int m0_, int lane) {
     n0 = n0_;
     m0 = m0_;
-    n_rows = W.rows;
+    n_rows = Map::kGated ? W.rows / 2 : W.rows;  // rows of one half of a packed gate/up weight
     m_rows = X.rows;
     ldw = WK ? W.k_stride : W.row_stride;  // K-major: elements between consecutive K rows
     ldx = XK ? X.k_stride : X.row_stride;
@@ -350,16 +384,16 @@ struct DmaLoader {
       __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + b * 1024), 16, 0, 0);
       return;
     }
-    const int r0 = b * 8;
-    const int row0 = (r0 / kWaveRows) * kWaveRows + ((r0 % kWaveRows) / 16) * 4;  // block-uniform feature offset
+    const int row0 = Map::block_offset(b);  // block-uniform feature offset
     const int parity = b & 1;
+    const bf16_bits* half_base = w_base + (int64_t)(Map::block_half(b) * n_rows) * ldw;
     const bf16_bits* src;
-    if (n0 + row0 + (parity * 2 + 1) * S::kRun + 3 < n_rows) {
-      src = w_base + (int64_t)row0 * ldw + k0 + w_lane_off[parity];
+    if (n0 + row0 + w_lane_row(parity, 7) < n_rows) {
+      src = half_base + (int64_t)row0 * ldw + k0 + w_lane_off[parity];
     } else {
       int g = n0 + row0 + w_lane_row(parity, rib);
       g = g < n_rows ? g : n_rows - 1;
-      src = w_base + (int64_t)(g - n0) * ldw + k0 + chunk_elems;
+      src = half_base + (int64_t)(g - n0) * ldw + k0 + chunk_elems;
     }
     __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + b * 1024), 16, 0, 0);
   }
@@ -403,11 +437,11 @@ constexpr bool pingpong_supported() {
 
 // With WK the accumulator of MFMA tile jn holds features wave_n*64 + jn*16 + (lane>>4)*4 + q
 // (no run permutation: a K-major chunk is eight consecutive features).
-template <class S, bool WK = false, bool XK = false>
+template <class S, bool WK = false, bool XK = false, class Map = PlainRowMap<S>>
 __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const MatView& X, int n0, int m0, int K,
                                                        char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
   static_assert(pingpong_supported<S>(), "two groups of four waves, 4 x 2 wave layout");
-  using Loader = DmaLoader<S, WK, XK>;
+  using Loader = DmaLoader<S, WK, XK, Map>;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -281,6 +281,79 @@ int rlk_logits_logp_backward(const void* logits, int dtype, int64_t row_stride, 
   return err == hipSuccess ? RLK_OK : device_error("rlk_logits_logp_backward", err);
 }
 
+int rlk_swiglu_fwd(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, void* y, int64_t ld_y, int rows,
+                   int cols, void* stream) {
+  if (rows < 0 || cols < 0) {
+    set_last_error("rlk_swiglu_fwd: negative sizes");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (rows == 0 || cols == 0) return RLK_OK;
+  if (gate == nullptr || up == nullptr || y == nullptr || ld_gate < cols || ld_up < cols || ld_y < cols) {
+    set_last_error("rlk_swiglu_fwd: null operand or row stride < cols");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  hipError_t err = swiglu_launch(gate, ld_gate, up, ld_up, nullptr, 0, y, ld_y, nullptr, 0, rows, cols, false,
+                                 reinterpret_cast<hipStream_t>(stream));
+  return err == hipSuccess ? RLK_OK : device_error("rlk_swiglu_fwd", err);
+}
+
+int rlk_swiglu_bwd(const void* dy, int64_t ld_dy, const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                   void* d_gate, int64_t ld_d_gate, void* d_up, int64_t ld_d_up, int rows, int cols, void* stream) {
+  if (rows < 0 || cols < 0) {
+    set_last_error("rlk_swiglu_bwd: negative sizes");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (rows == 0 || cols == 0) return RLK_OK;
+  if (dy == nullptr || gate == nullptr || up == nullptr || d_gate == nullptr || d_up == nullptr || ld_dy < cols ||
+      ld_gate < cols || ld_up < cols || ld_d_gate < cols || ld_d_up < cols) {
+    set_last_error("rlk_swiglu_bwd: null operand or row stride < cols");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  hipError_t err = swiglu_launch(gate, ld_gate, up, ld_up, dy, ld_dy, d_gate, ld_d_gate, d_up, ld_d_up, rows, cols,
+                                 true, reinterpret_cast<hipStream_t>(stream));
+  return err == hipSuccess ? RLK_OK : device_error("rlk_swiglu_bwd", err);
+}
+
+size_t rlk_det_gemm_swiglu_workspace_bytes(const void* a, int64_t a_row_stride, const void* w_packed,
+                                           int64_t w_row_stride, int M, int I, int K) {
+  if (M <= 0 || I <= 0 || K <= 0) return 0;
+  MatView X{reinterpret_cast<const bf16_bits*>(a), a_row_stride, 1, M};
+  MatView W{reinterpret_cast<const bf16_bits*>(w_packed), w_row_stride, 1, 2 * I};
+  return det_gemm_swiglu_fused_supported(W, X, M, K) ? 0 : (size_t)M * 2 * (size_t)I * sizeof(bf16_bits);
+}
+
+int rlk_det_gemm_swiglu_bf16(const void* a, int64_t a_row_stride, const void* w_packed, int64_t w_row_stride,
+                             void* y, int64_t ldy, void* workspace, size_t workspace_bytes, int M, int I, int K,
+                             void* stream) {
+  if (M < 0 || I < 0 || K < 0 || I > 0x3fffffff) {
+    set_last_error("rlk_det_gemm_swiglu_bf16: bad sizes M=%d I=%d K=%d", M, I, K);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (M == 0 || I == 0) return RLK_OK;
+  if (y == nullptr || ldy < I) {
+    set_last_error("rlk_det_gemm_swiglu_bf16: null output or ldy < I");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (K == 0) {  // both projections are zero and swiglu(0, 0) = 0
+    hipError_t err = fill_zero_launch(y, M, I, ldy, 2, s);
+    return err == hipSuccess ? RLK_OK : device_error("rlk_det_gemm_swiglu_bf16(fill)", err);
+  }
+  if (a == nullptr || w_packed == nullptr || a_row_stride < K || w_row_stride < K) {
+    set_last_error("rlk_det_gemm_swiglu_bf16: null operand or row stride < K");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  const size_t need = rlk_det_gemm_swiglu_workspace_bytes(a, a_row_stride, w_packed, w_row_stride, M, I, K);
+  if (need > 0 && (workspace == nullptr || workspace_bytes < need)) {
+    set_last_error("rlk_det_gemm_swiglu_bf16: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  MatView X{reinterpret_cast<const bf16_bits*>(a), a_row_stride, 1, M};
+  MatView W{reinterpret_cast<const bf16_bits*>(w_packed), w_row_stride, 1, 2 * I};
+  hipError_t err = det_gemm_swiglu_launch(W, X, y, ldy, workspace, M, I, K, s);
+  return err == hipSuccess ? RLK_OK : device_error("rlk_det_gemm_swiglu_bf16", err);
+}
+
 size_t rlk_grpo_workspace_bytes(int rollouts) { return rollouts > 0 ? (size_t)3 * rollouts * sizeof(float) : 0; }
 
 int rlk_grpo_ratio_kl_loss(const float* logp, const float* old_logp, const float* ref_logp,

@@ -552,6 +552,147 @@ def hip_deterministic_logp_backward(
     return grad
 
 
+def _check_act(t: torch.Tensor, name: str) -> None:
+    """Checks of check_cuda_contig (csrc/cuda/activation/activation.cu:145-156); this build's
+    activation kernels serve bf16, the dtype of the GEMMs either side."""
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if t.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        raise RuntimeError(f"{name} must be fp16, bf16, or fp32, got {t.dtype}")
+    if t.dtype != _BF16:
+        raise RuntimeError(f"{name}: the gfx950 SwiGLU kernels serve bf16 only, got {t.dtype}")
+
+
+def _rows_cols(t: torch.Tensor) -> tuple:
+    cols = t.size(-1) if t.dim() else 1
+    return (t.numel() // cols if cols else 0), cols
+
+
+def swiglu_forward(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """``silu(gate) * up`` elementwise (csrc/bindings/ops.cpp:400-402; activation.cu:211-240)."""
+    _check_act(gate, "gate")
+    _check_act(up, "up")
+    if gate.device != up.device:
+        raise RuntimeError(f"gate and up must be on the same CUDA device, got {gate.device} and {up.device}")
+    if gate.shape != up.shape:
+        raise RuntimeError("gate and up must share shape")
+    y = torch.empty_like(gate)
+    rows, cols = _rows_cols(gate)
+    if gate.numel():
+        with torch.cuda.device(gate.device):
+            status = _lib.load().rlk_swiglu_fwd(
+                gate.data_ptr(), cols, up.data_ptr(), cols, y.data_ptr(), cols, rows, cols, _stream_handle(gate.device)
+            )
+        _lib.check(status, "rlk_swiglu_fwd failed")
+    return y
+
+
+def swiglu_backward(dy: torch.Tensor, gate: torch.Tensor, up: torch.Tensor) -> List[torch.Tensor]:
+    """``[d_gate, d_up]`` of :func:`swiglu_forward` (ops.cpp:404-409; activation.cu:242-284)."""
+    _check_act(dy, "dy")
+    _check_act(gate, "gate")
+    _check_act(up, "up")
+    if gate.shape != up.shape:
+        raise RuntimeError("gate and up must share shape")
+    if dy.shape != gate.shape:
+        raise RuntimeError("dy and gate must share shape")
+    d_gate, d_up = torch.empty_like(gate), torch.empty_like(up)
+    rows, cols = _rows_cols(gate)
+    if gate.numel():
+        with torch.cuda.device(gate.device):
+            status = _lib.load().rlk_swiglu_bwd(
+                dy.data_ptr(), cols, gate.data_ptr(), cols, up.data_ptr(), cols, d_gate.data_ptr(), cols,
+                d_up.data_ptr(), cols, rows, cols, _stream_handle(gate.device),
+            )  # fmt: skip
+        _lib.check(status, "rlk_swiglu_bwd failed")
+    return [d_gate, d_up]
+
+
+def swiglu_packed_forward(gate_up: torch.Tensor) -> torch.Tensor:
+    """SwiGLU of a packed ``[rows, 2 * intermediate]`` projection -> ``[rows, intermediate]``
+    (ops.cpp:411-413; activation.cu:286-320)."""
+    _check_act(gate_up, "gate_up")
+    if gate_up.dim() != 2:
+        raise RuntimeError("gate_up must be [rows, 2 * intermediate]")
+    if gate_up.size(1) % 2:
+        raise RuntimeError("gate_up width must be even")
+    rows, width = gate_up.size(0), gate_up.size(1) // 2
+    y = torch.empty((rows, width), dtype=gate_up.dtype, device=gate_up.device)
+    if y.numel():
+        base = gate_up.data_ptr()
+        with torch.cuda.device(gate_up.device):
+            status = _lib.load().rlk_swiglu_fwd(
+                base, 2 * width, base + 2 * width, 2 * width, y.data_ptr(), width, rows, width,
+                _stream_handle(gate_up.device),
+            )  # fmt: skip
+        _lib.check(status, "rlk_swiglu_fwd failed")
+    return y
+
+
+def swiglu_packed_backward(dy: torch.Tensor, gate_up: torch.Tensor) -> List[torch.Tensor]:
+    """``[d_gate, d_up]`` (each ``[rows, intermediate]``) of :func:`swiglu_packed_forward`
+    (ops.cpp:415-419; activation.cu:322-370)."""
+    _check_act(dy, "dy")
+    _check_act(gate_up, "gate_up")
+    if gate_up.dim() != 2 or dy.dim() != 2:
+        raise RuntimeError("gate_up must be [rows, 2 * intermediate]")
+    if gate_up.size(1) % 2:
+        raise RuntimeError("gate_up width must be even")
+    rows, width = gate_up.size(0), gate_up.size(1) // 2
+    if tuple(dy.shape) != (rows, width):
+        raise RuntimeError("dy must be [rows, intermediate]")
+    d_gate = torch.empty((rows, width), dtype=gate_up.dtype, device=gate_up.device)
+    d_up = torch.empty_like(d_gate)
+    if d_gate.numel():
+        base = gate_up.data_ptr()
+        with torch.cuda.device(gate_up.device):
+            status = _lib.load().rlk_swiglu_bwd(
+                dy.data_ptr(), width, base, 2 * width, base + 2 * width, 2 * width, d_gate.data_ptr(), width,
+                d_up.data_ptr(), width, rows, width, _stream_handle(gate_up.device),
+            )  # fmt: skip
+        _lib.check(status, "rlk_swiglu_bwd failed")
+    return [d_gate, d_up]
+
+
+def det_gemm_swiglu(a: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``swiglu(a @ weight[:I].T, a @ weight[I:].T)`` for a packed ``[2 I, K]`` gate/up weight.
+
+    Equals ``swiglu_packed_forward(det_gemm_fwd_rhs_transposed(a, weight))`` bit for bit; with
+    contiguous operands, ``K % 64 == 0`` and more than 16 rows the ``[M, 2 I]`` projection is
+    never written (rl_engine/backends/rocm/gemm/swiglu_gemm.py:36-86).
+    """
+    _check_in(a, "A")
+    _check_in(weight, "weight")
+    if a.dim() != 2 or weight.dim() != 2:
+        raise RuntimeError("det_gemm_swiglu: expect a[M,K] and weight[2I,K]")
+    if weight.size(1) != a.size(1):
+        raise RuntimeError("det_gemm_swiglu: K mismatch")
+    if weight.size(0) % 2:
+        raise RuntimeError("det_gemm_swiglu: packed gate/up weight needs an even number of rows")
+    a_c = a if a.stride(1) == 1 else a.contiguous()
+    w_c = weight if weight.stride(1) == 1 else weight.contiguous()
+    m, k = a_c.shape
+    inter = w_c.size(0) // 2
+    if out is None:
+        out = torch.empty((m, inter), dtype=_BF16, device=a.device)
+    elif tuple(out.shape) != (m, inter) or out.dtype != _BF16 or out.stride(1) != 1:
+        raise RuntimeError(f"det_gemm_swiglu: out must be a row-contiguous bf16 [{m}, {inter}] tensor")
+    if m == 0 or inter == 0:
+        return out
+    lib = _lib.load()
+    ws_bytes = int(lib.rlk_det_gemm_swiglu_workspace_bytes(a_c.data_ptr(), a_c.stride(0), w_c.data_ptr(), w_c.stride(0), m, inter, k))
+    workspace = torch.empty((ws_bytes // 2,), dtype=_BF16, device=a.device) if ws_bytes else None
+    with torch.cuda.device(a.device):
+        status = lib.rlk_det_gemm_swiglu_bf16(
+            a_c.data_ptr(), a_c.stride(0), w_c.data_ptr(), w_c.stride(0), out.data_ptr(), out.stride(0),
+            workspace.data_ptr() if workspace is not None else None, ws_bytes, m, inter, k, _stream_handle(a.device),
+        )  # fmt: skip
+    _lib.check(status, "rlk_det_gemm_swiglu_bf16 failed")
+    return out
+
+
 def grpo_ratio_kl_loss(
     logp: torch.Tensor,
     old_logp: torch.Tensor,

@@ -57,6 +57,10 @@ EXPORTED_SYMBOLS = (
     "rlk_logp_from_logits_workspace_bytes",
     "rlk_logp_from_logits",
     "rlk_logits_logp_backward",
+    "rlk_swiglu_fwd",
+    "rlk_swiglu_bwd",
+    "rlk_det_gemm_swiglu_workspace_bytes",
+    "rlk_det_gemm_swiglu_bf16",
     "rlk_grpo_workspace_bytes",
     "rlk_grpo_ratio_kl_loss",
 )
@@ -125,6 +129,15 @@ def load() -> ctypes.CDLL:
     lib.rlk_logp_from_logits.argtypes = [vp, i32, i64, vp, vp, i32, i64, i64, i64, i32, vp, vp, vp, sz, vp]
     lib.rlk_logits_logp_backward.restype = i32
     lib.rlk_logits_logp_backward.argtypes = [vp, i32, i64, vp, vp, vp, vp, vp, vp, i64, i32, i64, i64, i64, vp]
+
+    lib.rlk_swiglu_fwd.restype = i32
+    lib.rlk_swiglu_fwd.argtypes = [vp, i64, vp, i64, vp, i64, i32, i32, vp]
+    lib.rlk_swiglu_bwd.restype = i32
+    lib.rlk_swiglu_bwd.argtypes = [vp, i64, vp, i64, vp, i64, vp, i64, vp, i64, i32, i32, vp]
+    lib.rlk_det_gemm_swiglu_workspace_bytes.restype = sz
+    lib.rlk_det_gemm_swiglu_workspace_bytes.argtypes = [vp, i64, vp, i64, i32, i32, i32]
+    lib.rlk_det_gemm_swiglu_bf16.restype = i32
+    lib.rlk_det_gemm_swiglu_bf16.argtypes = [vp, i64, vp, i64, vp, i64, vp, sz, i32, i32, i32, vp]
 
     lib.rlk_grpo_workspace_bytes.restype = sz
     lib.rlk_grpo_workspace_bytes.argtypes = [i32]

@@ -476,6 +476,59 @@ def test_logits_backward_matches_finite_differences(oracle):
 
 
 # ---------------------------------------------------------------------------
+# SwiGLU / gated FFN
+# ---------------------------------------------------------------------------
+
+
+def test_swiglu_closed_forms_and_finite_differences(oracle):
+    f = lambda arr: oracle.bf16_to_f32(arr).astype(np.float64)  # noqa: E731
+    zero = _bits(oracle, [0.0])
+    assert f(oracle.swiglu(zero, _bits(oracle, [3.0])))[0] == 0.0
+    # tails: silu(x) -> x for large x, -> 0 for very negative x
+    assert f(oracle.swiglu(_bits(oracle, [40.0]), _bits(oracle, [1.0])))[0] == 40.0
+    assert abs(f(oracle.swiglu(_bits(oracle, [-40.0]), _bits(oracle, [1.0])))[0]) < 1e-15
+    # silu(1) * 2 = 2 / (1 + e^-1)
+    assert abs(f(oracle.swiglu(_bits(oracle, [1.0]), _bits(oracle, [2.0])))[0] - 2.0 / (1.0 + math.exp(-1.0))) < 2.0**-8 * 1.5
+    rng = np.random.default_rng(41)
+    g = oracle.randn_bf16(rng, (64,), 2.0)
+    u = oracle.randn_bf16(rng, (64,), 1.0)
+    dy = oracle.randn_bf16(rng, (64,), 1.0)
+    gf, uf, dyf = f(g), f(u), f(dy)
+    exact = gf / (1.0 + np.exp(-gf)) * uf
+    assert np.all(np.abs(f(oracle.swiglu(g, u)) - exact) <= 2.0**-8 * np.abs(exact) + 1e-30)
+    # linear in up: swiglu(g, 2u) = 2 swiglu(g, u) exactly (a power-of-two scale commutes with rounding)
+    u2 = _bits(oracle, (2.0 * uf).astype(np.float32))
+    assert np.array_equal(f(oracle.swiglu(g, u2)), 2.0 * f(oracle.swiglu(g, u)))
+    # backward against central differences of the fp64 formula
+    eps = 1e-6
+    silu = lambda x: x / (1.0 + np.exp(-x))  # noqa: E731
+    d_gate_fd = dyf * uf * (silu(gf + eps) - silu(gf - eps)) / (2 * eps)
+    d_up_fd = dyf * silu(gf)
+    d_gate, d_up = oracle.swiglu_backward(dy, g, u)
+    assert np.all(np.abs(f(d_gate) - d_gate_fd) <= 2.0**-8 * np.abs(d_gate_fd) + 1e-6)
+    assert np.all(np.abs(f(d_up) - d_up_fd) <= 2.0**-8 * np.abs(d_up_fd) + 1e-30)
+    # packed layout: columns [0, I) gate, [I, 2I) up
+    packed = np.concatenate([g.reshape(4, 16), u.reshape(4, 16)], axis=1)
+    assert np.array_equal(oracle.swiglu_packed(packed), oracle.swiglu(g, u).reshape(4, 16))
+
+
+def test_gated_ffn_against_fp64(oracle):
+    rng = np.random.default_rng(42)
+    t, h, i = 6, 32, 48
+    x = oracle.randn_bf16(rng, (t, h))
+    w_gu = oracle.randn_bf16(rng, (2 * i, h), 0.2)
+    w_d = oracle.randn_bf16(rng, (h, i), 0.2)
+    f = lambda arr: oracle.bf16_to_f32(arr).astype(np.float64)  # noqa: E731
+    gu = f(x) @ f(w_gu).T
+    act = gu[:, :i] / (1.0 + np.exp(-gu[:, :i])) * gu[:, i:]
+    exact = act @ f(w_d).T
+    got = f(oracle.gated_ffn(x, w_gu, w_d))
+    # three roundings to bf16 along the way: gate_up, the activation, the output
+    scale = np.abs(act) @ np.abs(f(w_d)).T
+    assert np.all(np.abs(got - exact) <= 2.0**-8 * np.abs(exact) + 3 * 2.0**-8 * scale + 1e-6)
+
+
+# ---------------------------------------------------------------------------
 # GRPO
 # ---------------------------------------------------------------------------
 
