@@ -12,7 +12,9 @@ H[4096,12288] x W[4096,12288]^T, inputs resident in HBM. The JSON line also carr
                      this box's host cores on the same step;
 * ``shapes``       - every token count of the configuration (T = 1, 16, 256, 4096)
                      with its own MFMA or HBM fraction;
-* ``linear_logp``  - the fused linear-LogP at T=8192, V=151936, D=4096 in tokens/s.
+* ``linear_logp``  - the fused linear-LogP at T=8192, V=151936, D=4096 in tokens/s, with its
+                     backward and the from-logits stage;
+* ``ffn``          - the gated FFN (fused gate/up + SwiGLU, then down) at T=4096.
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-logp]
 """
@@ -46,12 +48,12 @@ MEASURED_TRAFFIC_BYTES = {"det_gemm_gate_up_T4096": 1.412e9}  # 1.209 GB fetched
 def _parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-logp", action="store_true", help="skip the linear-LogP leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-T table")
-    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|logp|copy (used for profiling)")
+    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|logp|logp_bwd|from_logits|ffn|copy (used for profiling)")
     return ap.parse_args()
 
 
@@ -146,6 +148,28 @@ def main() -> int:
         ms = _time_calls(lambda: deterministic_linear_logp(hid, w_lm, tgt), args.steps, args.warmup)
         print(json.dumps({"leg": "logp", "ms": ms, "tokens_per_s": tl / ms * 1e3, "launches": args.steps + args.warmup}))
         return 0
+    if args.only in ("logp_bwd", "from_logits"):
+        from rl_engine import _C
+
+        tl = 8192
+        hid = randn(tl, HIDDEN)
+        w_lm = randn(VOCAB, HIDDEN, 0.02)
+        tgt = torch.randint(0, VOCAB, (tl,), generator=gen, device=dev)
+        if args.only == "logp_bwd":
+            _, lse = _C.fused_linear_logp(hid, w_lm, tgt)
+            g = torch.randn((tl,), generator=gen, device=dev)
+            ms = _time_calls(lambda: _C.fused_linear_logp_bwd(hid, w_lm, tgt, lse, g, None), args.steps, args.warmup)
+        else:
+            logits = randn(tl, VOCAB, 4.0)
+            ms = _time_calls(lambda: _C.hip_deterministic_logp_from_logits(logits, tgt, 0, VOCAB, 64), args.steps, args.warmup)
+        print(json.dumps({"leg": args.only, "ms": ms, "tokens_per_s": tl / ms * 1e3, "launches": args.steps + args.warmup}))
+        return 0
+    if args.only == "ffn":
+        from rl_engine.ops.ffn import qwen3_ffn_packed_inference
+
+        ms = _time_calls(lambda: qwen3_ffn_packed_inference(x, w_gu, w_d), args.steps, args.warmup)
+        print(json.dumps({"leg": "ffn", "ms": ms, "launches": args.steps + args.warmup}))
+        return 0
     if args.only in ("gate_up", "down"):
         fn = gate_up if args.only == "gate_up" else down
         ms = _time_calls(fn, args.steps, args.warmup)
@@ -167,8 +191,8 @@ def main() -> int:
     tflops = (flops_gu + flops_d) / wall_ms * 1e-9
 
     # ---- dominant kernel, HIP events over the same launches
-    ms_gu = _time_calls(gate_up, args.steps, 2)
-    ms_d = _time_calls(down, args.steps, 2)
+    ms_gu = _time_calls(gate_up, args.steps, 5)
+    ms_d = _time_calls(down, args.steps, 5)
     achieved = flops_gu / ms_gu * 1e-9
     roofline = {
         "kernel": "det_gemm_kernel<256x256 tile, 8 waves> on gate_up [4096x4096]x[24576x4096]^T",
@@ -216,7 +240,7 @@ def main() -> int:
         for t in (1, 16, 256, 1024, 4096):
             for name, act, w, n, k, out in (("gate_up", x, w_gu, 2 * INTER, HIDDEN, out_gu), ("down", h, w_d, HIDDEN, INTER, out_d)):
                 a_t, o_t = act[:t], out[:t]
-                ms = _time_calls(lambda: gemm.mfma_gemm(a_t, w.t(), out=o_t), 30 if t <= 256 else 10, 3)
+                ms = _time_calls(lambda: gemm.mfma_gemm(a_t, w.t(), out=o_t), 30 if t <= 256 else 10, 10)
                 fl = 2.0 * t * n * k
                 by = _gemm_bytes(t, n, k)
                 tf, gb = fl / ms * 1e-9, by / ms * 1e-6
@@ -241,7 +265,9 @@ def main() -> int:
         hid = (hid.float() * torch.rsqrt(hid.float().pow(2).mean(-1, keepdim=True) + 1e-6)).to(torch.bfloat16)
         w_lm = randn(VOCAB, HIDDEN, 0.02)
         tgt = torch.randint(0, VOCAB, (tl,), generator=gen, device=dev)
-        ms_lp = _time_calls(lambda: deterministic_linear_logp(hid, w_lm, tgt), 5, 2)
+        from rl_engine import _C
+
+        ms_lp = _time_calls(lambda: deterministic_linear_logp(hid, w_lm, tgt), 10, 4)
         fl_lp = 2.0 * tl * VOCAB * HIDDEN
         result["linear_logp"] = {
             "workload": "hidden[8192,4096] x lm_head[151936,4096]^T -> online LSE -> target gather, fp32 logp",
@@ -250,6 +276,44 @@ def main() -> int:
             "tflops": round(fl_lp / ms_lp * 1e-9, 1),
             "frac_of_mfma_peak": round(fl_lp / ms_lp * 1e-9 / PEAK_BF16_TFLOPS, 4),
             "min_hbm_bytes": 2.0 * (VOCAB * HIDDEN + tl * HIDDEN) + 8.0 * tl,
+        }
+        # backward: logits recompute + grad_hidden + grad_weight = three GEMMs of the forward's size
+        _, lse_lp = _C.fused_linear_logp(hid, w_lm, tgt)
+        g_lp = torch.randn((tl,), generator=gen, device=dev)
+        ms_bwd = _time_calls(lambda: _C.fused_linear_logp_bwd(hid, w_lm, tgt, lse_lp, g_lp, None), 5, 2)
+        result["linear_logp"]["backward"] = {
+            "workload": "d(logits) recompute (bf16, 2.49 GB) -> grad_hidden[8192,4096] and grad_weight[151936,4096]",
+            "ms": round(ms_bwd, 3),
+            "tokens_per_s": round(tl / ms_bwd * 1e3, 1),
+            "tflops": round(3 * fl_lp / ms_bwd * 1e-9, 1),
+            "frac_of_mfma_peak": round(3 * fl_lp / ms_bwd * 1e-9 / PEAK_BF16_TFLOPS, 4),
+        }
+        del lse_lp, g_lp
+        # the stage that reuses materialised logits: one pass over [8192, 151936] bf16
+        logits = randn(tl, VOCAB, 4.0)
+        ms_fl = _time_calls(lambda: _C.hip_deterministic_logp_from_logits(logits, tgt, 0, VOCAB, 64), 10, 4)
+        by_fl = 2.0 * tl * VOCAB
+        result["linear_logp"]["from_logits"] = {
+            "workload": "bf16 logits[8192,151936] -> 64 tile statistics -> merge -> target gather",
+            "ms": round(ms_fl, 3),
+            "tokens_per_s": round(tl / ms_fl * 1e3, 1),
+            "bound": "hbm",
+            "gbps": round(by_fl / ms_fl * 1e-6, 1),
+            "frac_of_hbm_peak": round(by_fl / ms_fl * 1e-6 / PEAK_HBM_GBPS, 4),
+        }
+        del logits
+
+    # ---- gated FFN at T=4096: fused gate/up + SwiGLU, then down
+    if not args.no_shapes:
+        from rl_engine.ops.ffn import qwen3_ffn_packed_inference
+
+        ms_ffn = _time_calls(lambda: qwen3_ffn_packed_inference(x, w_gu, w_d), 20, 10)
+        result["ffn"] = {
+            "workload": "x[4096,4096] -> packed gate/up GEMM with SwiGLU epilogue -> down GEMM, bf16",
+            "ms": round(ms_ffn, 4),
+            "tflops": round((flops_gu + flops_d) / ms_ffn * 1e-9, 1),
+            "frac_of_mfma_peak": round((flops_gu + flops_d) / ms_ffn * 1e-9 / PEAK_BF16_TFLOPS, 4),
+            "tokens_per_s": round(T / ms_ffn * 1e3, 1),
         }
 
     # ---- CPU baseline: the oracle on the same step, on this box's host cores
