@@ -47,7 +47,10 @@ typedef enum rlk_gemm_config {
   RLK_GEMM_CFG_STREAM16_DEEP = 8, /* M <= 16: 16-feature panel per workgroup, 512-wide ring stages */
   RLK_GEMM_CFG_STREAM16 = 9,      /* M <= 16: same with 256-wide ring stages, two workgroups per CU */
   RLK_GEMM_CFG_256x64 = 10,
-  RLK_GEMM_CFG_COUNT = 11,
+  RLK_GEMM_CFG_64x64_DEEP = 11,   /* 64x64 tile, 256 K values per barrier pair (few, long tiles) */
+  RLK_GEMM_CFG_128x64_DEEP = 12,  /* 128x64 tile, 128 K values per barrier pair */
+  RLK_GEMM_CFG_128x128_DEEP = 13, /* 128x128 tile, 128 K values per barrier pair */
+  RLK_GEMM_CFG_COUNT = 14,
   /* OR-ed into a configuration: use the register-staged main loop even where the
    * direct-to-LDS ping-pong loop applies. Bit-neutral; exists so tests can
    * compare the two loops. */

@@ -26,7 +26,7 @@ enum : int {
 constexpr bool loop_weight_kmajor(int loop) { return loop == kLoopPingPongKMajor || loop == kLoopPingPongBothKMajor; }
 constexpr bool loop_act_kmajor(int loop) { return loop == kLoopPingPongXKMajor || loop == kLoopPingPongBothKMajor; }
 
-template <class S, int LOOP, bool OUT_F32>
+template <class S, int LOOP, bool OUT_F32, int KS = 1>
 __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatView X, void* __restrict__ C,
                                                                 int64_t ldc, int M, int N, int K,
                                                                 int tiles_m, int tiles_n, int group_m) {
@@ -50,7 +50,7 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
   if constexpr (LOOP >= kLoopPingPongKMajor) {
     tile_mainloop_pingpong<S, loop_weight_kmajor(LOOP), loop_act_kmajor(LOOP)>(W, X, n0, m0, K, lds, acc);
   } else if constexpr (LOOP == kLoopPingPong) {
-    tile_mainloop_pingpong<S>(W, X, n0, m0, K, lds, acc);
+    tile_mainloop_pingpong<S, false, false, PlainRowMap<S>, KS>(W, X, n0, m0, K, lds, acc);
   } else {
     tile_mainloop_staged<S, LOOP == kLoopStaged>(W, X, n0, m0, K, lds, acc);
   }
@@ -152,25 +152,25 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
 // Host side
 // ---------------------------------------------------------------------------
 
-template <class S, int LOOP, bool OUT_F32>
+template <class S, int LOOP, bool OUT_F32, int KS = 1>
 static hipError_t launch_tile(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
                               hipStream_t stream) {
-  auto kernel = det_gemm_kernel<S, LOOP, OUT_F32>;
+  auto kernel = det_gemm_kernel<S, LOOP, OUT_F32, KS>;
+  constexpr int kLds = KS * S::kLdsBytes;
   static bool configured[kMaxDevices] = {};
   int dev = 0;
   hipError_t err = hipGetDevice(&dev);
   if (err != hipSuccess) return err;
   if (dev >= 0 && dev < kMaxDevices && !configured[dev]) {
-    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              S::kLdsBytes);
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (err != hipSuccess) return err;
     configured[dev] = true;
   }
   const int tiles_m = (M + S::BM - 1) / S::BM;
   const int tiles_n = (N + S::BN - 1) / S::BN;
   int group_m = tiles_m < 8 ? tiles_m : 8;
-  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(S::kThreads), S::kLdsBytes, stream, W, X, C, ldc, M, N,
-                     K, tiles_m, tiles_n, group_m);
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(S::kThreads), kLds, stream, W, X, C, ldc, M, N, K,
+                     tiles_m, tiles_n, group_m);
   return hipGetLastError();
 }
 
@@ -203,6 +203,17 @@ static hipError_t launch_shape(const MatView& W, const MatView& X, void* C, int6
   return launch_loop<S, kLoopGeneric>(W, X, C, ldc, M, N, K, out_f32, stream);
 }
 
+constexpr int kDeep64 = 4;   // 64x64: 4 K tiles per stage, 2 x 64 KiB of LDS
+constexpr int kDeep128 = 2;  // 128x64 / 128x128: 2 K tiles per stage, 2 x 48 / 2 x 64 KiB
+
+// Deep-stage variant (KS K tiles per barrier pair) of a small tile; native layout only.
+template <class S, int KS>
+static hipError_t launch_deep(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
+                              bool out_f32, hipStream_t stream) {
+  return out_f32 ? launch_tile<S, kLoopPingPong, true, KS>(W, X, C, ldc, M, N, K, stream)
+                 : launch_tile<S, kLoopPingPong, false, KS>(W, X, C, ldc, M, N, K, stream);
+}
+
 // Tile shapes. Which one runs is a pure performance choice (see det_gemm_tile.h).
 using Shape256x256 = TileShape<256, 256, 4, 2>;
 using Shape256x128 = TileShape<256, 128, 4, 2>;
@@ -223,11 +234,18 @@ static int64_t tile_count(int M, int N, int bm, int bn) {
 }
 
 int pick_det_gemm_config(int M, int N, int K) {
-  (void)K;
   constexpr int kCus = 256;
   // Decode: many short panels keep the chip busy with one wave each; few long
   // panels need the streaming kernel's deep ring.
   if (M <= 16) return N >= 64 * kCus ? RLK_GEMM_CFG_16x16 : RLK_GEMM_CFG_STREAM16_DEEP;
+  // Problems that give the chip at most one small tile per CU: the deep-stage variants
+  // (one workgroup per CU, several K tiles per barrier pair) beat the same tile run several
+  // workgroups per CU. Smallest tile first: it spreads the weight stream over most CUs.
+  if (K % (kTileK * kDeep64) == 0 && tile_count(M, N, 64, 64) <= kCus) return RLK_GEMM_CFG_64x64_DEEP;
+  if (K % (kTileK * kDeep128) == 0) {
+    if (tile_count(M, N, 64, 128) <= kCus) return RLK_GEMM_CFG_128x64_DEEP;
+    if (tile_count(M, N, 128, 128) <= kCus) return RLK_GEMM_CFG_128x128_DEEP;
+  }
   // Estimated time = (rounds of 256 workgroups) x (tile area / measured relative
   // throughput of the shape when the chip is full). Larger tiles win ties.
   struct Candidate {
@@ -300,6 +318,19 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
       return det_gemm_stream_launch(W, X, C, ldc, M, N, K, out_f32, config == RLK_GEMM_CFG_STREAM16 ? 1 : 0, stream);
     }
     config = M <= 16 ? RLK_GEMM_CFG_16x16 : pick_det_gemm_config(M, N, K);
+  }
+  // Deep-stage variants need the fast layout and whole stages; otherwise the plain shape
+  // computes the same bits.
+  if (config == RLK_GEMM_CFG_64x64_DEEP || config == RLK_GEMM_CFG_128x64_DEEP || config == RLK_GEMM_CFG_128x128_DEEP) {
+    const int ks = config == RLK_GEMM_CFG_64x64_DEEP ? kDeep64 : kDeep128;
+    if (vec && allow_pingpong && K % (kTileK * ks) == 0) {
+      if (config == RLK_GEMM_CFG_64x64_DEEP) return launch_deep<Shape64x64, kDeep64>(W, X, C, ldc, M, N, K, out_f32, stream);
+      if (config == RLK_GEMM_CFG_128x64_DEEP) return launch_deep<Shape128x64, kDeep128>(W, X, C, ldc, M, N, K, out_f32, stream);
+      return launch_deep<Shape128x128, kDeep128>(W, X, C, ldc, M, N, K, out_f32, stream);
+    }
+    config = config == RLK_GEMM_CFG_64x64_DEEP    ? RLK_GEMM_CFG_64x64
+             : config == RLK_GEMM_CFG_128x64_DEEP ? RLK_GEMM_CFG_128x64
+                                                  : RLK_GEMM_CFG_128x128;
   }
   // The element-wise loader of the generic path keeps eight values per chunk in
   // flight; the largest shapes would spill registers with it.

@@ -437,10 +437,16 @@ constexpr bool pingpong_supported() {
 
 // With WK the accumulator of MFMA tile jn holds features wave_n*64 + jn*16 + (lane>>4)*4 + q
 // (no run permutation: a K-major chunk is eight consecutive features).
-template <class S, bool WK = false, bool XK = false, class Map = PlainRowMap<S>>
+//
+// KS > 1 makes a stage KS consecutive 64-wide K tiles (each laid out as above), so a phase
+// covers 64 * KS K values between two barriers: small tiles, whose phases would otherwise be
+// shorter than a barrier, stay on the matrix pipe. Needs K % (64 * KS) == 0 and
+// 2 * KS * S::kStageBytes of LDS; the MFMA chain is the same (K tiles ascending).
+template <class S, bool WK = false, bool XK = false, class Map = PlainRowMap<S>, int KS = 1>
 __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const MatView& X, int n0, int m0, int K,
                                                        char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
   static_assert(pingpong_supported<S>(), "two groups of four waves, 4 x 2 wave layout");
+  static_assert(KS >= 1 && KS * (DmaLoader<S, WK, XK, Map>::kLateLoads) <= 31, "loads in flight must fit vmcnt");
   using Loader = DmaLoader<S, WK, XK, Map>;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -463,12 +469,22 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
   const int w_row_base = (wave_n * 16 * S::TN + l16) * kRowBytes;
   const int x_row_base = S::BN * kRowBytes + (wave_m * 16 * S::TM + l16) * kRowBytes;
 
-  const int nk = K / kTileK;
-  // Loads past the last tile re-fetch the last tile into a stage nobody reads
+  constexpr int kStageSpan = KS * S::kStageBytes;  // bytes of one stage (KS K tiles)
+  constexpr int kStageK = KS * kTileK;             // K values of one stage
+  const int nk = K / kStageK;
+  // Loads past the last stage re-fetch the last one into a stage nobody reads
   // any more; that keeps the number of loads in flight (and so every s_waitcnt
   // immediate) the same in every iteration.
-  auto tile_k = [&](int t) { return (t < nk ? t : nk - 1) * kTileK; };
-  auto stage = [&](int t) { return lds + (t & 1) * S::kStageBytes; };
+  auto tile_k = [&](int t) { return (t < nk ? t : nk - 1) * kStageK; };
+  auto stage = [&](int t) { return lds + (t & 1) * kStageSpan; };
+  auto issue_early = [&](char* st, int k0) {
+#pragma unroll
+    for (int s = 0; s < KS; ++s) loader.issue_early(st + s * S::kStageBytes, k0 + s * kTileK, wave);
+  };
+  auto issue_late = [&](char* st, int k0) {
+#pragma unroll
+    for (int s = 0; s < KS; ++s) loader.issue_late(st + s * S::kStageBytes, k0 + s * kTileK, wave);
+  };
 
   // K-major fragments: the transposing read takes, from lane r of a 16-lane group, the address
   // of 4 features (tokens) at K row (r >> 2), positions 4 (r & 3) .. +3 of MFMA tile `j16` of a
@@ -494,52 +510,58 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
     return read_kmajor(st + S::BN * kRowBytes + col * (64 * kRowBytes), jm & 3, step);
   };
 
-  u32x4_t w0[S::TN], x0[S::TM], w1[S::TN], x1[S::TM];
+  u32x4_t w0[KS][S::TN], x0[KS][S::TM], w1[KS][S::TN], x1[KS][S::TM];
   auto read_tile = [&](int t) {
-    const char* st = stage(t);
 #pragma unroll
-    for (int jm = 0; jm < S::TM; ++jm) {
-      if constexpr (XK) {
-        x0[jm] = read_x_kmajor(st, jm, 0);
-      } else {
-        x0[jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + frag_lo);
+    for (int s = 0; s < KS; ++s) {
+      const char* st = stage(t) + s * S::kStageBytes;
+#pragma unroll
+      for (int jm = 0; jm < S::TM; ++jm) {
+        if constexpr (XK) {
+          x0[s][jm] = read_x_kmajor(st, jm, 0);
+        } else {
+          x0[s][jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + frag_lo);
+        }
       }
-    }
 #pragma unroll
-    for (int jn = 0; jn < S::TN; ++jn) {
-      if constexpr (WK) {
-        w0[jn] = read_w_kmajor(st, jn, 0);
-      } else {
-        w0[jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + frag_lo);
+      for (int jn = 0; jn < S::TN; ++jn) {
+        if constexpr (WK) {
+          w0[s][jn] = read_w_kmajor(st, jn, 0);
+        } else {
+          w0[s][jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + frag_lo);
+        }
       }
-    }
 #pragma unroll
-    for (int jm = 0; jm < S::TM; ++jm) {
-      if constexpr (XK) {
-        x1[jm] = read_x_kmajor(st, jm, 1);
-      } else {
-        x1[jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + (frag_lo ^ 64));
+      for (int jm = 0; jm < S::TM; ++jm) {
+        if constexpr (XK) {
+          x1[s][jm] = read_x_kmajor(st, jm, 1);
+        } else {
+          x1[s][jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + (frag_lo ^ 64));
+        }
       }
-    }
 #pragma unroll
-    for (int jn = 0; jn < S::TN; ++jn) {
-      if constexpr (WK) {
-        w1[jn] = read_w_kmajor(st, jn, 1);
-      } else {
-        w1[jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + (frag_lo ^ 64));
+      for (int jn = 0; jn < S::TN; ++jn) {
+        if constexpr (WK) {
+          w1[s][jn] = read_w_kmajor(st, jn, 1);
+        } else {
+          w1[s][jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + (frag_lo ^ 64));
+        }
       }
     }
   };
   auto compute = [&]() {
     __builtin_amdgcn_s_setprio(2);
 #pragma unroll
-    for (int jn = 0; jn < S::TN; ++jn)
+    for (int s = 0; s < KS; ++s) {
 #pragma unroll
-      for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = mfma_16x16x32(w0[jn], x0[jm], acc[jn][jm]);
+      for (int jn = 0; jn < S::TN; ++jn)
 #pragma unroll
-    for (int jn = 0; jn < S::TN; ++jn)
+        for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = mfma_16x16x32(w0[s][jn], x0[s][jm], acc[jn][jm]);
 #pragma unroll
-      for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = mfma_16x16x32(w1[jn], x1[jm], acc[jn][jm]);
+      for (int jn = 0; jn < S::TN; ++jn)
+#pragma unroll
+        for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = mfma_16x16x32(w1[s][jn], x1[s][jm], acc[jn][jm]);
+    }
     __builtin_amdgcn_s_setprio(0);
   };
 
@@ -555,13 +577,13 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
   //   early wave, phase 2t + 2: starts its part of tile t + 2 (rows only the late
   //     group read, one phase earlier); confirms it at the end of phase 2t + 3.
   if (!late_group) {
-    loader.issue_early(stage(0), 0, wave);
-    loader.issue_early(stage(1), tile_k(1), wave);
-    __builtin_amdgcn_s_waitcnt(wait_vmcnt(Loader::kEarlyLoads));  // my part of tile 0 has landed
+    issue_early(stage(0), 0);
+    issue_early(stage(1), tile_k(1));
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt(KS * Loader::kEarlyLoads));  // my part of tile 0 has landed
     wg_barrier();
     for (int t = 0; t < nk; ++t) {
       read_tile(t);
-      if (t > 0) loader.issue_early(stage(t + 1), tile_k(t + 1), wave);
+      if (t > 0) issue_early(stage(t + 1), tile_k(t + 1));
       __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // my fragments are in registers
       wg_barrier();
       compute();
@@ -570,16 +592,16 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
     }
     wg_barrier();  // pairs with the late group's leading barrier
   } else {
-    loader.issue_late(stage(0), 0, wave);
-    loader.issue_late(stage(1), tile_k(1), wave);
-    __builtin_amdgcn_s_waitcnt(wait_vmcnt(Loader::kLateLoads));  // my part of tile 0 has landed
+    issue_late(stage(0), 0);
+    issue_late(stage(1), tile_k(1));
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt(KS * Loader::kLateLoads));  // my part of tile 0 has landed
     wg_barrier();
     wg_barrier();  // half an iteration behind the early group
     for (int t = 0; t < nk; ++t) {
       read_tile(t);
       __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // my fragments are in registers
-      loader.issue_late(stage(t), tile_k(t + 2), wave);
-      __builtin_amdgcn_s_waitcnt(wait_vmcnt(Loader::kLateLoads));  // my part of tile t+1 has landed
+      issue_late(stage(t), tile_k(t + 2));
+      __builtin_amdgcn_s_waitcnt(wait_vmcnt(KS * Loader::kLateLoads));  // my part of tile t+1 has landed
       wg_barrier();
       compute();
       wg_barrier();

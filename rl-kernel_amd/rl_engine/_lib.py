@@ -33,6 +33,9 @@ GEMM_CONFIGS = {
     "stream16_deep": 8,
     "stream16": 9,
     "256x64": 10,
+    "64x64_deep": 11,
+    "128x64_deep": 12,
+    "128x128_deep": 13,
 }
 # OR-ed into a GEMM or LogP configuration: register-staged main loop (bit-neutral).
 FORCE_STAGED = 0x100
