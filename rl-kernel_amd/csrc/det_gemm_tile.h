@@ -238,6 +238,7 @@ constexpr int kWaitVm0 = 0x0f70;     // vmcnt(0)
 constexpr int kWaitLgkm0 = 0xc07f;   // lgkmcnt(0)
 constexpr int kWaitAll0 = 0x0070;    // vmcnt(0) lgkmcnt(0)
 constexpr int wait_vmcnt(int n) { return 0x0f70 | (n & 15) | ((n >> 4) << 14); }
+constexpr int wait_lgkmcnt(int n) { return 0xc07f | ((n & 15) << 8); }  // vmcnt / expcnt left at their maxima
 
 // s_barrier without a fence; the empty asm statements only stop the compiler
 // from moving memory operations across it.
@@ -253,8 +254,12 @@ __device__ __forceinline__ void wg_barrier() {
 // [0, BM/2) and waves 4-7 token rows [BM/2, BM). A wave may overwrite a row
 // right after its own reads only if no other wave of its group reads that row
 // (a barrier orders the two groups, nothing orders the waves inside a group):
-//   late wave 4+j : the weight rows of column j, and a quarter of token rows [0, BM/2)
-//   early wave j  : a quarter of token rows [BM/2, BM)
+//   late wave 4+j : the first half of the weight blocks of column j, right after its own reads
+//                   of them, and a quarter of token rows [0, BM/2) at the start of its read phase
+//                   (the early group finished with those one phase earlier)
+//   early wave j  : the second half of the weight blocks of column j (the late wave read them one
+//                   phase earlier, behind a barrier) and a quarter of token rows [BM/2, BM)
+// so both groups issue the same number of loads and neither read phase outlasts a compute phase.
 // For a block inside the matrix the 64 lane addresses are a uniform block base
 // plus a per-lane offset that is the same for every block, so a wave keeps a few
 // 32-bit lane offsets instead of one pointer per block; a block that crosses the
@@ -319,10 +324,16 @@ struct DmaLoader {
   static constexpr int kWaveRows = 16 * S::TN;
   static_assert(!WK || S::TN == 4, "K-major weights need 64-feature wave columns");
   static_assert(!XK || S::BM % 128 == 0, "K-major activations need whole 64-token columns per wave group");
-  static constexpr int kWBlocksPerWave = kWaveRows / 8;     // late waves only
+  static constexpr int kWBlocksPerWave = kWaveRows / 8;     // blocks of one weight column
+  // Native layout: the two waves that read a weight column split its refill. K-major operands
+  // (twice as many, transposing, fragment reads per phase) measured faster with the whole column
+  // refilled by the late wave after all of its reads.
+  static constexpr bool kSplitColumn = !WK && !XK;
+  static constexpr int kWBlocksLate = kSplitColumn ? kWBlocksPerWave / 2 : kWBlocksPerWave;
+  static constexpr int kWBlocksEarly = kWBlocksPerWave - kWBlocksLate;
   static constexpr int kXBlocksPerWave = (S::BM / 16) / 4;  // every wave
-  static constexpr int kLateLoads = kWBlocksPerWave + kXBlocksPerWave;
-  static constexpr int kEarlyLoads = kXBlocksPerWave;
+  static constexpr int kLateLoads = kWBlocksLate + kXBlocksPerWave;
+  static constexpr int kEarlyLoads = kWBlocksEarly + kXBlocksPerWave;
   static constexpr int kBlocksW = S::BN / 8;
 
   const bf16_bits* w_base;  // W + n0 * ldw   (uniform)
@@ -419,14 +430,19 @@ struct DmaLoader {
   // `wave` is the workgroup wave index 0..7.
   __device__ __forceinline__ void issue_early(char* stage, int k0, int wave) const {
 #pragma unroll
+    for (int j = kWBlocksLate; j < kWBlocksPerWave; ++j) load_w_block(stage, k0, wave * kWBlocksPerWave + j);
+#pragma unroll
     for (int j = 0; j < kXBlocksPerWave; ++j) load_x_block(stage, k0, S::BM / 16 + wave * kXBlocksPerWave + j);
   }
-  __device__ __forceinline__ void issue_late(char* stage, int k0, int wave) const {
+  __device__ __forceinline__ void issue_late_x(char* stage, int k0, int wave) const {
     const int col = wave - 4;
 #pragma unroll
-    for (int j = 0; j < kWBlocksPerWave; ++j) load_w_block(stage, k0, col * kWBlocksPerWave + j);
-#pragma unroll
     for (int j = 0; j < kXBlocksPerWave; ++j) load_x_block(stage, k0, col * kXBlocksPerWave + j);
+  }
+  __device__ __forceinline__ void issue_late_w(char* stage, int k0, int wave) const {
+    const int col = wave - 4;
+#pragma unroll
+    for (int j = 0; j < kWBlocksLate; ++j) load_w_block(stage, k0, col * kWBlocksPerWave + j);
   }
 };
 
@@ -481,9 +497,13 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
 #pragma unroll
     for (int s = 0; s < KS; ++s) loader.issue_early(st + s * S::kStageBytes, k0 + s * kTileK, wave);
   };
-  auto issue_late = [&](char* st, int k0) {
+  auto issue_late_x = [&](char* st, int k0) {
 #pragma unroll
-    for (int s = 0; s < KS; ++s) loader.issue_late(st + s * S::kStageBytes, k0 + s * kTileK, wave);
+    for (int s = 0; s < KS; ++s) loader.issue_late_x(st + s * S::kStageBytes, k0 + s * kTileK, wave);
+  };
+  auto issue_late_w = [&](char* st, int k0) {
+#pragma unroll
+    for (int s = 0; s < KS; ++s) loader.issue_late_w(st + s * S::kStageBytes, k0 + s * kTileK, wave);
   };
 
   // K-major fragments: the transposing read takes, from lane r of a 16-lane group, the address
@@ -511,43 +531,48 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
   };
 
   u32x4_t w0[KS][S::TN], x0[KS][S::TM], w1[KS][S::TN], x1[KS][S::TM];
-  auto read_tile = [&](int t) {
+  // Weight fragments of both K steps (2 TN KS reads) ...
+  auto read_w = [&](int t) {
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const char* st = stage(t) + s * S::kStageBytes;
+#pragma unroll
+      for (int jn = 0; jn < S::TN; ++jn) {
+        if constexpr (WK) {
+          w0[s][jn] = read_w_kmajor(st, jn, 0);
+          w1[s][jn] = read_w_kmajor(st, jn, 1);
+        } else {
+          w0[s][jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + frag_lo);
+          w1[s][jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + (frag_lo ^ 64));
+        }
+      }
+    }
+  };
+  // ... and the token fragments of one K step (TM KS reads).
+  auto read_x = [&](int t, int step) {
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const char* st = stage(t) + s * S::kStageBytes;
 #pragma unroll
       for (int jm = 0; jm < S::TM; ++jm) {
+        u32x4_t v;
         if constexpr (XK) {
-          x0[s][jm] = read_x_kmajor(st, jm, 0);
+          v = read_x_kmajor(st, jm, step);
         } else {
-          x0[s][jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + frag_lo);
+          v = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + (frag_lo ^ (step << 6)));
         }
-      }
-#pragma unroll
-      for (int jn = 0; jn < S::TN; ++jn) {
-        if constexpr (WK) {
-          w0[s][jn] = read_w_kmajor(st, jn, 0);
+        if (step == 0) {
+          x0[s][jm] = v;
         } else {
-          w0[s][jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + frag_lo);
-        }
-      }
-#pragma unroll
-      for (int jm = 0; jm < S::TM; ++jm) {
-        if constexpr (XK) {
-          x1[s][jm] = read_x_kmajor(st, jm, 1);
-        } else {
-          x1[s][jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + (frag_lo ^ 64));
-        }
-      }
-#pragma unroll
-      for (int jn = 0; jn < S::TN; ++jn) {
-        if constexpr (WK) {
-          w1[s][jn] = read_w_kmajor(st, jn, 1);
-        } else {
-          w1[s][jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + (frag_lo ^ 64));
+          x1[s][jm] = v;
         }
       }
     }
+  };
+  auto read_tile = [&](int t) {
+    read_w(t);
+    read_x(t, 0);
+    read_x(t, 1);
   };
   auto compute = [&]() {
     __builtin_amdgcn_s_setprio(2);
@@ -571,11 +596,12 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
   // Tile t lives in stage t & 1, which is read in phases 2t and 2t + 1 and first
   // read again (tile t + 2) in phase 2t + 4. Every wave waits for its own
   // fragment reads before the barrier that ends its read phase.
-  //   late wave, phase 2t + 1: after its own reads, starts its part of tile t + 2
-  //     (rows only it and, one phase earlier, the early group read); it confirms
-  //     that part at the end of phase 2t + 3, behind the loads it starts there.
-  //   early wave, phase 2t + 2: starts its part of tile t + 2 (rows only the late
-  //     group read, one phase earlier); confirms it at the end of phase 2t + 3.
+  //   late wave, phase 2t + 1: starts its token rows of tile t + 2 at once (the early group
+  //     read them one phase earlier) and its weight blocks as soon as its own weight
+  //     fragments are in registers; it confirms that part at the end of phase 2t + 3,
+  //     behind the loads it starts there.
+  //   early wave, phase 2t + 2: starts its part of tile t + 2 (rows the late group read one
+  //     phase earlier); confirms it at the end of phase 2t + 3.
   if (!late_group) {
     issue_early(stage(0), 0);
     issue_early(stage(1), tile_k(1));
@@ -592,15 +618,32 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
     }
     wg_barrier();  // pairs with the late group's leading barrier
   } else {
-    issue_late(stage(0), 0);
-    issue_late(stage(1), tile_k(1));
+    issue_late_x(stage(0), 0);
+    issue_late_w(stage(0), 0);
+    issue_late_x(stage(1), tile_k(1));
+    issue_late_w(stage(1), tile_k(1));
     __builtin_amdgcn_s_waitcnt(wait_vmcnt(KS * Loader::kLateLoads));  // my part of tile 0 has landed
     wg_barrier();
     wg_barrier();  // half an iteration behind the early group
+    // LDS reads return in order, so once at most kXReads of them are outstanding the weight
+    // fragments (issued first) are in registers and their rows may be refilled.
+    // (lgkmcnt is a 4-bit counter, so this needs at most 15 token reads per K step.)
+    constexpr int kXReads = KS * S::TM * (XK ? 2 : 1);
     for (int t = 0; t < nk; ++t) {
-      read_tile(t);
-      __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // my fragments are in registers
-      issue_late(stage(t), tile_k(t + 2));
+      if constexpr (Loader::kSplitColumn && kXReads <= 15) {
+        issue_late_x(stage(t), tile_k(t + 2));  // token rows the early group read one phase ago
+        read_w(t);
+        read_x(t, 0);
+        __builtin_amdgcn_s_waitcnt(wait_lgkmcnt(kXReads));  // my weight fragments are in registers
+        issue_late_w(stage(t), tile_k(t + 2));
+        read_x(t, 1);
+      } else {
+        read_tile(t);
+        __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
+        issue_late_w(stage(t), tile_k(t + 2));
+        issue_late_x(stage(t), tile_k(t + 2));
+      }
+      __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // all my fragments are in registers
       __builtin_amdgcn_s_waitcnt(wait_vmcnt(KS * Loader::kLateLoads));  // my part of tile t+1 has landed
       wg_barrier();
       compute();
