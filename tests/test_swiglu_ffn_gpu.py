@@ -167,3 +167,49 @@ def test_argument_errors(native, ffn_mod):
         ffn_mod.qwen3_ffn(x[:0], w, w, wd)
     with pytest.raises(RuntimeError, match="deterministic FFN only"):
         ffn_mod.qwen3_ffn(x, w, w, wd, deterministic=False)
+
+
+@pytest.mark.parametrize("rows", [8, 64, 300])
+def test_ffn_and_logp_stages_replay_bit_identically_in_a_hip_graph(native, ffn_mod, rows):
+    """The rollout path is captured once and replayed against capture-time addresses: the FFN
+    (fused gate/up + SwiGLU, then down into a staging buffer), the LogP-from-logits stage and the
+    fused linear-LogP must give the eager bits on every replay (eager work and synchronisations
+    in between)."""
+    # (the `_C` layer: the Python entry points above it validate targets on the host, which a
+    # capture does not allow; the reference's wrapper has a `targets_validated` switch for this)
+    h, inter, vocab = 256, 384, 2048
+    x = inputs.randn_bf16(8500, rows, h).to(DEV)
+    w_gu = inputs.randn_bf16(8501, 2 * inter, h, 0.1).to(DEV)
+    w_d = inputs.randn_bf16(8502, h, inter, 0.1).to(DEV)
+    w_lm = inputs.randn_bf16(8503, vocab, h, 0.1).to(DEV)
+    target = torch.randint(0, vocab, (rows,), generator=torch.Generator().manual_seed(8504)).to(DEV)
+    staging = torch.zeros((rows, h), dtype=torch.bfloat16, device=DEV)
+
+    def step():
+        torch.ops.rl_kernel.qwen3_ffn_packed_inference_to_staging(x, w_gu, w_d, staging)
+        logp, lse, logits = native.fused_linear_logp(staging, w_lm, target, None, None, True)
+        logp2, _ = native.hip_deterministic_logp_from_logits(logits, target, 0, vocab, 64)
+        return logp, lse, logp2
+
+    with torch.no_grad():
+        eager = [t.clone() for t in step()]
+        eager_staging = staging.clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()  # warm-up outside capture
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            captured = step()
+        for _ in range(3):
+            staging.zero_()
+            for t in captured:
+                t.zero_()
+            native.swiglu_forward(x, x)  # unrelated eager work between replays
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert _same_bits(staging, eager_staging)
+            for got, want in zip(captured, eager):
+                assert torch.equal(got.view(torch.int32), want.view(torch.int32))
