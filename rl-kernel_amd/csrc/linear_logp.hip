@@ -285,9 +285,11 @@ static hipError_t launch_logp(LogpArgs a, hipStream_t stream) {
 
 int pick_linear_logp_config(int T, int V) {
   (void)V;
-  if (T <= 16) return RLK_LOGP_CFG_16;
+  // Measured at V = 151936, D = 4096: the 64-token tile (two workgroups per CU, direct-to-LDS
+  // loop) is the fastest from decode sizes up to 64 tokens, the 256-token tile from 256 tokens on
+  // even where it leaves the last round of workgroups part empty.
   if (T <= 64) return RLK_LOGP_CFG_64;
-  if (T <= 2048) return RLK_LOGP_CFG_128;
+  if (T <= 128) return RLK_LOGP_CFG_128;
   return RLK_LOGP_CFG_256;
 }
 
