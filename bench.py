@@ -42,7 +42,7 @@ HIDDEN, INTER, VOCAB = 4096, 12288, 151936
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs of this script (profiles/det_gemm_gate_up_T4096_pmc.md), scaled
 # by the same counters read on a plain device copy of known size. None = not measured.
-MEASURED_TRAFFIC_BYTES = {"det_gemm_gate_up_T4096": 1.412e9}  # 1.209 GB fetched + 0.203 GB written
+MEASURED_TRAFFIC_BYTES = {"det_gemm_gate_up_T4096": 1.417e9}  # 1.212 GB fetched + 0.205 GB written
 
 
 def _parse():
