@@ -223,3 +223,68 @@ def test_backward_argument_errors(native):
         dev["h"][:0], dev["w"], dev["target"][:0], lse[:0], dev["g_logp"][:0], None, need_grad_bias=False
     )
     assert tuple(empty[0].shape) == (0, 64) and not bool(empty[1].any())
+
+
+# ---------------------------------------------------------------------------
+# Full size (T = 8192, V = 151936, D = 4096): size-independent properties and sampled parity
+# ---------------------------------------------------------------------------
+
+
+def test_full_size_backward_properties_and_sampled_parity(native, oracle):
+    h, w, target = inputs.logp_inputs(8192)
+    t, v, d = 8192, w.size(0), w.size(1)
+    gen = torch.Generator().manual_seed(5701)
+    g_logp = torch.randn(t, generator=gen)
+    g_lse = torch.randn(t, generator=gen) * 0.25
+    bias = torch.randn(v, generator=gen) * 0.1
+    hd, wd, td, bd = h.to(DEV), w.to(DEV), target.to(DEV), bias.to(DEV)
+    _, lse = native.fused_linear_logp(hd, wd, td, bd)
+    gh, gw, gb = native.fused_linear_logp_bwd(hd, wd, td, lse, g_logp.to(DEV), g_lse.to(DEV), bd, need_grad_bias=True)
+    assert tuple(gh.shape) == (t, d) and tuple(gw.shape) == (v, d) and tuple(gb.shape) == (v,)
+    assert bool(torch.isfinite(gh.float()).all()) and bool(torch.isfinite(gw.float()).all())
+    # run to run: every output bit
+    gh2, gw2, gb2 = native.fused_linear_logp_bwd(hd, wd, td, lse, g_logp.to(DEV), g_lse.to(DEV), bd, need_grad_bias=True)
+    assert torch.equal(_bits16(gh), _bits16(gh2)) and torch.equal(_bits16(gw), _bits16(gw2)) and torch.equal(gb, gb2)
+    # rows of grad_hidden are bit-identical at M = 1, M = 7, a ragged cut and another packing
+    for lo, hi in ((0, 1), (0, 7), (8191, 8192), (5000, 5130)):
+        part, _, _ = native.fused_linear_logp_bwd(
+            hd[lo:hi], wd, td[lo:hi], lse[lo:hi], g_logp[lo:hi].to(DEV), g_lse[lo:hi].to(DEV), bd, need_grad_weight=False
+        )
+        assert torch.equal(_bits16(part), _bits16(gh[lo:hi])), (lo, hi)
+    perm = torch.randperm(t, generator=torch.Generator().manual_seed(5702)).to(DEV)
+    packed, _, _ = native.fused_linear_logp_bwd(
+        hd[perm], wd, td[perm], lse[perm], g_logp.to(DEV)[perm], g_lse.to(DEV)[perm], bd, need_grad_weight=False
+    )
+    assert torch.equal(_bits16(packed), _bits16(gh[perm]))
+    # probabilities sum to one: the bias gradient summed over the vocabulary is sum_t g_lse[t]
+    expect = float(g_lse.double().sum())
+    scale = float(g_logp.abs().double().sum() * 2 + g_lse.abs().double().sum())
+    assert abs(float(gb.double().sum()) - expect) <= 2.0**-8 * scale
+    # sampled parity: four token rows of grad_hidden and six vocabulary rows of grad_weight
+    lse64 = lse.double().cpu().numpy()
+    hb, wb = inputs.bits(h), inputs.bits(w)
+    rows = np.array([0, 1777, 4096, 8191])
+    dz = oracle.linear_logp_dlogits(
+        hb[rows], wb, target.numpy()[rows], lse64[rows], g_logp.numpy()[rows], g_lse.numpy()[rows], bias.numpy(),
+        dtype=np.float64,
+    )  # fmt: skip
+    wf = oracle.bf16_to_f32(wb).astype(np.float64)
+    want = dz @ wf
+    bound = 2.0**-8 * np.abs(want) + (2.0**-8 + v * 2.0**-24 + 2e-5) * (np.abs(dz) @ np.abs(wf)) + 1e-30
+    got = gh[torch.from_numpy(rows).to(DEV)].double().cpu().numpy()
+    assert float((np.abs(got - want) / bound).max()) <= 1.0
+    cols = np.array([0, 1, 70000, 151935] + [int(target[5]), int(target[4096])])
+    hf = oracle.bf16_to_f32(hb).astype(np.float64)
+    z = hf @ wf[cols].T + bias.numpy().astype(np.float64)[cols]  # [T, 6] logits of the sampled columns
+    p = np.exp(z - lse64[:, None])
+    dz_cols = p * (g_lse.numpy().astype(np.float64) - g_logp.numpy().astype(np.float64))[:, None]
+    for j, col in enumerate(cols):
+        hit = target.numpy() == col
+        dz_cols[hit, j] += g_logp.numpy().astype(np.float64)[hit]
+    want_w = dz_cols.T @ hf
+    bound_w = 2.0**-8 * np.abs(want_w) + (2.0**-8 + t * 2.0**-24 + 2e-5) * (np.abs(dz_cols).T @ np.abs(hf)) + 1e-30
+    got_w = gw[torch.from_numpy(cols).to(DEV)].double().cpu().numpy()
+    assert float((np.abs(got_w - want_w) / bound_w).max()) <= 1.0
+    want_b = dz_cols.sum(axis=0)
+    got_b = gb[torch.from_numpy(cols).to(DEV)].double().cpu().numpy()
+    assert np.all(np.abs(got_b - want_b) <= (2.0**-8 + t * 2.0**-24 + 2e-5) * np.abs(dz_cols).sum(axis=0) + 1e-30)

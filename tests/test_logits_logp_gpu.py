@@ -150,3 +150,25 @@ def test_argument_errors(native, logp_mod):
         )  # fmt: skip
     empty = native.hip_deterministic_logp_tile_stats(z[:0], 0, 64, 8)
     assert tuple(empty[0].shape) == (0, 8)
+
+
+def test_full_size_rows_are_batch_invariant_and_normalised(native, logp_mod):
+    """bf16 logits [8192, 151936] (2.5 GB): a row's (logp, lse) has the same bits alone, in a cut and
+    in another packing; exp(logp) over every target id of a row sums to one."""
+    rows, v = 8192, 151936
+    gen = torch.Generator(device=DEV).manual_seed(7400)
+    z = torch.empty((rows, v), dtype=torch.bfloat16, device=DEV)
+    for r0 in range(0, rows, 1024):
+        z[r0 : r0 + 1024] = (torch.randn((1024, v), generator=gen, device=DEV) * 3).to(torch.bfloat16)
+    target = torch.randint(0, v, (rows,), generator=gen, device=DEV)
+    logp, lse = logp_mod.deterministic_logp_from_logits(z, target)
+    assert bool(torch.isfinite(logp).all()) and bool((logp <= 1e-6).all())
+    for lo, hi in ((0, 1), (4095, 4102), (8191, 8192)):
+        part = logp_mod.deterministic_logp_from_logits(z[lo:hi], target[lo:hi])
+        assert torch.equal(part[0].view(torch.int32), logp[lo:hi].view(torch.int32))
+        assert torch.equal(part[1].view(torch.int32), lse[lo:hi].view(torch.int32))
+    perm = torch.randperm(rows, generator=torch.Generator().manual_seed(7401))[:512].to(DEV)
+    packed = logp_mod.deterministic_logp_from_logits(z[perm], target[perm])
+    assert torch.equal(packed[0].view(torch.int32), logp[perm].view(torch.int32))
+    total = (z[77].float() - lse[77]).double().exp().sum()
+    assert abs(float(total) - 1.0) < 1e-4
