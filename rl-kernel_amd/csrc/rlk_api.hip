@@ -159,15 +159,21 @@ int rlk_linear_logp_bwd(const void* hidden, int64_t h_row_stride, const void* we
     set_last_error("rlk_linear_logp_bwd: unknown config %d", config);
     return RLK_ERR_INVALID_ARGUMENT;
   }
-  if (hidden == nullptr || weight == nullptr || (T > 0 && (target == nullptr || lse == nullptr))) {
-    set_last_error("rlk_linear_logp_bwd: null hidden / weight / target / lse");
-    return RLK_ERR_INVALID_ARGUMENT;
-  }
-  if (h_row_stride < D || w_row_stride < D || (grad_hidden && gh_row_stride < D) || (grad_weight && gw_row_stride < D)) {
-    set_last_error("rlk_linear_logp_bwd: row strides must be >= D");
+  if ((grad_hidden && gh_row_stride < D) || (grad_weight && gw_row_stride < D)) {
+    set_last_error("rlk_linear_logp_bwd: gradient row strides must be >= D");
     return RLK_ERR_INVALID_ARGUMENT;
   }
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (T > 0) {
+    if (hidden == nullptr || weight == nullptr || target == nullptr || lse == nullptr) {
+      set_last_error("rlk_linear_logp_bwd: null hidden / weight / target / lse");
+      return RLK_ERR_INVALID_ARGUMENT;
+    }
+    if (h_row_stride < D || w_row_stride < D) {
+      set_last_error("rlk_linear_logp_bwd: row strides must be >= D");
+      return RLK_ERR_INVALID_ARGUMENT;
+    }
+  }
   if (T == 0) {
     // No tokens: the token-summed gradients are zero.
     hipError_t err = hipSuccess;
