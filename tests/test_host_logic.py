@@ -204,3 +204,27 @@ def test_ctypes_prototypes_cover_every_argument(rlk_lib):
         params = re.search(name + r"\s*\((.*?)\)\s*;", text, flags=re.S).group(1)
         assert len(getattr(rlk_lib, name).argtypes) == params.count(",") + 1, name
     assert rlk_lib.rlk_linear_logp_workspace_bytes.restype is ctypes.c_size_t
+
+
+def test_linear_logp_wrapper_contract_errors_without_a_gpu():
+    """Shape / dtype / placement rules of the engine-facing wrapper are checked before any GPU work."""
+    import torch
+
+    from rl_engine.integrations.common.linear_logp import LinearLogpWrapper
+
+    wrapper = LinearLogpWrapper()
+    ids = torch.zeros(2, dtype=torch.long)
+    with pytest.raises(ValueError, match=r"expects hidden \[tokens, hidden\]"):
+        wrapper(torch.zeros(3), torch.zeros(2, 3), ids)
+    with pytest.raises(RuntimeError, match="requires CUDA/ROCm GPU tensors"):
+        wrapper(torch.zeros(2, 3, dtype=torch.bfloat16), torch.zeros(4, 3, dtype=torch.bfloat16), ids)
+    with pytest.raises(TypeError, match="2-D bf16/fp16/fp32"):
+        wrapper.from_local_logits(torch.zeros(2, 8, dtype=torch.float64), ids, tp_group=None, vocab_start_index=0, global_vocab_size=8, real_vocab_size=8)
+    with pytest.raises(ValueError, match="temperature must be positive"):
+        LinearLogpWrapper._temperature_tensor(0.0, rows=2, device=torch.device("cpu"))
+    assert LinearLogpWrapper._temperature_tensor(1.0, rows=2, device=torch.device("cpu")) is None
+    with pytest.raises(ValueError, match=r"target_ids must be in \[0, 4\)"):
+        LinearLogpWrapper._validate_targets(torch.tensor([0, 4]), rows=2, real_vocab_size=4)
+    with pytest.raises(TypeError, match="integer dtype"):
+        LinearLogpWrapper._validate_targets(torch.tensor([0.0, 1.0]), rows=2, real_vocab_size=4)
+    assert wrapper.provenance == {}

@@ -297,3 +297,70 @@ def test_config5_rollout_scale(logp_mod, loss_mod, oracle, config4):
         assert float(out.loss) == pytest.approx(float(e_loss), rel=1e-4, abs=1e-6)
         rerun = loss_mod.grpo_ratio_kl_loss(lp2d, old.view(rollouts, per).to(DEV), ref.view(rollouts, per).to(DEV), adv.to(DEV), clip_eps=0.2, beta=beta)
         assert _same_bits(rerun.loss.reshape(1), out.loss.reshape(1))
+
+
+# ---------------------------------------------------------------------------
+# Engine-facing wrapper
+# ---------------------------------------------------------------------------
+
+
+def test_linear_logp_wrapper_entries(logp_mod):
+    from rl_engine.integrations.common.linear_logp import LinearLogpWrapper
+
+    h, w, target = inputs.logp_inputs(48, vocab=4096, hidden=256, seed=4600, rms_norm=False)
+    hd, wd, td = h.to(DEV), w.to(DEV), target.to(DEV) % 4000
+    wrapper = LinearLogpWrapper()
+    temp = torch.rand(48, generator=torch.Generator().manual_seed(4601)).to(DEV) + 0.5
+    out = wrapper(hd, wd, td, real_vocab_size=4000, temperature=temp, target="rollout")
+    want, lse = logp_mod.deterministic_linear_logp(hd, wd, td, temperature=temp, real_vocab_size=4000)
+    assert out.dtype == torch.float32 and _same_bits(out, want)
+    prov = wrapper.provenance
+    assert prov["deterministic_linear_logp"] is True and prov["real_vocab_size"] == 4000 and prov["target"] == "rollout"
+    assert prov["logits_materialized"] is False and prov["hidden_shape"] == [48, 256]
+    assert _same_bits(wrapper(hd, wd, td, real_vocab_size=4000, temperature=1.0), logp_mod.deterministic_linear_logp(hd, wd, td, real_vocab_size=4000)[0])
+    # reused logits: same numbers as the from-logits operator, lse on request
+    _, _, logits = logp_mod.deterministic_linear_logp(hd, wd, td, return_logits=True)
+    got, got_lse = wrapper.from_local_logits(
+        logits, td, tp_group=None, vocab_start_index=0, global_vocab_size=4096, real_vocab_size=4000, return_lse=True
+    )
+    ref = logp_mod.deterministic_logp_from_logits(logits, td, real_vocab_size=4000)
+    assert _same_bits(got, ref[0]) and _same_bits(got_lse, ref[1])
+    assert wrapper.provenance["lm_head_result_reused"] is True
+    # training: gradients flow through the wrapper
+    hg = hd.clone().requires_grad_(True)
+    wrapper(hg, wd, td).sum().backward()
+    assert hg.grad is not None and hg.grad.dtype == torch.bfloat16
+    # contract errors keep the reference's wording
+    with pytest.raises(ValueError, match="complete local vocab at offset zero"):
+        wrapper(hd, wd, td, vocab_start_index=8)
+    with pytest.raises(ValueError, match="real_vocab_size must be in"):
+        wrapper(hd, wd, td, real_vocab_size=5000)
+    with pytest.raises(TypeError, match="bfloat16 hidden and LM-head"):
+        wrapper(hd.float(), wd, td)
+    with pytest.raises(ValueError, match="equal rank-ordered TP shards"):
+        wrapper.from_local_logits(logits, td, tp_group=None, vocab_start_index=0, global_vocab_size=8192, real_vocab_size=4000)
+
+
+def test_linear_logp_wrapper_is_graph_capturable():
+    """No host synchronisation on the call path: value checks are device-side assertions."""
+    from rl_engine.integrations.common.linear_logp import LinearLogpWrapper
+
+    h, w, target = inputs.logp_inputs(16, vocab=2048, hidden=128, seed=4700, rms_norm=False)
+    hd, wd, td = h.to(DEV), w.to(DEV), target.to(DEV)
+    wrapper = LinearLogpWrapper()
+    with torch.no_grad():
+        eager = wrapper(hd, wd, td, temperature=0.7).clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            wrapper(hd, wd, td, temperature=0.7)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            captured = wrapper(hd, wd, td, temperature=0.7)
+        for _ in range(3):
+            captured.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert _same_bits(captured, eager)
