@@ -102,7 +102,8 @@ typedef enum rlk_logp_config {
   RLK_LOGP_CFG_128 = 2,
   RLK_LOGP_CFG_64 = 3,
   RLK_LOGP_CFG_16 = 4,
-  RLK_LOGP_CFG_COUNT = 5,
+  RLK_LOGP_CFG_64_STREAMS = 5, /* <= 64 tokens: four workgroups per vocabulary split, four streams each */
+  RLK_LOGP_CFG_COUNT = 6,
   /* OR-ed into a configuration: register-staged main loop instead of the
    * direct-to-LDS ping-pong loop (bit-neutral; for tests). */
   RLK_LOGP_CFG_FORCE_STAGED = 0x100
@@ -118,7 +119,8 @@ const char* rlk_linear_logp_contract_id(void);
  * (linear_logp.py:274; csrc/cuda/logprob/fused_linear_logp_sm90.cu:50, 2120-2124). */
 int rlk_linear_logp_split_count(int V);
 
-/* Bytes of fp32 partials rlk_linear_logp_fwd needs for T tokens and V vocabulary rows. */
+/* Bytes of fp32 partials rlk_linear_logp_fwd needs for T tokens and V vocabulary rows
+ * (3 * splits * T floats; 17 times that for T <= 64, where per-stream states are staged). */
 size_t rlk_linear_logp_workspace_bytes(int T, int V);
 
 /*

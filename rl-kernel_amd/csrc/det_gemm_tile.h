@@ -318,6 +318,24 @@ struct GatedRowMap {
   }
 };
 
+// StridedColumnRowMap<S, STRIDE>: wave column c of the stage holds the 64 weight rows that
+// start STRIDE * c after the tile origin (same order inside a column as PlainRowMap), so one
+// workgroup covers a 64-row slice of four blocks of rows STRIDE apart.
+template <class S, int STRIDE>
+struct StridedColumnRowMap {
+  static_assert(S::TN == 4, "64-row wave columns");
+  static constexpr bool kGated = false;
+  static __device__ __forceinline__ int block_offset(int b) {
+    const int r0 = b * 8;
+    return (r0 / 64) * STRIDE + ((r0 % 64) / 16) * 4;
+  }
+  static __device__ __forceinline__ int block_half(int) { return 0; }
+  static __device__ __forceinline__ int lane_offset(int parity, int rib) {
+    const int i = parity * 8 + rib;
+    return (i >> 2) * S::kRun + (i & 3);
+  }
+};
+
 template <class S, bool WK = false, bool XK = false, class Map = PlainRowMap<S>>
 struct DmaLoader {
   static_assert(!(WK && Map::kGated), "the gated row map is for the native weight layout");

@@ -170,6 +170,134 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_partial_kernel(LogpAr
   }
 }
 
+// Small token counts (one 64-token tile): a split of 1024 columns gives the chip only
+// ceil(V / 1024) workgroups. Streams are independent until the stream merge, so here a
+// workgroup takes four of the sixteen streams of a split, i.e. the 64-column slice
+// [64 g, 64 g + 64) of each of the split's four tiles, as ONE 256-row GEMM tile (wave column t
+// holds tile t's slice): four times the workgroups, one K loop each. The per-tile scaled
+// logits go through LDS to the threads that run the same ascending online chain over the four
+// tiles; per-(split, stream) states are merged by linear_logp_stream_merge_kernel with the
+// arithmetic of the in-kernel stream merge above. Same bits as every other configuration.
+template <class S>
+__global__ __launch_bounds__(S::kThreads) void linear_logp_streamgroup_kernel(LogpArgs a, float* __restrict__ spart) {
+  static_assert(S::BN == kLogpTileCols && S::kRun == 16 && S::WN == 4 && S::TM == 2, "256 x 64 tile, 4 x 2 waves");
+  constexpr int kGroups = kLogpStreams / 4;  // stream groups per split
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int total = a.tiles_m * a.n_split * kGroups;
+  const int id = xcd_compact_id(blockIdx.x, total);
+  const int tile_m = id % a.tiles_m;
+  const int unit = id / a.tiles_m;
+  const int split = unit / kGroups;
+  const int sg = unit % kGroups;
+  const int m0 = tile_m * S::BM;
+  const int n0 = split * kLogpSplitCols + sg * 64;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int tile = wave % S::WN;  // wave column = tile of the split
+  const int wave_m = wave / S::WN;
+  const int l16 = lane & 15;
+  const int grp = lane >> 4;  // stream inside the group
+
+  f32x4_t acc[S::TN][S::TM];
+  tile_mainloop_pingpong<S, false, false, StridedColumnRowMap<S, kLogpTileCols>>(a.W, a.H, n0, m0, a.D, lds, acc);
+
+  // Scaled logits of this lane's (token, tile, stream) into LDS: ybuf[tile][stream][token][16].
+  float* ybuf = reinterpret_cast<float*>(lds);
+  {
+    const int col0 = n0 + tile * kLogpTileCols + grp * 16;
+    float bias_run[16];
+#pragma unroll
+    for (int c = 0; c < 16; ++c) bias_run[c] = (a.bias && col0 + c < a.V) ? a.bias[col0 + c] : 0.f;
+#pragma unroll
+    for (int jm = 0; jm < S::TM; ++jm) {
+      const int tok = wave_m * 16 * S::TM + jm * 16 + l16;
+      const int m = m0 + tok;
+      const float inv_t = (a.temperature && m < a.T) ? 1.0f / a.temperature[m] : 1.0f;
+      float* dst = ybuf + ((tile * 4 + grp) * S::BM + tok) * 16;
+#pragma unroll
+      for (int c = 0; c < 16; ++c)
+        dst[c] = scaled_logit(acc[c >> 2][jm][c & 3], a.bias != nullptr, bias_run[c], col0 + c, a.vocab_limit,
+                              a.temperature != nullptr, inv_t);
+    }
+  }
+  __syncthreads();
+
+  // One thread per (stream of the group, token): the chain over the split's tiles, ascending.
+  if (threadIdx.x < 4 * S::BM) {
+    const int sl = threadIdx.x / S::BM;
+    const int tok = threadIdx.x % S::BM;
+    const int m = m0 + tok;
+    if (m < a.T) {
+      const int64_t local = a.target[m] - a.vocab_start;
+      const int tgt = (local >= 0 && local < a.vocab_limit) ? (int)local : -1;
+      float run_m = kNegInf, run_s = 0.f, run_zt = 0.f;
+      for (int t = 0; t < kLogpSplitTiles; ++t) {
+        const int v0 = split * kLogpSplitCols + t * kLogpTileCols;
+        if (v0 >= a.V) break;
+        const int col0 = v0 + (sg * 4 + sl) * 16;
+        const float* src = ybuf + ((t * 4 + sl) * S::BM + tok) * 16;
+        float y[16];
+        float tmax = kNegInf;
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+          y[c] = src[c];
+          tmax = fmaxf(tmax, y[c]);
+        }
+        const int tl = tgt - col0;
+        if (tl >= 0 && tl < 16) {
+          float sel = y[0];
+#pragma unroll
+          for (int c = 1; c < 16; ++c) sel = (tl == c) ? y[c] : sel;
+          run_zt = sel;
+        }
+        const float old_m = run_m;
+        const float new_m = fmaxf(old_m, tmax);
+        float sum = pinned_exp(y[0] - new_m);
+#pragma unroll
+        for (int c = 1; c < 16; ++c) sum = sum + pinned_exp(y[c] - new_m);
+        const float scaled = run_s * pinned_exp(old_m - new_m);
+        run_s = (new_m > kNegInf) ? (scaled + sum) : run_s;
+        run_m = new_m;
+      }
+      const int64_t plane = (int64_t)a.n_split * kLogpStreams * a.T;
+      const int64_t at = ((int64_t)split * kLogpStreams + sg * 4 + sl) * a.T + m;
+      spart[at] = run_m;
+      spart[plane + at] = run_s;
+      spart[2 * plane + at] = run_zt;
+    }
+  }
+}
+
+// Per-(split, stream) states [3][n_split * 16][T] -> per-split partials [3][n_split][T], streams
+// ascending: the arithmetic of the stream merge at the end of linear_logp_partial_kernel.
+__global__ __launch_bounds__(256) void linear_logp_stream_merge_kernel(const float* __restrict__ spart,
+                                                                      float* __restrict__ part, int T, int n_split) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= T * n_split) return;
+  const int m = idx % T;
+  const int split = idx / T;
+  const int64_t splane = (int64_t)n_split * kLogpStreams * T;
+  const float* xm = spart + (int64_t)split * kLogpStreams * T + m;
+  float big = kNegInf;
+#pragma unroll
+  for (int j = 0; j < kLogpStreams; ++j) big = fmaxf(big, xm[(int64_t)j * T]);
+  float sum = 0.f, zt = 0.f;
+#pragma unroll
+  for (int j = 0; j < kLogpStreams; ++j) {
+    const float pm = xm[(int64_t)j * T];
+    const float term = xm[splane + (int64_t)j * T] * pinned_exp(pm - big);
+    sum = sum + ((pm > kNegInf) ? term : 0.f);
+    zt = zt + xm[2 * splane + (int64_t)j * T];
+  }
+  const int64_t plane = (int64_t)n_split * T;
+  const int64_t at = (int64_t)split * T + m;
+  part[at] = big;
+  part[plane + at] = sum;
+  part[2 * plane + at] = zt;
+}
+
 // Final merge over splits. 16 tokens per workgroup, 16 threads per token: the maximum and
 // the rescaled terms s_p * e(m_p - M) are computed by all threads (neither depends on an
 // order), then one thread per token adds the terms of a chunk in ascending split order,
@@ -258,8 +386,13 @@ using LogpShape16 = TileShape<256, 16, 4, 1>;
 
 int linear_logp_split_count(int V) { return (V + kLogpSplitCols - 1) / kLogpSplitCols; }
 
+constexpr int kStreamGroupMaxTokens = 64;  // token counts the stream-group kernel serves
+
 size_t linear_logp_workspace_bytes(int T, int V) {
-  return (size_t)3 * linear_logp_split_count(V) * (size_t)(T > 0 ? T : 0) * sizeof(float);
+  if (T <= 0) return 0;
+  // per-split partials, plus per-(split, stream) states where the stream-group kernel may run
+  const size_t per_split = (size_t)3 * linear_logp_split_count(V) * (size_t)T * sizeof(float);
+  return T <= kStreamGroupMaxTokens ? per_split * (1 + kLogpStreams) : per_split;
 }
 
 template <class S, int LOOP>
@@ -283,12 +416,39 @@ static hipError_t launch_logp(LogpArgs a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+static hipError_t launch_streamgroup(LogpArgs a, hipStream_t stream) {
+  using S = LogpShape64;
+  auto kernel = linear_logp_streamgroup_kernel<S>;
+  constexpr int kYBytes = kLogpSplitTiles * 4 * S::BM * 16 * (int)sizeof(float);
+  constexpr int kLds = S::kLdsBytes > kYBytes ? S::kLdsBytes : kYBytes;
+  static bool configured[kMaxDevices] = {};
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev >= 0 && dev < kMaxDevices && !configured[dev]) {
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              kLds);
+    if (err != hipSuccess) return err;
+    configured[dev] = true;
+  }
+  a.tiles_m = (a.T + S::BM - 1) / S::BM;
+  float* spart = a.part + (size_t)3 * a.n_split * a.T;  // behind the per-split partials
+  hipLaunchKernelGGL(kernel, dim3(a.tiles_m * a.n_split * (kLogpStreams / 4)), dim3(S::kThreads), kLds, stream, a,
+                     spart);
+  err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  const int threads = a.T * a.n_split;
+  hipLaunchKernelGGL(linear_logp_stream_merge_kernel, dim3((threads + 255) / 256), dim3(256), 0, stream, spart,
+                     a.part, a.T, a.n_split);
+  return hipGetLastError();
+}
+
 int pick_linear_logp_config(int T, int V) {
   (void)V;
   // Measured at V = 151936, D = 4096: the 64-token tile (two workgroups per CU, direct-to-LDS
   // loop) is the fastest from decode sizes up to 64 tokens, the 256-token tile from 256 tokens on
   // even where it leaves the last round of workgroups part empty.
-  if (T <= 64) return RLK_LOGP_CFG_64;
+  if (T <= kStreamGroupMaxTokens) return RLK_LOGP_CFG_64_STREAMS;
   if (T <= 128) return RLK_LOGP_CFG_128;
   return RLK_LOGP_CFG_256;
 }
@@ -319,8 +479,13 @@ hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t*
   if (config == RLK_LOGP_CFG_AUTO) config = pick_linear_logp_config(T, V);
   if (!vec && config == RLK_LOGP_CFG_256) config = RLK_LOGP_CFG_128;
   const int loop = !vec ? 0 : (D % kTileK == 0 && !force_staged) ? 2 : 1;
+  // The stream-group kernel has the direct-to-LDS loop only and serves one token tile.
+  if (config == RLK_LOGP_CFG_64_STREAMS && (loop != 2 || T > kStreamGroupMaxTokens)) config = RLK_LOGP_CFG_64;
   hipError_t err;
   switch (config) {
+    case RLK_LOGP_CFG_64_STREAMS:
+      err = launch_streamgroup(a, stream);
+      break;
     case RLK_LOGP_CFG_256:
       err = loop == 2 ? launch_logp<LogpShape256, 2>(a, stream) : launch_logp<LogpShape256, 1>(a, stream);
       break;
