@@ -102,8 +102,11 @@ typedef enum rlk_logp_config {
   RLK_LOGP_CFG_128 = 2,
   RLK_LOGP_CFG_64 = 3,
   RLK_LOGP_CFG_16 = 4,
-  RLK_LOGP_CFG_64_STREAMS = 5, /* <= 64 tokens: four workgroups per vocabulary split, four streams each */
-  RLK_LOGP_CFG_COUNT = 6,
+  /* up to 1024 tokens: four workgroups per vocabulary split, four streams each (64 / 128 / 256-token tiles) */
+  RLK_LOGP_CFG_64_STREAMS = 5,
+  RLK_LOGP_CFG_128_STREAMS = 6,
+  RLK_LOGP_CFG_256_STREAMS = 7,
+  RLK_LOGP_CFG_COUNT = 8,
   /* OR-ed into a configuration: register-staged main loop instead of the
    * direct-to-LDS ping-pong loop (bit-neutral; for tests). */
   RLK_LOGP_CFG_FORCE_STAGED = 0x100
@@ -120,7 +123,7 @@ const char* rlk_linear_logp_contract_id(void);
 int rlk_linear_logp_split_count(int V);
 
 /* Bytes of fp32 partials rlk_linear_logp_fwd needs for T tokens and V vocabulary rows
- * (3 * splits * T floats; 17 times that for T <= 64, where per-stream states are staged). */
+ * (3 * splits * T floats; 17 times that for T <= 1024, where per-stream states are staged). */
 size_t rlk_linear_logp_workspace_bytes(int T, int V);
 
 /*

@@ -170,17 +170,18 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_partial_kernel(LogpAr
   }
 }
 
-// Small token counts (one 64-token tile): a split of 1024 columns gives the chip only
-// ceil(V / 1024) workgroups. Streams are independent until the stream merge, so here a
+// Few token tiles: a split of 1024 columns gives the chip only tiles_m * ceil(V / 1024)
+// workgroups of four K loops each. Streams are independent until the stream merge, so here a
 // workgroup takes four of the sixteen streams of a split, i.e. the 64-column slice
 // [64 g, 64 g + 64) of each of the split's four tiles, as ONE 256-row GEMM tile (wave column t
-// holds tile t's slice): four times the workgroups, one K loop each. The per-tile scaled
-// logits go through LDS to the threads that run the same ascending online chain over the four
-// tiles; per-(split, stream) states are merged by linear_logp_stream_merge_kernel with the
-// arithmetic of the in-kernel stream merge above. Same bits as every other configuration.
+// holds tile t's slice): four times the workgroups, one K loop each. The online chain of a
+// (token, stream) still visits the tiles in ascending order: wave column t folds its sixteen
+// columns into the state that column t - 1 left in LDS. Per-(split, stream) states go to
+// linear_logp_stream_merge_kernel, which repeats the in-kernel stream merge above. Same bits
+// as every other configuration.
 template <class S>
 __global__ __launch_bounds__(S::kThreads) void linear_logp_streamgroup_kernel(LogpArgs a, float* __restrict__ spart) {
-  static_assert(S::BN == kLogpTileCols && S::kRun == 16 && S::WN == 4 && S::TM == 2, "256 x 64 tile, 4 x 2 waves");
+  static_assert(S::BN == kLogpTileCols && S::kRun == 16 && S::WN == 4, "wave column = tile of the split");
   constexpr int kGroups = kLogpStreams / 4;  // stream groups per split
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -195,55 +196,53 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_streamgroup_kernel(Lo
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int tile = wave % S::WN;  // wave column = tile of the split
+  const int tile = wave % S::WN;
   const int wave_m = wave / S::WN;
   const int l16 = lane & 15;
   const int grp = lane >> 4;  // stream inside the group
+  const int tok_local = wave_m * 16 * S::TM + l16;
 
   f32x4_t acc[S::TN][S::TM];
   tile_mainloop_pingpong<S, false, false, StridedColumnRowMap<S, kLogpTileCols>>(a.W, a.H, n0, m0, a.D, lds, acc);
 
-  // Scaled logits of this lane's (token, tile, stream) into LDS: ybuf[tile][stream][token][16].
-  float* ybuf = reinterpret_cast<float*>(lds);
-  {
-    const int col0 = n0 + tile * kLogpTileCols + grp * 16;
-    float bias_run[16];
+  const int v0 = split * kLogpSplitCols + tile * kLogpTileCols;
+  const int col0 = v0 + (sg * 4 + grp) * 16;  // first column of this lane's run
+  float bias_run[16];
 #pragma unroll
-    for (int c = 0; c < 16; ++c) bias_run[c] = (a.bias && col0 + c < a.V) ? a.bias[col0 + c] : 0.f;
-#pragma unroll
-    for (int jm = 0; jm < S::TM; ++jm) {
-      const int tok = wave_m * 16 * S::TM + jm * 16 + l16;
-      const int m = m0 + tok;
-      const float inv_t = (a.temperature && m < a.T) ? 1.0f / a.temperature[m] : 1.0f;
-      float* dst = ybuf + ((tile * 4 + grp) * S::BM + tok) * 16;
-#pragma unroll
-      for (int c = 0; c < 16; ++c)
-        dst[c] = scaled_logit(acc[c >> 2][jm][c & 3], a.bias != nullptr, bias_run[c], col0 + c, a.vocab_limit,
-                              a.temperature != nullptr, inv_t);
-    }
-  }
-  __syncthreads();
+  for (int c = 0; c < 16; ++c) bias_run[c] = (a.bias && col0 + c < a.V) ? a.bias[col0 + c] : 0.f;
 
-  // One thread per (stream of the group, token): the chain over the split's tiles, ascending.
-  if (threadIdx.x < 4 * S::BM) {
-    const int sl = threadIdx.x / S::BM;
-    const int tok = threadIdx.x % S::BM;
-    const int m = m0 + tok;
-    if (m < a.T) {
-      const int64_t local = a.target[m] - a.vocab_start;
-      const int tgt = (local >= 0 && local < a.vocab_limit) ? (int)local : -1;
-      float run_m = kNegInf, run_s = 0.f, run_zt = 0.f;
-      for (int t = 0; t < kLogpSplitTiles; ++t) {
-        const int v0 = split * kLogpSplitCols + t * kLogpTileCols;
-        if (v0 >= a.V) break;
-        const int col0 = v0 + (sg * 4 + sl) * 16;
-        const float* src = ybuf + ((t * 4 + sl) * S::BM + tok) * 16;
+  // The main loop ended on a barrier, so the staging LDS is free: states [3][4 streams][BM].
+  float* sm = reinterpret_cast<float*>(lds);
+  float* ss = sm + 4 * S::BM;
+  float* sz = ss + 4 * S::BM;
+#pragma unroll 1
+  for (int t = 0; t < kLogpSplitTiles; ++t) {
+    if (tile == t && v0 < a.V) {  // a tile past the vocabulary leaves the states alone
+#pragma unroll
+      for (int jm = 0; jm < S::TM; ++jm) {
+        const int slot = grp * S::BM + tok_local + jm * 16;
+        const int m = m0 + tok_local + jm * 16;
+        int tgt = -1;
+        float inv_t = 1.0f;
+        if (m < a.T) {
+          const int64_t local = a.target[m] - a.vocab_start;
+          tgt = (local >= 0 && local < a.vocab_limit) ? (int)local : -1;
+          if (a.temperature) inv_t = 1.0f / a.temperature[m];
+        }
+        float run_m = kNegInf, run_s = 0.f, run_zt = 0.f;
+        if (t > 0) {
+          run_m = sm[slot];
+          run_s = ss[slot];
+          run_zt = sz[slot];
+        }
         float y[16];
         float tmax = kNegInf;
 #pragma unroll
         for (int c = 0; c < 16; ++c) {
-          y[c] = src[c];
-          tmax = fmaxf(tmax, y[c]);
+          const float z = scaled_logit(acc[c >> 2][jm][c & 3], a.bias != nullptr, bias_run[c], col0 + c,
+                                       a.vocab_limit, a.temperature != nullptr, inv_t);
+          y[c] = z;
+          tmax = fmaxf(tmax, z);
         }
         const int tl = tgt - col0;
         if (tl >= 0 && tl < 16) {
@@ -259,14 +258,23 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_streamgroup_kernel(Lo
         for (int c = 1; c < 16; ++c) sum = sum + pinned_exp(y[c] - new_m);
         const float scaled = run_s * pinned_exp(old_m - new_m);
         run_s = (new_m > kNegInf) ? (scaled + sum) : run_s;
-        run_m = new_m;
+        sm[slot] = new_m;
+        ss[slot] = run_s;
+        sz[slot] = run_zt;
       }
-      const int64_t plane = (int64_t)a.n_split * kLogpStreams * a.T;
-      const int64_t at = ((int64_t)split * kLogpStreams + sg * 4 + sl) * a.T + m;
-      spart[at] = run_m;
-      spart[plane + at] = run_s;
-      spart[2 * plane + at] = run_zt;
     }
+    __syncthreads();
+  }
+
+  const int64_t plane = (int64_t)a.n_split * kLogpStreams * a.T;
+  for (int idx = threadIdx.x; idx < 4 * S::BM; idx += S::kThreads) {
+    const int sl = idx / S::BM;
+    const int m = m0 + idx % S::BM;
+    if (m >= a.T) continue;
+    const int64_t at = ((int64_t)split * kLogpStreams + sg * 4 + sl) * a.T + m;
+    spart[at] = sm[idx];
+    spart[plane + at] = ss[idx];
+    spart[2 * plane + at] = sz[idx];
   }
 }
 
@@ -386,7 +394,7 @@ using LogpShape16 = TileShape<256, 16, 4, 1>;
 
 int linear_logp_split_count(int V) { return (V + kLogpSplitCols - 1) / kLogpSplitCols; }
 
-constexpr int kStreamGroupMaxTokens = 64;  // token counts the stream-group kernel serves
+constexpr int kStreamGroupMaxTokens = 1024;  // token counts the stream-group kernels serve
 
 size_t linear_logp_workspace_bytes(int T, int V) {
   if (T <= 0) return 0;
@@ -416,25 +424,23 @@ static hipError_t launch_logp(LogpArgs a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+template <class S>
 static hipError_t launch_streamgroup(LogpArgs a, hipStream_t stream) {
-  using S = LogpShape64;
   auto kernel = linear_logp_streamgroup_kernel<S>;
-  constexpr int kYBytes = kLogpSplitTiles * 4 * S::BM * 16 * (int)sizeof(float);
-  constexpr int kLds = S::kLdsBytes > kYBytes ? S::kLdsBytes : kYBytes;
   static bool configured[kMaxDevices] = {};
   int dev = 0;
   hipError_t err = hipGetDevice(&dev);
   if (err != hipSuccess) return err;
   if (dev >= 0 && dev < kMaxDevices && !configured[dev]) {
     err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              kLds);
+                              S::kLdsBytes);
     if (err != hipSuccess) return err;
     configured[dev] = true;
   }
   a.tiles_m = (a.T + S::BM - 1) / S::BM;
   float* spart = a.part + (size_t)3 * a.n_split * a.T;  // behind the per-split partials
-  hipLaunchKernelGGL(kernel, dim3(a.tiles_m * a.n_split * (kLogpStreams / 4)), dim3(S::kThreads), kLds, stream, a,
-                     spart);
+  hipLaunchKernelGGL(kernel, dim3(a.tiles_m * a.n_split * (kLogpStreams / 4)), dim3(S::kThreads), S::kLdsBytes, stream,
+                     a, spart);
   err = hipGetLastError();
   if (err != hipSuccess) return err;
   const int threads = a.T * a.n_split;
@@ -448,8 +454,9 @@ int pick_linear_logp_config(int T, int V) {
   // Measured at V = 151936, D = 4096: the 64-token tile (two workgroups per CU, direct-to-LDS
   // loop) is the fastest from decode sizes up to 64 tokens, the 256-token tile from 256 tokens on
   // even where it leaves the last round of workgroups part empty.
-  if (T <= kStreamGroupMaxTokens) return RLK_LOGP_CFG_64_STREAMS;
-  if (T <= 128) return RLK_LOGP_CFG_128;
+  if (T <= 64) return RLK_LOGP_CFG_64_STREAMS;
+  if (T <= 128) return RLK_LOGP_CFG_128_STREAMS;
+  if (T <= 1024) return RLK_LOGP_CFG_256_STREAMS;
   return RLK_LOGP_CFG_256;
 }
 
@@ -479,12 +486,22 @@ hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t*
   if (config == RLK_LOGP_CFG_AUTO) config = pick_linear_logp_config(T, V);
   if (!vec && config == RLK_LOGP_CFG_256) config = RLK_LOGP_CFG_128;
   const int loop = !vec ? 0 : (D % kTileK == 0 && !force_staged) ? 2 : 1;
-  // The stream-group kernel has the direct-to-LDS loop only and serves one token tile.
-  if (config == RLK_LOGP_CFG_64_STREAMS && (loop != 2 || T > kStreamGroupMaxTokens)) config = RLK_LOGP_CFG_64;
+  // The stream-group kernels have the direct-to-LDS loop only and a bounded workspace.
+  if (loop != 2 || T > kStreamGroupMaxTokens) {
+    if (config == RLK_LOGP_CFG_64_STREAMS) config = RLK_LOGP_CFG_64;
+    if (config == RLK_LOGP_CFG_128_STREAMS) config = RLK_LOGP_CFG_128;
+    if (config == RLK_LOGP_CFG_256_STREAMS) config = RLK_LOGP_CFG_256;
+  }
   hipError_t err;
   switch (config) {
     case RLK_LOGP_CFG_64_STREAMS:
-      err = launch_streamgroup(a, stream);
+      err = launch_streamgroup<LogpShape64>(a, stream);
+      break;
+    case RLK_LOGP_CFG_128_STREAMS:
+      err = launch_streamgroup<LogpShape128>(a, stream);
+      break;
+    case RLK_LOGP_CFG_256_STREAMS:
+      err = launch_streamgroup<LogpShape256>(a, stream);
       break;
     case RLK_LOGP_CFG_256:
       err = loop == 2 ? launch_logp<LogpShape256, 2>(a, stream) : launch_logp<LogpShape256, 1>(a, stream);

@@ -229,7 +229,10 @@ hipError_t linear_logp_bwd_launch(const MatView& H, const MatView& W, const int6
   const bool force_staged = (config & RLK_LOGP_CFG_FORCE_STAGED) != 0;
   config &= ~RLK_LOGP_CFG_FORCE_STAGED;
   if (config == RLK_LOGP_CFG_AUTO) config = pick_linear_logp_config(T, V);
-  if (config == RLK_LOGP_CFG_64_STREAMS) config = RLK_LOGP_CFG_64;  // a forward-only work split
+  // the stream-group configurations are forward-only work splits
+  if (config == RLK_LOGP_CFG_64_STREAMS) config = RLK_LOGP_CFG_64;
+  if (config == RLK_LOGP_CFG_128_STREAMS) config = RLK_LOGP_CFG_128;
+  if (config == RLK_LOGP_CFG_256_STREAMS) config = RLK_LOGP_CFG_256;
   if (!vec && config == RLK_LOGP_CFG_256) config = RLK_LOGP_CFG_128;
   const int loop = !vec ? 0 : (D % kTileK == 0 && !force_staged) ? 2 : 1;
   hipError_t err;

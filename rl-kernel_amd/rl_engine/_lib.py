@@ -42,7 +42,7 @@ FORCE_STAGED = 0x100
 # rlk_dtype (element types of materialised logits)
 DTYPE_BF16, DTYPE_FP16, DTYPE_FP32 = 0, 1, 2
 # rlk_logp_config
-LOGP_CONFIGS = {"auto": 0, "256": 1, "128": 2, "64": 3, "16": 4, "64_streams": 5}
+LOGP_CONFIGS = {"auto": 0, "256": 1, "128": 2, "64": 3, "16": 4, "64_streams": 5, "128_streams": 6, "256_streams": 7}
 
 EXPORTED_SYMBOLS = (
     "rlk_contract_id",

@@ -72,7 +72,7 @@ def test_parity_with_oracle_and_config_neutrality(logp_mod, oracle, shape):
     dense_logp = oracle.linear_logp_dense(inputs.bits(h), inputs.bits(w), target.numpy())[0]
     h_d, w_d, t_d = h.to(DEV), w.to(DEV), target.to(DEV)
     base = None
-    for name in ("256", "128", "64", "16", "64_streams", "auto"):
+    for name in ("256", "128", "64", "16", "64_streams", "128_streams", "256_streams", "auto"):
         logp, lse = logp_mod.deterministic_linear_logp(h_d, w_d, t_d, config=name)
         assert np.abs(logp.cpu().numpy() - ref_logp).max() <= TOL_NATS
         assert np.abs(lse.cpu().numpy() - ref_lse).max() <= TOL_NATS
@@ -113,9 +113,12 @@ def test_row_alone_equals_row_in_batch_with_bias_temperature_padding(logp_mod):
     assert float((picked - logp.double()).abs().max()) < 1e-4
 
 
-@pytest.mark.parametrize("shape", [(1, 5000, 256, 4900), (17, 3072, 128, 3000), (64, 9001, 320, 9001), (33, 1024, 64, 1000)])
+@pytest.mark.parametrize(
+    "shape",
+    [(1, 5000, 256, 4900), (17, 3072, 128, 3000), (64, 9001, 320, 9001), (33, 1024, 64, 1000), (130, 4608, 128, 4500), (700, 2300, 192, 2290)],
+)
 def test_stream_group_split_keeps_the_bits(logp_mod, oracle, shape):
-    # Up to 64 tokens the vocabulary splits are cut into four stream groups, one workgroup each:
+    # For few token tiles the vocabulary splits are cut into four stream groups, one workgroup each:
     # a different work split, the same contract. Bias, temperature and padded vocabulary included.
     n, v, d, real = shape
     h, w, target = inputs.logp_inputs(n, vocab=v, hidden=d, seed=4350 + n, rms_norm=False)
@@ -130,7 +133,7 @@ def test_stream_group_split_keeps_the_bits(logp_mod, oracle, shape):
     h_d, w_d, t_d, b_d, tmp_d = h.to(DEV), w.to(DEV), target.to(DEV), bias.to(DEV), temp.to(DEV)
     for extra in ({}, {"bias": b_d, "temperature": tmp_d, "real_vocab_size": real}):
         base = logp_mod.deterministic_linear_logp(h_d, w_d, t_d, config="256", **extra)
-        for name in ("64_streams", "auto"):
+        for name in ("64_streams", "128_streams", "256_streams", "auto"):
             got = logp_mod.deterministic_linear_logp(h_d, w_d, t_d, config=name, **extra)
             assert _same_bits(got[0], base[0]) and _same_bits(got[1], base[1]), (name, sorted(extra))
     assert np.abs(got[0].cpu().numpy() - ref_logp).max() <= TOL_NATS
