@@ -258,6 +258,22 @@ def main() -> int:
                 )
         result["shapes"] = shapes
 
+    # ---- attention projections at the packed token count (ragged packing does not change the launch)
+    if not args.no_shapes:
+        tp = 16384
+        xa = randn(tp, HIDDEN)
+        proj = []
+        for name, n in (("qkv_proj", 6144), ("o_proj", 4096)):
+            w_p = randn(n, HIDDEN, 0.02)
+            o_p = torch.empty((tp, n), dtype=torch.bfloat16, device=dev)
+            ms = _time_calls(lambda: gemm.mfma_gemm(xa, w_p.t(), out=o_p), 20, 20)
+            fl = 2.0 * tp * n * HIDDEN
+            proj.append({"op": name, "T": tp, "N": n, "K": HIDDEN, "ms": round(ms, 4), "tflops": round(fl / ms * 1e-9, 1),
+                         "bound": "mfma", "frac": round(fl / ms * 1e-9 / PEAK_BF16_TFLOPS, 4)})
+            del w_p, o_p
+        result["attention_projections"] = proj
+        del xa
+
     # ---- fused linear-LogP at T=8192, V=151936
     if not args.no_logp:
         tl = 8192
@@ -302,6 +318,33 @@ def main() -> int:
             "frac_of_hbm_peak": round(by_fl / ms_fl * 1e-6 / PEAK_HBM_GBPS, 4),
         }
         del logits
+        # rollout scale: 64 rollouts x 1024 tokens through the fused LogP, then the GRPO ratio / k3-KL epilogue
+        from rl_engine.ops.loss import grpo_ratio_kl_loss
+
+        rollouts, per = 64, 1024
+        tr = rollouts * per
+        hid_r = randn(tr, HIDDEN)
+        tgt_r = torch.randint(0, VOCAB, (tr,), generator=gen, device=dev)
+        logp_r, _ = deterministic_linear_logp(hid_r, w_lm, tgt_r)
+        old_r = (logp_r + 0.05 * torch.randn((tr,), generator=gen, device=dev)).view(rollouts, per)
+        ref_r = (logp_r + 0.05 * torch.randn((tr,), generator=gen, device=dev)).view(rollouts, per)
+        adv_r = torch.randn((rollouts,), generator=gen, device=dev)
+
+        def rollout_step():
+            lp, _ = deterministic_linear_logp(hid_r, w_lm, tgt_r)
+            return grpo_ratio_kl_loss(lp.view(rollouts, per), old_r, ref_r, adv_r, clip_eps=0.2, beta=0.01)
+
+        ms_r = _time_calls(rollout_step, 3, 2)
+        ms_g = _time_calls(lambda: grpo_ratio_kl_loss(logp_r.view(rollouts, per), old_r, ref_r, adv_r, clip_eps=0.2, beta=0.01), 20, 5)
+        result["linear_logp"]["rollout_grpo"] = {
+            "workload": "64 rollouts x 1024 tokens: fused LogP (V=151936) -> ratio, k3-KL, clipped loss",
+            "ms": round(ms_r, 3),
+            "tokens_per_s": round(tr / ms_r * 1e3, 1),
+            "tflops": round(2.0 * tr * VOCAB * HIDDEN / ms_r * 1e-9, 1),
+            "frac_of_mfma_peak": round(2.0 * tr * VOCAB * HIDDEN / ms_r * 1e-9 / PEAK_BF16_TFLOPS, 4),
+            "grpo_epilogue_ms": round(ms_g, 4),
+        }
+        del hid_r, tgt_r, logp_r, old_r, ref_r
 
     # ---- gated FFN at T=4096: fused gate/up + SwiGLU, then down
     if not args.no_shapes:
