@@ -246,23 +246,28 @@ int pick_det_gemm_config(int M, int N, int K) {
     if (tile_count(M, N, 64, 128) <= kCus) return RLK_GEMM_CFG_128x64_DEEP;
     if (tile_count(M, N, 128, 128) <= kCus) return RLK_GEMM_CFG_128x128_DEEP;
   }
-  // Estimated time = (rounds of 256 workgroups) x (tile area / measured relative
-  // throughput of the shape when the chip is full). Larger tiles win ties.
+  // Estimated time = (rounds of 256 workgroups) x (tile area / relative throughput of the
+  // shape when the chip is full), fitted to sweeps over the Qwen3-8B projection shapes at
+  // 384 ... 6144 tokens. A last, partly filled round is nearly free beyond its own share: the
+  // chip is power limited, and a round that keeps fewer CUs busy runs at a higher clock, so
+  // the 256 x 256 tile wins unless its tiles cover well under one round. Larger tiles win ties.
   struct Candidate {
     int config, bn, bm;
     double quality;
   };
   static const Candidate kCandidates[] = {
-      {RLK_GEMM_CFG_256x256, 256, 256, 1.00}, {RLK_GEMM_CFG_256x128, 256, 128, 0.95},
-      {RLK_GEMM_CFG_256x64, 256, 64, 0.75},
-      {RLK_GEMM_CFG_128x128, 128, 128, 0.90}, {RLK_GEMM_CFG_128x64, 128, 64, 0.70},
-      {RLK_GEMM_CFG_64x64, 64, 64, 0.55},
+      {RLK_GEMM_CFG_256x256, 256, 256, 1.00}, {RLK_GEMM_CFG_256x128, 256, 128, 0.65},
+      {RLK_GEMM_CFG_256x64, 256, 64, 0.50},
+      {RLK_GEMM_CFG_128x128, 128, 128, 0.65}, {RLK_GEMM_CFG_128x64, 128, 64, 0.45},
+      {RLK_GEMM_CFG_64x64, 64, 64, 0.42},
   };
   int best = RLK_GEMM_CFG_64x64;
   double best_time = 1e300;
   for (const Candidate& c : kCandidates) {
     const int64_t tiles = tile_count(M, N, c.bm, c.bn);
-    const double rounds = (double)((tiles + kCus - 1) / kCus);
+    const int64_t full = tiles / kCus;
+    const double part = (double)(tiles - full * kCus) / kCus;
+    const double rounds = (double)full + (part > 0.0 ? (part > 0.9 ? part : 0.9) : 0.0);
     const double t = rounds * (double)(c.bn * c.bm) / c.quality;
     if (t < best_time * 0.999) {
       best_time = t;

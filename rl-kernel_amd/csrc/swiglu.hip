@@ -224,7 +224,15 @@ hipError_t det_gemm_swiglu_launch(const MatView& W, const MatView& X, void* Y, i
   if (det_gemm_swiglu_fused_supported(W, X, M, K)) {
     const int64_t t256 = (int64_t)((M + 255) / 256) * ((I + 127) / 128);
     const int64_t t128 = (int64_t)((M + 127) / 128) * ((I + 127) / 128);
-    if (M > 128 && t256 >= 256) return launch_gated<GatedShape256>(W, X, Y, ldy, M, I, K, stream);
+    // Rounds of 256 workgroups x tokens per tile / relative throughput, as in pick_det_gemm_config:
+    // a partly filled last round costs little more than its share, so the large tile wins early.
+    auto cost = [](int64_t tiles, double tokens, double quality) {
+      const int64_t full = tiles / 256;
+      const double part = (double)(tiles - full * 256) / 256.0;
+      return ((double)full + (part > 0.0 ? (part > 0.9 ? part : 0.9) : 0.0)) * tokens / quality;
+    };
+    if (M > 128 && cost(t256, 256.0, 1.0) <= cost(t128, 128.0, 0.65))
+      return launch_gated<GatedShape256>(W, X, Y, ldy, M, I, K, stream);
     if (M > 64 && t128 >= 128) return launch_gated<GatedShape128>(W, X, Y, ldy, M, I, K, stream);
     return launch_gated<GatedShape64>(W, X, Y, ldy, M, I, K, stream);
   }
