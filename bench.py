@@ -274,6 +274,17 @@ def main() -> int:
         result["attention_projections"] = proj
         del xa
 
+    # ---- the k-tree contract (vector-ALU kernel) on the same gate_up step
+    if not args.no_shapes:
+        ms_tree = _time_calls(lambda: gemm.tree_gemm(x, w_gu.t(), out=out_gu), 3, 1)
+        result["det_gemm_tree"] = {
+            "workload": "gate_up X[4096,4096]xW[24576,4096]^T under the k-tree contract (fp32 FMA leaves of 32, bf16 midpoint tree)",
+            "ms": round(ms_tree, 3),
+            "tflops": round(flops_gu / ms_tree * 1e-9, 1),
+            "bound": "fp32 vector FMA",
+            "contract": _lib.load().rlk_det_gemm_tree_contract_id().decode(),
+        }
+
     # ---- fused linear-LogP at T=8192, V=151936
     if not args.no_logp:
         tl = 8192

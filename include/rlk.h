@@ -91,6 +91,29 @@ int rlk_det_gemm_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stride, c
                       int64_t b_k_stride, int64_t b_n_stride, void* c, int64_t ldc, int M, int N, int K,
                       int out_fp32, int config, void* stream);
 
+/*
+ * C[M,N] = A[M,K] @ B[K,N] under the k-tree contract (rlk_det_gemm_tree_contract_id):
+ *   T(lo,hi) = bf16(sum of a_k*b_k, k = lo..hi-1, fp32 from +0, k ascending, fused multiply-add)
+ *              when hi - lo <= 32, else bf16(float(T(lo,mid)) + float(T(mid,hi))) with
+ *              mid = lo + (hi - lo) / 2;  C = T(0, K).
+ * Rounding points depend on K only: rows are batch invariant, and a K range that is a subtree
+ * (the contiguous half, quarter, ... of a K-sharded rank) evaluates to exactly that node.
+ * Strides as in rlk_det_gemm_bf16; any non-negative strides are accepted (no fast layout:
+ * this is a vector-ALU kernel, about 20 times slower than the MFMA contract). bf16 output only.
+ *
+ * Stands in for the reference's "triton_tree" backend: _triton_tree_gemm and its tree plan
+ * (rl_engine/backends/shared/triton/gemm/det_gemm.py:218-258, 355-417, 514-546), the CUDA
+ * k_tree_naive kernel (csrc/cuda/gemm/det_gemm_kernel.cu:74-85) and the specification the
+ * reference's tests evaluate (tests/ops/gemm/test_det_gemm.py:156-168).
+ */
+int rlk_det_gemm_tree_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stride, const void* b,
+                           int64_t b_k_stride, int64_t b_n_stride, void* c, int64_t ldc, int M, int N, int K,
+                           void* stream);
+
+/* Contract id of rlk_det_gemm_tree_bf16 (the reference reports
+ * "rlkernel.det_gemm.triton_tree_rocm.v1", rl_engine/backends/rocm/gemm/det_gemm.py:101-104). */
+const char* rlk_det_gemm_tree_contract_id(void);
+
 /* The configuration RLK_GEMM_CFG_AUTO resolves to for a shape (host only, no GPU call).
  * Stands in for select_config, rl_engine/backends/rocm/gemm/mfma_gemm.py:76-92. */
 int rlk_det_gemm_pick_config(int M, int N, int K);

@@ -75,11 +75,15 @@ void oracle_gemm_f64(const uint16_t* a, const uint16_t* bt, double* c, int M, in
  * children, rounded to bf16); the split point is the midpoint in ELEMENT space.
  * Follows tests/ops/gemm/test_det_gemm.py:156-168 (_k_tree_gemm) and
  * csrc/cuda/gemm/det_gemm_kernel.cu:74-85 (k_tree_naive).
+ * A leaf term is one fused multiply-add, as in the reference's GPU kernels ("scalar-FMA
+ * leaves", rl_engine/backends/rocm/gemm/det_gemm.py:35-36; nvcc contracts acc += a*b).
+ * The product of two bf16 values is exact in fp32 unless it underflows below 2^-126,
+ * so fmaf and multiply-then-add differ only there.
  */
 static uint16_t k_tree_element(const uint16_t* arow, const uint16_t* brow, int lo, int hi) {
   if (hi - lo <= 32) {
     float acc = 0.0f;
-    for (int k = lo; k < hi; ++k) acc = acc + bf16_to_f32(arow[k]) * bf16_to_f32(brow[k]);
+    for (int k = lo; k < hi; ++k) acc = fmaf(bf16_to_f32(arow[k]), bf16_to_f32(brow[k]), acc);
     return f32_to_bf16(acc);
   }
   const int mid = lo + (hi - lo) / 2;
@@ -99,7 +103,7 @@ static uint16_t k_tree_leaf(const uint16_t* arow, const uint16_t* brow, int K, i
     const int lo = leaf_lo * 32;
     const int hi = (lo + 32 < K) ? lo + 32 : K;
     float acc = 0.0f;
-    for (int k = lo; k < hi; ++k) acc = acc + bf16_to_f32(arow[k]) * bf16_to_f32(brow[k]);
+    for (int k = lo; k < hi; ++k) acc = fmaf(bf16_to_f32(arow[k]), bf16_to_f32(brow[k]), acc);
     return f32_to_bf16(acc);
   }
   const int mid = leaf_lo + (leaf_hi - leaf_lo) / 2;

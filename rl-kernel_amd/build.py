@@ -14,7 +14,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "librlk_gfx950.so"
-SOURCES = ["det_gemm.hip", "det_gemm_stream.hip", "linear_logp.hip",
+SOURCES = ["det_gemm.hip", "det_gemm_stream.hip", "det_gemm_tree.hip", "linear_logp.hip",
     "linear_logp_bwd.hip", "logits_logp.hip", "swiglu.hip", "grpo.hip", "rlk_api.hip"]
 
 HIPCC_FLAGS = [

@@ -89,6 +89,44 @@ int rlk_det_gemm_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stride, c
   return err == hipSuccess ? RLK_OK : device_error("rlk_det_gemm_bf16", err);
 }
 
+const char* rlk_det_gemm_tree_contract_id(void) { return "rlkernel.det_gemm.hip_ktree32_gfx950.v1"; }
+
+int rlk_det_gemm_tree_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stride, const void* b,
+                           int64_t b_k_stride, int64_t b_n_stride, void* c, int64_t ldc, int M, int N, int K,
+                           void* stream) {
+  if (M < 0 || N < 0 || K < 0) {
+    set_last_error("rlk_det_gemm_tree_bf16: negative size M=%d N=%d K=%d", M, N, K);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (K > det_gemm_tree_max_k()) {
+    set_last_error("rlk_det_gemm_tree_bf16: K=%d exceeds the supported %d", K, det_gemm_tree_max_k());
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (a_row_stride < 0 || a_k_stride < 0 || b_k_stride < 0 || b_n_stride < 0) {
+    set_last_error("rlk_det_gemm_tree_bf16: operands must not use negative strides");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (M == 0 || N == 0) return RLK_OK;
+  if (c == nullptr || ldc < N) {
+    set_last_error("rlk_det_gemm_tree_bf16: output needs a non-null pointer and ldc >= N (ldc=%lld N=%d)",
+                   (long long)ldc, N);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (K == 0) {
+    hipError_t err = fill_zero_launch(c, M, N, ldc, 2, s);
+    return err == hipSuccess ? RLK_OK : device_error("rlk_det_gemm_tree_bf16(fill)", err);
+  }
+  if (a == nullptr || b == nullptr) {
+    set_last_error("rlk_det_gemm_tree_bf16: null operand");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  MatView A{reinterpret_cast<const bf16_bits*>(a), a_row_stride, a_k_stride, M};
+  MatView B{reinterpret_cast<const bf16_bits*>(b), b_n_stride, b_k_stride, N};
+  hipError_t err = det_gemm_tree_launch(A, B, c, ldc, M, N, K, s);
+  return err == hipSuccess ? RLK_OK : device_error("rlk_det_gemm_tree_bf16", err);
+}
+
 const char* rlk_linear_logp_contract_id(void) { return "rlkernel.linear_logp.hip_streams16x256_split1024_gfx950.v1"; }
 
 int rlk_linear_logp_split_count(int V) { return V > 0 ? linear_logp_split_count(V) : 0; }

@@ -18,6 +18,12 @@ int pick_det_gemm_config(int M, int N, int K);
 hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
                            bool out_f32, int config, hipStream_t stream);
 
+// The k-tree contract (fp32 leaves of at most 32 K values, bf16 midpoint tree). A[M, K]; B holds
+// one row per output column (B.rows == N); any strides. K <= det_gemm_tree_max_k().
+int det_gemm_tree_max_k();
+hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int64_t ldc, int M, int N, int K,
+                                hipStream_t stream);
+
 // Decode-sized batches (M <= 16), unit K stride, K % 64 == 0.
 hipError_t det_gemm_stream_launch(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
                                   bool out_f32, int variant, hipStream_t stream);

@@ -81,6 +81,32 @@ def gemm_strided(
     return out
 
 
+def gemm_tree_strided(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``out[M,N] = a[M,K] @ b[K,N]`` under the k-tree contract, arbitrary non-negative strides."""
+    m, k = a.shape
+    n = b.shape[1]
+    if m == 0 or n == 0:
+        return out
+    lib = _lib.load()
+    with torch.cuda.device(a.device):
+        status = lib.rlk_det_gemm_tree_bf16(
+            a.data_ptr(),
+            a.stride(0),
+            a.stride(1),
+            b.data_ptr(),
+            b.stride(0),
+            b.stride(1),
+            out.data_ptr(),
+            out.stride(0),
+            m,
+            n,
+            k,
+            _stream_handle(a.device),
+        )
+    _lib.check(status, "rlk_det_gemm_tree_bf16 failed")
+    return out
+
+
 def det_gemm_sm90_compiled() -> bool:
     """Always False here (csrc/cuda/gemm/det_gemm_kernel.cu:511-517): no SM90 code exists."""
     return False

@@ -50,6 +50,8 @@ EXPORTED_SYMBOLS = (
     "rlk_last_error",
     "rlk_det_gemm_bf16",
     "rlk_det_gemm_pick_config",
+    "rlk_det_gemm_tree_bf16",
+    "rlk_det_gemm_tree_contract_id",
     "rlk_linear_logp_contract_id",
     "rlk_linear_logp_split_count",
     "rlk_linear_logp_workspace_bytes",
@@ -105,6 +107,10 @@ def load() -> ctypes.CDLL:
 
     lib.rlk_det_gemm_bf16.restype = i32
     lib.rlk_det_gemm_bf16.argtypes = [vp, i64, i64, vp, i64, i64, vp, i64, i32, i32, i32, i32, i32, vp]
+    lib.rlk_det_gemm_tree_bf16.restype = i32
+    lib.rlk_det_gemm_tree_bf16.argtypes = [vp, i64, i64, vp, i64, i64, vp, i64, i32, i32, i32, vp]
+    lib.rlk_det_gemm_tree_contract_id.restype = c.c_char_p
+    lib.rlk_det_gemm_tree_contract_id.argtypes = []
     lib.rlk_det_gemm_pick_config.restype = i32
     lib.rlk_det_gemm_pick_config.argtypes = [i32, i32, i32]
 

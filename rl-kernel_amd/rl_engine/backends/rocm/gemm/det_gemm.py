@@ -1,13 +1,19 @@
 """Strict deterministic GEMM facade for ROCm, gfx950 build.
 
 Public names, argument meaning and error behaviour follow the reference facade
-(rl_engine/backends/rocm/gemm/det_gemm.py:178-197, 411-465, 491-593) and its MFMA
-host layer (rl_engine/backends/rocm/gemm/mfma_gemm.py:277-458). There is one
-backend: the HIP MFMA kernel of librlk_gfx950.so. It never falls back.
+(rl_engine/backends/rocm/gemm/det_gemm.py:32-105, 178-197, 411-465, 491-593) and its MFMA
+host layer (rl_engine/backends/rocm/gemm/mfma_gemm.py:277-458). Two contracts, both HIP
+kernels of librlk_gfx950.so, selected by ``RL_KERNEL_DET_GEMM_BACKEND`` as in the
+reference; neither ever falls back.
 
-Arithmetic: bf16 operands, one fp32 accumulator per output element updated by
-ascending 32-wide MFMA steps over the whole K range, one rounding to bf16. A
-row's result does not depend on how many other rows share the call.
+``hip_mfma`` (default; the reference's ``triton_mfma`` role): bf16 operands, one fp32
+accumulator per output element updated by ascending 32-wide MFMA steps over the whole K
+range, one rounding to bf16. A row's result does not depend on how many other rows share
+the call.
+
+``hip_tree`` (the reference's ``triton_tree`` role): fp32 scalar-FMA leaves of at most 32 K
+values rounded to bf16, combined by the bf16 midpoint tree over K. Batch invariant as well,
+and invariant to the tensor-parallel degree of a K-sharded layer; about 20 times slower.
 """
 
 from __future__ import annotations
@@ -21,31 +27,50 @@ import torch
 from rl_engine import _C, _lib
 
 _BACKEND_ENV = "RL_KERNEL_DET_GEMM_BACKEND"
+_AUTO_BACKEND = "auto"
 _HIP_BACKEND = "hip_mfma"
-# Names the reference accepts for its own backends; all of them select the one
-# implementation that exists here.
-_ACCEPTED_REQUESTS = {"auto", _HIP_BACKEND, "mfma", "triton_mfma", "rocm"}
+_TREE_BACKEND = "hip_tree"
+# Names the reference accepts (rl_engine/backends/rocm/gemm/det_gemm.py:33-48) select the
+# contract that plays the same role here; "auto" is the MFMA contract on gfx950.
+_BACKEND_ALIASES = {
+    "rocm": _TREE_BACKEND,
+    "triton": _TREE_BACKEND,
+    "tree": _TREE_BACKEND,
+    "triton_tree": _TREE_BACKEND,
+    "mfma": _HIP_BACKEND,
+    "triton_mfma": _HIP_BACKEND,
+}
 _ROUTE_REPORTED = False
 _ROUTE_REPORT_LOCK = Lock()
 _WEIGHT_TRANSPOSE_CACHE: dict[tuple[int, str, tuple[int, ...], torch.dtype], tuple[int | None, torch.Tensor]] = {}
 _WEIGHT_TRANSPOSE_CACHE_LIMIT = 256
 
 
-def _requested_backend() -> str:
-    value = os.getenv(_BACKEND_ENV, "auto").strip().lower()
-    if value not in _ACCEPTED_REQUESTS:
+def _resolve_backend_request(value: str) -> str:
+    value = value.strip().lower()
+    value = _BACKEND_ALIASES.get(value, value)
+    if value not in {_AUTO_BACKEND, _HIP_BACKEND, _TREE_BACKEND}:
         raise RuntimeError(
-            f"{_BACKEND_ENV} must be one of {sorted(_ACCEPTED_REQUESTS)} on the gfx950 build, got {value!r}"
+            f"{_BACKEND_ENV} must be '{_AUTO_BACKEND}', '{_TREE_BACKEND}' or '{_HIP_BACKEND}' "
+            f"on the gfx950 build, got {value!r}"
         )
     return value
+
+
+def _requested_backend() -> str:
+    return _resolve_backend_request(os.getenv(_BACKEND_ENV, _AUTO_BACKEND))
 
 
 _REQUESTED_BACKEND = _requested_backend()
 
 
 def det_gemm_backend() -> str:
-    """Name of the strict GEMM implementation (there is exactly one)."""
-    return _HIP_BACKEND
+    """Name of the strict GEMM implementation in use."""
+    return _TREE_BACKEND if _REQUESTED_BACKEND == _TREE_BACKEND else _HIP_BACKEND
+
+
+def _use_tree() -> bool:
+    return det_gemm_backend() == _TREE_BACKEND
 
 
 def det_gemm_fallback_reason() -> str | None:
@@ -54,7 +79,8 @@ def det_gemm_fallback_reason() -> str | None:
 
 def det_gemm_backend_id() -> str:
     """Arithmetic-contract id reported in provenance records."""
-    return _lib.load().rlk_contract_id().decode()
+    lib = _lib.load()
+    return (lib.rlk_det_gemm_tree_contract_id() if _use_tree() else lib.rlk_contract_id()).decode()
 
 
 def _report_strict_route_once() -> None:
@@ -131,6 +157,41 @@ def mfma_gemm(
     return out
 
 
+def tree_gemm(a: torch.Tensor, b: torch.Tensor, *, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``a[M,K] @ b[K,N]`` in bf16 under the k-tree contract (any strided views).
+
+    Equals the specification the reference's tests evaluate
+    (tests/ops/gemm/test_det_gemm.py:156-168) bit for bit; a contiguous half of K is
+    exactly one child of the root, so K-sharded partial results combined by bf16
+    adds in a balanced rank tree reproduce the unsharded result.
+    """
+    _validate_operands(a, b)
+    m_size, n_size = a.size(0), b.size(1)
+    if out is None:
+        out = torch.empty((m_size, n_size), dtype=torch.bfloat16, device=a.device)
+    else:
+        if tuple(out.shape) != (m_size, n_size):
+            raise ValueError(f"MFMA GEMM output must have shape {(m_size, n_size)}, got {tuple(out.shape)}")
+        if out.dtype != torch.bfloat16:
+            raise TypeError(f"MFMA GEMM output must be BF16, got {out.dtype}")
+        if out.device != a.device:
+            raise RuntimeError("MFMA GEMM output must live on the input device")
+        if out.stride(1) != 1:
+            raise ValueError("MFMA GEMM output rows must be contiguous")
+        if out.requires_grad:
+            raise ValueError("MFMA GEMM output buffer must not require gradients")
+    if m_size == 0 or n_size == 0:
+        return out
+    return _C.gemm_tree_strided(a, b, out)
+
+
+def _strict_gemm(a: torch.Tensor, b: torch.Tensor, *, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``a @ b`` under the contract selected at import."""
+    if _use_tree():
+        return tree_gemm(a, b, out=out)
+    return mfma_gemm(a, b, out=out)
+
+
 def _reduction_major(tensor: torch.Tensor) -> torch.Tensor:
     """``tensor.t()`` for a GEMM that reduces over ``tensor``'s rows: the plain view when
     the library's K-major loader can take it, else a value-preserving copy."""
@@ -139,17 +200,21 @@ def _reduction_major(tensor: torch.Tensor) -> torch.Tensor:
 
 def mfma_linear(a: torch.Tensor, weight: torch.Tensor, *, out: torch.Tensor | None = None) -> torch.Tensor:
     """``a @ weight.T`` for a native ``[N,K]`` weight, no transpose copy."""
-    return mfma_gemm(a, weight.t(), out=out)
+    return _strict_gemm(a, weight.t(), out=out)
 
 
 def mfma_linear_input_gradient(grad_output: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """``dX = dY @ W`` with ``W`` in native ``[N,K]`` layout."""
+    if _use_tree():
+        return tree_gemm(grad_output, weight)
     # The reduction runs over N, the slow axis of W: a K-major operand of the kernel.
     return mfma_gemm(grad_output, _reduction_major(weight).t())
 
 
 def mfma_linear_weight_gradient(a: torch.Tensor, grad_output: torch.Tensor) -> torch.Tensor:
     """``dW = dY.T @ X`` returned in native ``[N,K]`` layout."""
+    if _use_tree():
+        return tree_gemm(grad_output.t(), a)
     return mfma_gemm(_reduction_major(grad_output), _reduction_major(a).t())
 
 
@@ -259,7 +324,7 @@ def det_gemm_linear_prepared(a: torch.Tensor, weight_t: torch.Tensor, *, out: to
         raise ValueError("prepared deterministic linear weight must be contiguous")
     if out is not None and (torch._C._overlaps(out, a) or torch._C._overlaps(out, weight_t)):
         raise ValueError("prepared deterministic linear output must not alias its inputs")
-    return mfma_gemm(a, weight_t, out=out)
+    return _strict_gemm(a, weight_t, out=out)
 
 
 def det_gemm_linear_input_gradient(
@@ -335,12 +400,16 @@ class MfmaGemmFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         ctx.save_for_backward(a, b)
-        return mfma_gemm(a, b)
+        return _strict_gemm(a, b)
 
     @staticmethod
     def backward(ctx, grad_out: torch.Tensor):
         a, b = ctx.saved_tensors
         grad_out = _as_bf16_grad(grad_out)
+        if _use_tree():
+            da = tree_gemm(grad_out, b.t()) if ctx.needs_input_grad[0] else None
+            db = tree_gemm(a.t(), grad_out) if ctx.needs_input_grad[1] else None
+            return da, db
         da = mfma_gemm(grad_out, b.t()) if ctx.needs_input_grad[0] else None
         db = mfma_gemm(_reduction_major(a), _reduction_major(grad_out).t()) if ctx.needs_input_grad[1] else None
         return da, db
@@ -407,7 +476,7 @@ def deterministic_gemm(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     """Functional strict GEMM entry for ``[M,K] @ [K,N]``."""
     if torch.is_grad_enabled() and (a.requires_grad or b.requires_grad):
         return MfmaGemmFn.apply(a, b)
-    return mfma_gemm(a, b)
+    return _strict_gemm(a, b)
 
 
 __all__ = [
@@ -417,6 +486,7 @@ __all__ = [
     "MfmaLinearFn",
     "det_gemm_backend",
     "det_gemm_backend_id",
+    "tree_gemm",
     "det_gemm_fallback_reason",
     "det_gemm_linear",
     "det_gemm_linear_prepared",

@@ -1,0 +1,164 @@
+"""The k-tree GEMM contract on a real MI355X, through the C ABI.
+
+This contract is fully specified (fp32 scalar-FMA leaves of at most 32 K values, bf16
+midpoint tree over K; tests/ops/gemm/test_det_gemm.py:156-168 of the reference), so the
+bar is bit-exactness against the CPU oracle's restatement, not a tolerance."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+import inputs
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def gemm():
+    from rl_engine.backends.rocm.gemm import det_gemm
+
+    return det_gemm
+
+
+def _same_bits(x: torch.Tensor, y: torch.Tensor) -> bool:
+    return torch.equal(x.contiguous().view(torch.int16), y.contiguous().view(torch.int16))
+
+
+def _oracle_tree(oracle, a: torch.Tensor, w_nk: torch.Tensor) -> np.ndarray:
+    return oracle.k_tree_gemm(inputs.bits(a), inputs.bits(w_nk))
+
+
+# (M, K, N); the first three are the shapes of the reference's bitwise test
+# (tests/ops/gemm/test_det_gemm.py:510), the rest cover one leaf, uneven leaves
+# (K = 33 -> 16 + 17, K = 100 -> 25 x 4, K = 12288 -> 512 leaves of 24) and tile edges.
+TREE_SHAPES = [
+    (4, 65, 129),
+    (8, 4096, 128),
+    (4, 12288, 64),
+    (1, 1, 1),
+    (3, 32, 5),
+    (7, 33, 130),
+    (70, 100, 200),
+    (128, 1024, 1024),
+    (65, 1536, 257),
+    (16, 6144, 96),
+]
+
+
+@pytest.mark.parametrize("shape", TREE_SHAPES)
+def test_tree_gemm_is_bit_exact_against_the_oracle(gemm, oracle, shape):
+    m, k, n = shape
+    a = inputs.randn_bf16(9100 + k, m, k)
+    w = inputs.randn_bf16(9101 + k, n, k, 0.02)  # [N, K]
+    want = _oracle_tree(oracle, a, w)
+    a_d, w_d = a.to(DEV), w.to(DEV)
+    got_linear = gemm.tree_gemm(a_d, w_d.t())  # K-contiguous right-hand side
+    got_plain = gemm.tree_gemm(a_d, w_d.t().contiguous())  # B[K, N]
+    got_at = gemm.tree_gemm(a_d.t().contiguous().t(), w_d.t())  # A stored [K, M]
+    assert np.array_equal(inputs.bits(got_linear), want)
+    assert _same_bits(got_plain, got_linear) and _same_bits(got_at, got_linear)
+    assert _same_bits(gemm.tree_gemm(a_d, w_d.t()), got_linear)  # run to run
+
+
+def test_tree_gemm_differs_from_the_round_once_contract_only_by_rounding(gemm, oracle):
+    a = inputs.randn_bf16(9200, 32, 4096).to(DEV)
+    w = inputs.randn_bf16(9201, 256, 4096, 0.02).to(DEV)
+    tree = gemm.tree_gemm(a, w.t()).float()
+    once = gemm.mfma_gemm(a, w.t()).float()
+    assert not torch.equal(tree, once)  # two different contracts
+    assert float((tree - once).abs().max()) <= 0.05 * float(once.abs().max())  # the reference's reduction atol scale
+
+
+def test_tree_rows_are_batch_invariant(gemm):
+    a = inputs.randn_bf16(9300, 300, 2048).to(DEV)
+    w = inputs.randn_bf16(9301, 384, 2048, 0.02).to(DEV)
+    full = gemm.tree_gemm(a, w.t())
+    for lo, hi in ((0, 1), (37, 38), (0, 7), (100, 229), (299, 300)):
+        assert _same_bits(gemm.tree_gemm(a[lo:hi], w.t()), full[lo:hi]), (lo, hi)
+    perm = torch.randperm(300, generator=torch.Generator().manual_seed(9302)).to(DEV)
+    assert _same_bits(gemm.tree_gemm(a[perm], w.t()), full[perm])
+
+
+@pytest.mark.parametrize("k", (2048, 12288, 1000))
+def test_k_shards_combined_by_bf16_adds_reproduce_the_unsharded_result(gemm, k):
+    # The purpose of the contract (tests/ops/gemm/test_det_gemm.py:276-300): a contiguous half of K
+    # is exactly one child of the root, a quarter one grandchild.
+    a = inputs.randn_bf16(9400 + k, 24, k).to(DEV)
+    w = inputs.randn_bf16(9401 + k, 160, k, 0.02).to(DEV)
+    full = gemm.tree_gemm(a, w.t())
+    h = k // 2
+    halves = gemm.tree_gemm(a[:, :h], w[:, :h].t()) + gemm.tree_gemm(a[:, h:], w[:, h:].t())  # torch bf16 add
+    assert _same_bits(halves, full)
+    q0, q1 = h // 2, h + (k - h) // 2
+    cuts = [0, q0, h, q1, k]
+    parts = [gemm.tree_gemm(a[:, cuts[i] : cuts[i + 1]], w[:, cuts[i] : cuts[i + 1]].t()) for i in range(4)]
+    assert _same_bits((parts[0] + parts[1]) + (parts[2] + parts[3]), full)
+
+
+def test_tree_special_values(gemm, oracle):
+    # Finite extremes value-exact against the oracle; Inf / NaN surface as Inf / NaN in the same places.
+    finite = np.array([0x0000, 0x8000, 0x3F80, 0xBF80, 0x0080, 0x8080, 0x0001, 0x7F7F, 0xFF7F, 0x4000, 0x3F00], dtype=np.uint16)
+    rng = np.random.default_rng(9500)
+    for k in (1, 31, 32, 33, 64, 200):
+        a_bits = rng.choice(finite, size=(5, k))
+        w_bits = rng.choice(np.array([0x0000, 0x8000, 0x3F80, 0xBF80, 0x0080, 0x0001], dtype=np.uint16), size=(9, k))
+        got = gemm.tree_gemm(inputs.from_bits(a_bits, DEV), inputs.from_bits(w_bits, DEV).t())
+        want = oracle.k_tree_gemm(a_bits, w_bits)
+        got_bits = inputs.bits(got)
+        want_nan = (want & 0x7FFF) > 0x7F80
+        got_nan = (got_bits & 0x7FFF) > 0x7F80
+        assert np.array_equal(got_nan, want_nan), k
+        assert np.array_equal(got_bits[~want_nan], want[~want_nan]), k
+    a_bits = rng.choice(finite[:6], size=(4, 96)).astype(np.uint16)
+    a_bits[1, 40] = 0x7F80  # +inf
+    a_bits[2, 70] = 0x7FC1  # NaN
+    w_bits = rng.choice(np.array([0x3F80, 0xBF80, 0x4000], dtype=np.uint16), size=(6, 96))
+    got = gemm.tree_gemm(inputs.from_bits(a_bits, DEV), inputs.from_bits(w_bits, DEV).t()).float().cpu()
+    assert bool(torch.isfinite(got[0]).all()) and bool(torch.isinf(got[1]).all()) and bool(torch.isnan(got[2]).all())
+
+
+def test_tree_out_argument_empty_shapes_and_errors(gemm):
+    a = inputs.randn_bf16(9600, 20, 256).to(DEV)
+    w = inputs.randn_bf16(9601, 48, 256, 0.02).to(DEV)
+    base = gemm.tree_gemm(a, w.t())
+    staging = torch.zeros((20, 64), dtype=torch.bfloat16, device=DEV)
+    out = gemm.tree_gemm(a, w.t(), out=staging.narrow(1, 8, 48))
+    assert out.data_ptr() == staging.data_ptr() + 16 and _same_bits(out, base)
+    assert bool((staging[:, :8] == 0).all()) and bool((staging[:, 56:] == 0).all())
+    assert gemm.tree_gemm(a[:0], w.t()).shape == (0, 48)
+    zero_k = gemm.tree_gemm(a[:, :0], w[:, :0].t())
+    assert zero_k.shape == (20, 48) and bool((zero_k == 0).all())
+    with pytest.raises(ValueError):
+        gemm.tree_gemm(a, w)  # K mismatch
+    with pytest.raises(TypeError):
+        gemm.tree_gemm(a.float(), w.t().float())
+
+
+def test_tree_gradient_forms_are_the_tree_over_their_own_reduction_axis(gemm, oracle):
+    # dX = dY @ W reduces over N, dW = dY^T @ X over tokens (tests/ops/gemm/test_det_gemm.py:538-541).
+    m, n, k = 96, 160, 192
+    x = inputs.randn_bf16(9700, m, k)
+    w = inputs.randn_bf16(9701, n, k, 0.05)
+    dy = inputs.randn_bf16(9702, m, n)
+    dx = gemm.tree_gemm(dy.to(DEV), w.to(DEV))
+    dw = gemm.tree_gemm(dy.to(DEV).t(), x.to(DEV))
+    assert np.array_equal(inputs.bits(dx), oracle.k_tree_gemm(inputs.bits(dy), inputs.bits(w.t().contiguous())))
+    assert np.array_equal(inputs.bits(dw), oracle.k_tree_gemm(inputs.bits(dy.t().contiguous()), inputs.bits(x.t().contiguous())))
+
+
+def test_tree_contract_id_and_backend_names(gemm):
+    from rl_engine import _lib
+
+    lib = _lib.load()
+    assert lib.rlk_det_gemm_tree_contract_id().decode() == "rlkernel.det_gemm.hip_ktree32_gfx950.v1"
+    assert gemm._resolve_backend_request("tree") == "hip_tree"
+    assert gemm._resolve_backend_request("triton_tree") == "hip_tree"
+    assert gemm._resolve_backend_request("rocm") == "hip_tree"
+    assert gemm._resolve_backend_request("triton_mfma") == "hip_mfma"
+    assert gemm._resolve_backend_request("auto") == "auto"
+    with pytest.raises(RuntimeError):
+        gemm._resolve_backend_request("cublas")
