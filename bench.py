@@ -53,7 +53,7 @@ def _parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-logp", action="store_true", help="skip the linear-LogP leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-T table")
-    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|logp|logp_bwd|from_logits|ffn|copy (used for profiling)")
+    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|logp|logp_decode|logp_mid|logp_bwd|from_logits|ffn|tree|copy (used for profiling)")
     return ap.parse_args()
 
 
@@ -147,6 +147,21 @@ def main() -> int:
         tgt = torch.randint(0, VOCAB, (tl,), generator=gen, device=dev)
         ms = _time_calls(lambda: deterministic_linear_logp(hid, w_lm, tgt), args.steps, args.warmup)
         print(json.dumps({"leg": "logp", "ms": ms, "tokens_per_s": tl / ms * 1e3, "launches": args.steps + args.warmup}))
+        return 0
+    if args.only in ("logp_decode", "logp_mid"):
+        # the stream-group grid: 16 tokens (decode) or 512 tokens against the full vocabulary
+        tl = 16 if args.only == "logp_decode" else 512
+        hid = randn(tl, HIDDEN)
+        w_lm = randn(VOCAB, HIDDEN, 0.02)
+        tgt = torch.randint(0, VOCAB, (tl,), generator=gen, device=dev)
+        ms = _time_calls(lambda: deterministic_linear_logp(hid, w_lm, tgt), args.steps, args.warmup)
+        print(json.dumps({"leg": args.only, "tokens": tl, "ms": ms, "weight_gbps": 2.0 * VOCAB * HIDDEN / ms * 1e-6,
+                          "launches": args.steps + args.warmup}))
+        return 0
+    if args.only == "tree":
+        ms = _time_calls(lambda: gemm.tree_gemm(x, w_gu.t(), out=out_gu), args.steps, args.warmup)
+        print(json.dumps({"leg": "tree", "ms": ms, "tflops": 2.0 * T * 2 * INTER * HIDDEN / ms * 1e-9,
+                          "launches": args.steps + args.warmup}))
         return 0
     if args.only in ("logp_bwd", "from_logits"):
         from rl_engine import _C
