@@ -99,6 +99,31 @@ def test_k_shards_combined_by_bf16_adds_reproduce_the_unsharded_result(gemm, k):
     assert _same_bits((parts[0] + parts[1]) + (parts[2] + parts[3]), full)
 
 
+def test_simulated_tp_left_fold_differs_and_tp2_is_batch_invariant(gemm):
+    # The reference's simulated tensor parallelism (tests/distributed/tp/test_det_gemm_simulated_tp.py:58-102):
+    # eight K shards folded left to right are a different parenthesisation from the kernel's tree and must
+    # diverge; two shards added once match the unsharded result for a row alone and inside a batch.
+    m, k, n = 16, 256, 64
+    a = inputs.randn_bf16(9450, m, k).to(DEV)
+    b = inputs.randn_bf16(9451, k, n).to(DEV)
+    full = gemm.tree_gemm(a, b)
+    width = k // 8
+    parts = [gemm.tree_gemm(a[:, i * width : (i + 1) * width], b[i * width : (i + 1) * width]) for i in range(8)]
+    folded = parts[0]
+    for part in parts[1:]:
+        folded = folded + part
+    assert int((full != folded).sum()) > 0
+    balanced = ((parts[0] + parts[1]) + (parts[2] + parts[3])) + ((parts[4] + parts[5]) + (parts[6] + parts[7]))
+    assert _same_bits(balanced, full)
+
+    def tp2(x):
+        return gemm.tree_gemm(x[:, : k // 2], b[: k // 2]) + gemm.tree_gemm(x[:, k // 2 :], b[k // 2 :])
+
+    big = inputs.randn_bf16(9452, 32, k).to(DEV)
+    row = big[:1].clone()
+    assert _same_bits(tp2(row)[0], tp2(big)[0]) and _same_bits(tp2(row)[0], gemm.tree_gemm(big, b)[0])
+
+
 def test_tree_special_values(gemm, oracle):
     # Finite extremes value-exact against the oracle; Inf / NaN surface as Inf / NaN in the same places.
     finite = np.array([0x0000, 0x8000, 0x3F80, 0xBF80, 0x0080, 0x8080, 0x0001, 0x7F7F, 0xFF7F, 0x4000, 0x3F00], dtype=np.uint16)
@@ -162,3 +187,33 @@ def test_tree_contract_id_and_backend_names(gemm):
     assert gemm._resolve_backend_request("auto") == "auto"
     with pytest.raises(RuntimeError):
         gemm._resolve_backend_request("cublas")
+
+
+def test_tree_backend_routes_the_whole_facade(gemm, oracle, monkeypatch):
+    # RL_KERNEL_DET_GEMM_BACKEND is read at import; switching the resolved request exercises the same routing.
+    monkeypatch.setattr(gemm, "_REQUESTED_BACKEND", "hip_tree")
+    assert gemm.det_gemm_backend() == "hip_tree"
+    assert gemm.det_gemm_backend_id() == "rlkernel.det_gemm.hip_ktree32_gfx950.v1"
+    m, n, k = 40, 72, 320
+    x = inputs.randn_bf16(9800, m, k)
+    w = inputs.randn_bf16(9801, n, k, 0.05)
+    dy = inputs.randn_bf16(9802, m, n)
+    want = oracle.k_tree_gemm(inputs.bits(x), inputs.bits(w))
+    xd = x.to(DEV).requires_grad_(True)
+    wd = w.to(DEV).requires_grad_(True)
+    op = gemm.DetGemmOp()
+    y = op.linear(xd, wd)
+    assert np.array_equal(inputs.bits(y.detach()), want)
+    assert np.array_equal(inputs.bits(gemm.det_gemm_linear(x.to(DEV), w.to(DEV))), want)
+    assert np.array_equal(inputs.bits(gemm.deterministic_gemm(x.to(DEV), w.to(DEV).t())), want)
+    y.backward(dy.to(DEV))
+    want_dx = oracle.k_tree_gemm(inputs.bits(dy), inputs.bits(w.t().contiguous()))
+    want_dw = oracle.k_tree_gemm(inputs.bits(dy.t().contiguous()), inputs.bits(x.t().contiguous()))
+    assert np.array_equal(inputs.bits(xd.grad), want_dx) and np.array_equal(inputs.bits(wd.grad), want_dw)
+    a2 = x.to(DEV).requires_grad_(True)
+    b2 = w.to(DEV).t().contiguous().requires_grad_(True)  # [K, N]
+    gemm.deterministic_gemm(a2, b2).backward(dy.to(DEV))
+    assert np.array_equal(inputs.bits(a2.grad), want_dx)
+    assert np.array_equal(inputs.bits(b2.grad), oracle.k_tree_gemm(inputs.bits(x.t().contiguous()), inputs.bits(dy.t().contiguous())))
+    monkeypatch.setattr(gemm, "_REQUESTED_BACKEND", "auto")
+    assert gemm.det_gemm_backend() == "hip_mfma"
