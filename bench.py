@@ -74,6 +74,23 @@ def _time_calls(fn, iters: int, warmup: int) -> float:
     return start.elapsed_time(stop) / iters
 
 
+def _launch_percentiles(fn, iters: int, warmup: int) -> dict:
+    """Median and 95th percentile of single launches (one HIP event pair per launch), in ms."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    torch.cuda.synchronize()
+    for start, stop in pairs:
+        start.record()
+        fn()
+        stop.record()
+    torch.cuda.synchronize()
+    times = sorted(start.elapsed_time(stop) for start, stop in pairs)
+    return {"median_ms": round(times[len(times) // 2], 4), "p95_ms": round(times[min(len(times) - 1, int(0.95 * len(times)))], 4)}
+
+
 def _gemm_bytes(m, n, k):
     return 2.0 * (m * k + n * k + m * n)
 
@@ -220,6 +237,7 @@ def main() -> int:
         "flops_per_launch": flops_gu,
         "traffic": MEASURED_TRAFFIC_BYTES["det_gemm_gate_up_T4096"],
     }
+    roofline.update(_launch_percentiles(gate_up, args.steps, 5))
 
     result = {
         "metric": "bf16 det-GEMM TFLOP/s at Qwen3-8B FFN shapes (gate_up + down, T=4096)",
