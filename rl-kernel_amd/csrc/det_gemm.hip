@@ -157,15 +157,9 @@ static hipError_t launch_tile(const MatView& W, const MatView& X, void* C, int64
                               hipStream_t stream) {
   auto kernel = det_gemm_kernel<S, LOOP, OUT_F32, KS>;
   constexpr int kLds = KS * S::kLdsBytes;
-  static bool configured[kMaxDevices] = {};
-  int dev = 0;
-  hipError_t err = hipGetDevice(&dev);
+  static PerDeviceOnce once;
+  hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLds, once);
   if (err != hipSuccess) return err;
-  if (dev >= 0 && dev < kMaxDevices && !configured[dev]) {
-    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (err != hipSuccess) return err;
-    configured[dev] = true;
-  }
   const int tiles_m = (M + S::BM - 1) / S::BM;
   const int tiles_n = (N + S::BN - 1) / S::BN;
   int group_m = tiles_m < 8 ? tiles_m : 8;

@@ -149,16 +149,9 @@ static hipError_t launch_stream(const MatView& W, const MatView& X, void* C, int
                                 hipStream_t stream) {
   auto kernel = det_gemm_stream_kernel<KT, RING, HALF_X, OUT_F32>;
   constexpr int kLds = RING * 2 * KT * 16 * kRowBytes;
-  static bool configured[kMaxDevices] = {};
-  int dev = 0;
-  hipError_t err = hipGetDevice(&dev);
+  static PerDeviceOnce once;
+  hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLds, once);
   if (err != hipSuccess) return err;
-  if (dev >= 0 && dev < kMaxDevices && !configured[dev]) {
-    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              kLds);
-    if (err != hipSuccess) return err;
-    configured[dev] = true;
-  }
   hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(320), kLds, stream, W, X, C, ldc, M, N, K);
   return hipGetLastError();
 }

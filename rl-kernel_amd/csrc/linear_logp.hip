@@ -408,16 +408,9 @@ static hipError_t launch_logp(LogpArgs a, hipStream_t stream) {
   auto kernel = linear_logp_partial_kernel<S, LOOP>;
   constexpr int kMergeBytes = 3 * kLogpStreams * S::BM * (int)sizeof(float);
   constexpr int kLds = S::kLdsBytes > kMergeBytes ? S::kLdsBytes : kMergeBytes;
-  static bool configured[kMaxDevices] = {};
-  int dev = 0;
-  hipError_t err = hipGetDevice(&dev);
+  static PerDeviceOnce once;
+  hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLds, once);
   if (err != hipSuccess) return err;
-  if (dev >= 0 && dev < kMaxDevices && !configured[dev]) {
-    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              kLds);
-    if (err != hipSuccess) return err;
-    configured[dev] = true;
-  }
   a.tiles_m = (a.T + S::BM - 1) / S::BM;
   a.group_m = a.tiles_m < 8 ? a.tiles_m : 8;
   hipLaunchKernelGGL(kernel, dim3(a.tiles_m * a.n_split), dim3(S::kThreads), kLds, stream, a);
@@ -427,16 +420,9 @@ static hipError_t launch_logp(LogpArgs a, hipStream_t stream) {
 template <class S>
 static hipError_t launch_streamgroup(LogpArgs a, hipStream_t stream) {
   auto kernel = linear_logp_streamgroup_kernel<S>;
-  static bool configured[kMaxDevices] = {};
-  int dev = 0;
-  hipError_t err = hipGetDevice(&dev);
+  static PerDeviceOnce once;
+  hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), S::kLdsBytes, once);
   if (err != hipSuccess) return err;
-  if (dev >= 0 && dev < kMaxDevices && !configured[dev]) {
-    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              S::kLdsBytes);
-    if (err != hipSuccess) return err;
-    configured[dev] = true;
-  }
   a.tiles_m = (a.T + S::BM - 1) / S::BM;
   float* spart = a.part + (size_t)3 * a.n_split * a.T;  // behind the per-split partials
   hipLaunchKernelGGL(kernel, dim3(a.tiles_m * a.n_split * (kLogpStreams / 4)), dim3(S::kThreads), S::kLdsBytes, stream,

@@ -182,16 +182,9 @@ size_t linear_logp_bwd_workspace_bytes(int T, int V, bool with_bias) {
 template <class S, int LOOP>
 static hipError_t launch_dlogits(LogpBwdArgs a, hipStream_t stream) {
   auto kernel = linear_logp_dlogits_kernel<S, LOOP>;
-  static bool configured[kMaxDevices] = {};
-  int dev = 0;
-  hipError_t err = hipGetDevice(&dev);
+  static PerDeviceOnce once;
+  hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), S::kLdsBytes, once);
   if (err != hipSuccess) return err;
-  if (dev >= 0 && dev < kMaxDevices && !configured[dev]) {
-    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              S::kLdsBytes);
-    if (err != hipSuccess) return err;
-    configured[dev] = true;
-  }
   a.tiles_m = (a.T + S::BM - 1) / S::BM;
   a.tiles_v = (a.V + kLogpTileCols - 1) / kLogpTileCols;
   a.group_m = a.tiles_m < 8 ? a.tiles_m : 8;

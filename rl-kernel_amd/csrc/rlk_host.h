@@ -4,12 +4,32 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/rlk.h"
 #include "det_gemm_tile.h"
 
 namespace rlk {
 
 constexpr int kMaxDevices = 64;
+
+// Raises a kernel's dynamic-LDS limit once per device (the attribute is per device and
+// sticky). Safe to call from several host threads: the flag is only ever set after the
+// attribute call has succeeded, and setting the attribute twice is harmless.
+struct PerDeviceOnce {
+  std::atomic<bool> done[kMaxDevices];
+};
+
+inline hipError_t allow_dynamic_lds(const void* kernel, int bytes, PerDeviceOnce& once) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  const bool tracked = dev >= 0 && dev < kMaxDevices;
+  if (tracked && once.done[dev].load(std::memory_order_acquire)) return hipSuccess;
+  err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (err == hipSuccess && tracked) once.done[dev].store(true, std::memory_order_release);
+  return err;
+}
 
 int pick_det_gemm_config(int M, int N, int K);
 

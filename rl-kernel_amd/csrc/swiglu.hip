@@ -191,16 +191,9 @@ template <class S>
 static hipError_t launch_gated(const MatView& W, const MatView& X, void* Y, int64_t ldy, int M, int I, int K,
                                hipStream_t stream) {
   auto kernel = det_gemm_swiglu_kernel<S>;
-  static bool configured[kMaxDevices] = {};
-  int dev = 0;
-  hipError_t err = hipGetDevice(&dev);
+  static PerDeviceOnce once;
+  hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), S::kLdsBytes, once);
   if (err != hipSuccess) return err;
-  if (dev >= 0 && dev < kMaxDevices && !configured[dev]) {
-    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              S::kLdsBytes);
-    if (err != hipSuccess) return err;
-    configured[dev] = true;
-  }
   const int tiles_m = (M + S::BM - 1) / S::BM;
   const int tiles_n = (I + S::BN / 2 - 1) / (S::BN / 2);
   const int group_m = tiles_m < 8 ? tiles_m : 8;
