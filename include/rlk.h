@@ -44,13 +44,14 @@ typedef enum rlk_gemm_config {
   RLK_GEMM_CFG_64x64 = 5,
   RLK_GEMM_CFG_64x16 = 6,
   RLK_GEMM_CFG_16x16 = 7,
-  RLK_GEMM_CFG_STREAM16_DEEP = 8, /* M <= 16: 16-feature panel per workgroup, 512-wide ring stages */
-  RLK_GEMM_CFG_STREAM16 = 9,      /* M <= 16: same with 256-wide ring stages, two workgroups per CU */
+  RLK_GEMM_CFG_STREAM16_DEEP = 8, /* M <= 16: 16-feature panel per workgroup streamed through a 128 KiB LDS ring */
+  RLK_GEMM_CFG_STREAM16 = 9,      /* M <= 16: same with a 64 KiB ring, two workgroups per CU */
   RLK_GEMM_CFG_256x64 = 10,
   RLK_GEMM_CFG_64x64_DEEP = 11,   /* 64x64 tile, 256 K values per barrier pair (few, long tiles) */
   RLK_GEMM_CFG_128x64_DEEP = 12,  /* 128x64 tile, 128 K values per barrier pair */
   RLK_GEMM_CFG_128x128_DEEP = 13, /* 128x128 tile, 128 K values per barrier pair */
-  RLK_GEMM_CFG_COUNT = 14,
+  RLK_GEMM_CFG_STREAM64 = 14,     /* M <= 64: 16-feature panels streamed through an LDS ring, one consumer wave per 16 tokens */
+  RLK_GEMM_CFG_COUNT = 15,
   /* OR-ed into a configuration: use the register-staged main loop even where the
    * direct-to-LDS ping-pong loop applies. Bit-neutral; exists so tests can
    * compare the two loops. */
@@ -284,7 +285,7 @@ int rlk_swiglu_bwd(const void* dy, int64_t ld_dy, const void* gate, int64_t ld_g
                    void* d_gate, int64_t ld_d_gate, void* d_up, int64_t ld_d_up, int rows, int cols, void* stream);
 
 /* Bytes of workspace rlk_det_gemm_swiglu_bf16 needs for these operands: 0 when the fused
- * kernel applies (unit K strides, 16-byte aligned rows, K % 64 == 0, M > 16), else the
+ * kernel applies (unit K strides, 16-byte aligned rows, K % 64 == 0, M > 128), else the
  * bf16 [M, 2 I] projection. */
 size_t rlk_det_gemm_swiglu_workspace_bytes(const void* a, int64_t a_row_stride, const void* w_packed,
                                            int64_t w_row_stride, int M, int I, int K);

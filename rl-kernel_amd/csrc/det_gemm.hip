@@ -231,7 +231,14 @@ int pick_det_gemm_config(int M, int N, int K) {
   constexpr int kCus = 256;
   // Decode: many short panels keep the chip busy with one wave each; few long
   // panels need the streaming kernel's deep ring.
-  if (M <= 16) return N >= 64 * kCus ? RLK_GEMM_CFG_16x16 : RLK_GEMM_CFG_STREAM16_DEEP;
+  // Decode: many short panels keep the chip busy with one wave each; few long panels need
+  // the streaming kernel's deep ring (one 16-feature panel per workgroup). Up to 32 / 64
+  // tokens the same holds while there are at most 1.5 / 1 panels per CU: a 64-token tile
+  // kernel would run on N / 64 CUs only (down projection at 32 tokens: 38 -> 19 us). A CU's
+  // direct-to-LDS path moves about 31 bytes per clock, which bounds both kernels.
+  if (M <= 16) return N >= 64 * kCus ? RLK_GEMM_CFG_16x16 : RLK_GEMM_CFG_STREAM64;
+  if (K >= 1024 && K % kTileK == 0 && ((M <= 32 && N <= 24 * kCus) || (M <= 64 && N <= 16 * kCus)))
+    return RLK_GEMM_CFG_STREAM64;
   // Problems that give the chip at most one small tile per CU: the deep-stage variants
   // (one workgroup per CU, several K tiles per barrier pair) beat the same tile run several
   // workgroups per CU. Smallest tile first: it spreads the weight stream over most CUs.
@@ -310,13 +317,14 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
     }
   }
   if (config == RLK_GEMM_CFG_AUTO) config = pick_det_gemm_config(M, N, K);
-  if (config == RLK_GEMM_CFG_STREAM16_DEEP || config == RLK_GEMM_CFG_STREAM16) {
-    // The streaming kernel serves one 16-token tile and needs the fast layout; otherwise the
-    // 16x16 tile kernel computes the same bits.
-    if (M <= 16 && vec && allow_pingpong && K % kTileK == 0) {
-      return det_gemm_stream_launch(W, X, C, ldc, M, N, K, out_f32, config == RLK_GEMM_CFG_STREAM16 ? 1 : 0, stream);
-    }
-    config = M <= 16 ? RLK_GEMM_CFG_16x16 : pick_det_gemm_config(M, N, K);
+  if (config == RLK_GEMM_CFG_STREAM16_DEEP || config == RLK_GEMM_CFG_STREAM16 || config == RLK_GEMM_CFG_STREAM64) {
+    // The streaming kernel serves up to 16 (STREAM16*) or 64 tokens and needs the fast layout;
+    // otherwise a tile kernel computes the same bits.
+    const int max_m = config == RLK_GEMM_CFG_STREAM64 ? 64 : 16;
+    if (M <= max_m && vec && allow_pingpong && K % kTileK == 0)
+      return det_gemm_stream_launch(W, X, C, ldc, M, N, K, out_f32, config == RLK_GEMM_CFG_STREAM16, stream);
+    config = M <= 16 ? RLK_GEMM_CFG_16x16 : M <= 64 ? RLK_GEMM_CFG_64x64 : pick_det_gemm_config(M, N, K);
+    if (config == RLK_GEMM_CFG_STREAM64) config = RLK_GEMM_CFG_64x64;
   }
   // Deep-stage variants need the fast layout and whole stages; otherwise the plain shape
   // computes the same bits.

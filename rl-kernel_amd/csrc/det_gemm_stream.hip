@@ -1,78 +1,76 @@
-// det_gemm for decode-sized batches (M <= 16): one workgroup streams a 16-feature
-// weight panel through a deep LDS ring while a single wave runs the MFMA chain.
+// det_gemm for up to 64 tokens against few, long weight panels: one workgroup streams a
+// 16-feature weight panel through a deep LDS ring while one wave per 16-token tile runs the
+// MFMA chain.
 //
-// With M <= 16 the GEMM is a read of W at HBM speed. The contract allows no
-// split-K, so the K/32 MFMA steps of an output element run one after the other
-// in one wave, and a 16-row panel is the finest unit of work (N / 16 workgroups:
-// 256 for the Qwen3-8B down projection, one per CU). To keep enough bytes in
-// flight with one workgroup per CU, four producer waves issue direct-to-LDS loads
-// several stages (of 256 or 512 K values) ahead; a fifth wave only reads fragments
-// and issues the dependent MFMA chain, which is short (K/32 steps of ~21 cycles).
-// The vector-memory front end of a CU retires about one 1 KiB load per 33 cycles,
-// so the loop is bound by the number of loads: the consumer issues none, and for
-// M <= 8 only half of each activation sub-tile is fetched (the upper eight MFMA
-// columns then hold stale LDS; columns are independent and never stored).
-// Same instruction, same ascending K order, same zero start as every other
-// det_gemm kernel, so the bits match.
+// With M <= 64 the GEMM is a read of W at HBM speed. The contract allows no split-K, so the
+// K/32 MFMA steps of an output element run one after the other in one wave, and a 16-row
+// panel is the finest unit of work (N / 16 workgroups: 256 for the Qwen3-8B down projection,
+// one per CU). To keep enough bytes in flight with one workgroup per CU, four producer waves
+// issue direct-to-LDS loads several stages ahead; the consumer waves only read fragments and
+// issue the dependent MFMA chain, which is short (K/32 steps of ~21 cycles). The vector-memory
+// front end of a CU retires about one 1 KiB load per 33 cycles (about 31 bytes per clock), so
+// the loop is bound by the number of loads and the consumers issue none. Same instruction,
+// same ascending K order, same zero start as every other det_gemm kernel, so the bits match.
 #include "det_gemm_tile.h"
 #include "rlk_host.h"
 
 namespace rlk {
 
-// KT: 64-wide K sub-tiles per ring stage; RING: stages in the ring; HALF_X: M <= 8.
-template <int KT, int RING, bool HALF_X, bool OUT_F32>
-__global__ __launch_bounds__(320) void det_gemm_stream_kernel(MatView W, MatView X, void* __restrict__ C, int64_t ldc,
-                                                               int M, int N, int K) {
-  constexpr int kSubBytes = 16 * kRowBytes;        // one operand, one 64-wide sub-tile: 16 rows x 128 B
-  constexpr int kStageBytes = 2 * KT * kSubBytes;  // W sub-tiles, then X sub-tiles
-  constexpr int kProducers = 4;
-  // 1 KiB blocks per stage: 2 KT of weights, then 2 KT (or, HALF_X, KT) of activations.
-  constexpr int kBlocksPerStage = HALF_X ? 3 * KT : 4 * KT;
-  constexpr int kLoads = kBlocksPerStage / kProducers;  // per producer wave per stage
-  static_assert(RING >= 2 && kBlocksPerStage % kProducers == 0, "ring geometry");
+// MT token tiles of 16 rows. Wave t < MT is the consumer of token tile t (its own MFMA chain
+// over the shared weight fragments), the next four waves are the producers. A stage holds KT
+// weight sub-tiles (64 K values each), then KT sub-tiles per token tile; a producer always
+// fetches the same 8-row half (producer & 1) of the (tile, sub-tile) pairs
+// (producer >> 1) + 2 j. Rows past M or N are clamped to the last valid row: computed, never
+// stored (MFMA columns and rows are independent).
+template <int KT, int RING, int MT, bool OUT_F32>
+__global__ __launch_bounds__(64 * (MT + 4)) void det_gemm_stream_kernel(MatView W, MatView X,
+                                                                              void* __restrict__ C, int64_t ldc, int M,
+                                                                              int N, int K) {
+  constexpr int kSubBytes = 16 * kRowBytes;
+  constexpr int kPairs = KT * (1 + MT);
+  constexpr int kStageBytes = kPairs * kSubBytes;
+  constexpr int kLoads = kPairs / 2;  // per producer wave per stage
+  static_assert(RING >= 2 && kPairs % 2 == 0 && MT >= 1 && MT <= 4, "ring geometry");
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // 0: consumer, 1..4: producers
-  const int producer = wave - 1;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // [0, MT): consumers, then 4 producers
+  const int producer = wave - MT;
   const int n0 = blockIdx.x * 16;
-  const int nsub = K / kTileK;               // K % 64 == 0 on this path
+  const int nsub = K / kTileK;  // K % 64 == 0 on this path
   const int nstage = (nsub + KT - 1) / KT;
 
-  // This lane's source row / chunk for a block of 8 rows.
+  // Producer: this lane's row inside a 16-row tile and its 16-byte chunk.
   const int rib = lane >> 3;
   const int chunk_elems = ((lane & 7) ^ rib) * kChunkElems;
-  const bf16_bits* w_src[2];
-  const bf16_bits* x_src[2];
+  const int half = producer & 1;
+  const int r16 = half * 8 + rib;
+  const int wr = n0 + r16 < N ? n0 + r16 : N - 1;  // rows past an edge are computed, never stored
+  const bf16_bits* w_base = W.ptr + (int64_t)wr * W.row_stride + chunk_elems;
+  const bf16_bits* x_base[MT];
 #pragma unroll
-  for (int blk = 0; blk < 2; ++blk) {
-    int wr = n0 + blk * 8 + rib;
-    wr = wr < N ? wr : N - 1;  // rows past the edge are computed, never stored
-    int xr = blk * 8 + rib;
-    xr = xr < M ? xr : M - 1;
-    w_src[blk] = W.ptr + (int64_t)wr * W.row_stride + chunk_elems;
-    x_src[blk] = X.ptr + (int64_t)xr * X.row_stride + chunk_elems;
+  for (int t = 0; t < MT; ++t) {
+    const int xr = t * 16 + r16 < M ? t * 16 + r16 : M - 1;
+    x_base[t] = X.ptr + (int64_t)xr * X.row_stride + chunk_elems;
   }
 
-  // Load j of producer p in a stage is entry p + 4 j of the stage's block list:
-  // [0, 2 KT) weight blocks (sub-tile = e / 2, half = e % 2), then the token blocks
-  // (both halves of every sub-tile, or with HALF_X only the lower half).
   auto issue_stage = [&](int s) {
     if (producer < 0) return;
     char* base = lds + (s % RING) * kStageBytes;
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
-      const int e = producer + kProducers * j;
-      const bool is_w = e < 2 * KT;
-      const int local = is_w ? e : (HALF_X ? 2 * (e - 2 * KT) : e - 2 * KT);
-      const int sub = local >> 1;
-      const int blk = local & 1;
-      const int idx = (is_w ? 0 : 2 * KT) + local;  // 1 KiB slot inside the stage
+      const int q = (producer >> 1) + 2 * j;  // pair: [0, KT) weights, then KT per token tile
+      const bool is_w = q < KT;
+      const int tile = is_w ? 0 : (q - KT) / KT;
+      const int sub = is_w ? q : (q - KT) % KT;
       int ks = s * KT + sub;
       ks = ks < nsub ? ks : nsub - 1;  // past the end: re-fetch the last sub-tile (never consumed)
-      const bf16_bits* src = (is_w ? w_src[blk] : x_src[blk]) + ks * kTileK;
-      __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(base + idx * 1024), 16, 0, 0);
+      const bf16_bits* row = w_base;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) row = (!is_w && tile == t) ? x_base[t] : row;
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(row + ks * kTileK), (lds_ptr_t)(base + (2 * q + half) * 1024), 16,
+                                       0, 0);
     }
   };
 
@@ -86,19 +84,17 @@ __global__ __launch_bounds__(320) void det_gemm_stream_kernel(MatView W, MatView
   for (int s = 0; s < RING - 1; ++s) issue_stage(s);
   for (int s = 0; s < nstage; ++s) {
     __builtin_amdgcn_s_waitcnt(wait_vmcnt((RING - 2) * kLoads));  // my loads of stage s have landed
-    wg_barrier();  // stage s is complete; the consumer is done with stage s - 1
+    wg_barrier();  // stage s is complete; the consumers are done with stage s - 1
     issue_stage(s + RING - 1);
-    if (wave == 0) {
+    if (wave < MT) {
       const char* base = lds + (s % RING) * kStageBytes;
       const int remaining = nsub - s * KT;
       const int count = remaining < KT ? remaining : KT;
-      // All fragments of the stage first (2 KT reads per operand in flight at once), then the
-      // dependent MFMA chain; the scheduling barrier keeps the compiler from serialising them.
       u32x4_t wf[2 * KT], xf[2 * KT];
 #pragma unroll
       for (int sub = 0; sub < KT; ++sub) {
         const char* wt = base + sub * kSubBytes;
-        const char* xt = base + (KT + sub) * kSubBytes;
+        const char* xt = base + (KT + wave * KT + sub) * kSubBytes;
         wf[2 * sub] = *reinterpret_cast<const u32x4_t*>(wt + frag_lo);
         xf[2 * sub] = *reinterpret_cast<const u32x4_t*>(xt + frag_lo);
         wf[2 * sub + 1] = *reinterpret_cast<const u32x4_t*>(wt + frag_hi);
@@ -106,30 +102,25 @@ __global__ __launch_bounds__(320) void det_gemm_stream_kernel(MatView W, MatView
       }
       __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
       __builtin_amdgcn_sched_barrier(0);
-      if (count == KT) {
 #pragma unroll
-        for (int i = 0; i < 2 * KT; ++i) acc = mfma_16x16x32(wf[i], xf[i], acc);
-      } else {
-        // Last, partial stage: sub-tiles past K were re-fetched copies and must not be added.
-#pragma unroll
-        for (int i = 0; i < 2 * KT; ++i)
-          if (i < 2 * count) acc = mfma_16x16x32(wf[i], xf[i], acc);
-      }
+      for (int i = 0; i < 2 * KT; ++i)
+        if (i < 2 * count) acc = mfma_16x16x32(wf[i], xf[i], acc);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
   __builtin_amdgcn_s_waitcnt(kWaitAll0);
   wg_barrier();
 
-  if (wave == 0 && l16 < M) {
+  const int m = wave * 16 + l16;
+  if (wave < MT && m < M) {
     const int n = n0 + grp * 4;
     if (OUT_F32) {
-      float* row = reinterpret_cast<float*>(C) + (int64_t)l16 * ldc;
+      float* row = reinterpret_cast<float*>(C) + (int64_t)m * ldc;
 #pragma unroll
       for (int q = 0; q < 4; ++q)
         if (n + q < N) row[n + q] = acc[q];
     } else {
-      bf16_bits* row = reinterpret_cast<bf16_bits*>(C) + (int64_t)l16 * ldc;
+      bf16_bits* row = reinterpret_cast<bf16_bits*>(C) + (int64_t)m * ldc;
       const uint32_t lo = pack_bf16x2(acc[0], acc[1]);
       const uint32_t hi = pack_bf16x2(acc[2], acc[3]);
       if (n + 4 <= N && (reinterpret_cast<uintptr_t>(row + n) & 7) == 0) {
@@ -144,35 +135,37 @@ __global__ __launch_bounds__(320) void det_gemm_stream_kernel(MatView W, MatView
   }
 }
 
-template <int KT, int RING, bool HALF_X, bool OUT_F32>
+template <int KT, int RING, int MT, bool OUT_F32>
 static hipError_t launch_stream(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
-                                hipStream_t stream) {
-  auto kernel = det_gemm_stream_kernel<KT, RING, HALF_X, OUT_F32>;
-  constexpr int kLds = RING * 2 * KT * 16 * kRowBytes;
+                                      hipStream_t stream) {
+  auto kernel = det_gemm_stream_kernel<KT, RING, MT, OUT_F32>;
+  constexpr int kLds = RING * KT * (1 + MT) * 16 * kRowBytes;
+  static_assert(kLds <= 160 * 1024, "ring exceeds the LDS");
   static PerDeviceOnce once;
   hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLds, once);
   if (err != hipSuccess) return err;
-  hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(320), kLds, stream, W, X, C, ldc, M, N, K);
+  hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(64 * (MT + 4)), kLds, stream, W, X, C, ldc, M, N, K);
   return hipGetLastError();
 }
 
-// variant 0: 512-wide stages, ring of 4 (128 KiB, one workgroup per CU: few, long panels)
-// variant 1: 256-wide stages, ring of 4 (64 KiB, two workgroups per CU: many, short panels)
+// One to four token tiles; the ring takes 128 - 144 KiB (one workgroup per CU). `shallow`
+// (M <= 16 only) halves the stage so that two workgroups share a CU.
 hipError_t det_gemm_stream_launch(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
-                                  bool out_f32, int variant, hipStream_t stream) {
-  const bool half = M <= 8;
-  if (variant == 0) {
-    if (half)
-      return out_f32 ? launch_stream<8, 4, true, true>(W, X, C, ldc, M, N, K, stream)
-                     : launch_stream<8, 4, true, false>(W, X, C, ldc, M, N, K, stream);
-    return out_f32 ? launch_stream<8, 4, false, true>(W, X, C, ldc, M, N, K, stream)
-                   : launch_stream<8, 4, false, false>(W, X, C, ldc, M, N, K, stream);
-  }
-  if (half)
-    return out_f32 ? launch_stream<4, 4, true, true>(W, X, C, ldc, M, N, K, stream)
-                   : launch_stream<4, 4, true, false>(W, X, C, ldc, M, N, K, stream);
-  return out_f32 ? launch_stream<4, 4, false, true>(W, X, C, ldc, M, N, K, stream)
-                 : launch_stream<4, 4, false, false>(W, X, C, ldc, M, N, K, stream);
+                                  bool out_f32, bool shallow, hipStream_t stream) {
+  if (M <= 16 && shallow)
+    return out_f32 ? launch_stream<2, 8, 1, true>(W, X, C, ldc, M, N, K, stream)
+                   : launch_stream<2, 8, 1, false>(W, X, C, ldc, M, N, K, stream);
+  if (M <= 16)
+    return out_f32 ? launch_stream<4, 8, 1, true>(W, X, C, ldc, M, N, K, stream)
+                   : launch_stream<4, 8, 1, false>(W, X, C, ldc, M, N, K, stream);
+  if (M <= 32)
+    return out_f32 ? launch_stream<4, 6, 2, true>(W, X, C, ldc, M, N, K, stream)
+                   : launch_stream<4, 6, 2, false>(W, X, C, ldc, M, N, K, stream);
+  if (M <= 48)
+    return out_f32 ? launch_stream<2, 9, 3, true>(W, X, C, ldc, M, N, K, stream)
+                   : launch_stream<2, 9, 3, false>(W, X, C, ldc, M, N, K, stream);
+  return out_f32 ? launch_stream<2, 7, 4, true>(W, X, C, ldc, M, N, K, stream)
+                 : launch_stream<2, 7, 4, false>(W, X, C, ldc, M, N, K, stream);
 }
 
 }  // namespace rlk

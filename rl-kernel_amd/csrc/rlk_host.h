@@ -44,9 +44,10 @@ int det_gemm_tree_max_k();
 hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int64_t ldc, int M, int N, int K,
                                 hipStream_t stream);
 
-// Decode-sized batches (M <= 16), unit K stride, K % 64 == 0.
+// Up to 64 tokens, unit K stride, 16-byte aligned rows, K % 64 == 0. `shallow`: M <= 16 with
+// two workgroups per CU.
 hipError_t det_gemm_stream_launch(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
-                                  bool out_f32, int variant, hipStream_t stream);
+                                  bool out_f32, bool shallow, hipStream_t stream);
 
 hipError_t fill_zero_launch(void* dst, int64_t rows, int64_t cols, int64_t ld, int elem_bytes,
                             hipStream_t stream);

@@ -206,11 +206,12 @@ bool det_gemm_swiglu_fused_supported(const MatView& W, const MatView& X, int M, 
   auto native = [](const MatView& v) {
     return v.k_stride == 1 && (v.row_stride % kChunkElems) == 0 && (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0;
   };
-  return native(W) && native(X) && (K % kTileK) == 0 && M > 16;
+  return native(W) && native(X) && (K % kTileK) == 0 && M > 128;
 }
 
 // Y[M, I] = swiglu(X @ W[0:I]^T, X @ W[I:2I]^T). `workspace` ([M, 2 I] bf16) is used only when
-// the fused kernel does not apply (other layouts, ragged K, decode-sized M), where the
+// the fused kernel does not apply (other layouts, ragged K, up to 128 tokens: there the weight read bounds the time and the
+// GEMM kernels for few tokens spread it over more CUs than a gated 128-feature tile), where the
 // projection and the activation run as two kernels with the same result.
 hipError_t det_gemm_swiglu_launch(const MatView& W, const MatView& X, void* Y, int64_t ldy, void* workspace, int M,
                                   int I, int K, hipStream_t stream) {

@@ -36,6 +36,7 @@ GEMM_CONFIGS = {
     "64x64_deep": 11,
     "128x64_deep": 12,
     "128x128_deep": 13,
+    "stream64": 14,
 }
 # OR-ed into a GEMM or LogP configuration: register-staged main loop (bit-neutral).
 FORCE_STAGED = 0x100

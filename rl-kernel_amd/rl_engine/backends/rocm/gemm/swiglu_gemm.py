@@ -2,9 +2,9 @@
 
 Stands in for rl_engine/backends/rocm/gemm/swiglu_gemm.py:36-86 of the reference, whose
 fused path serves decode-sized batches through split-K partials. Here one MFMA kernel
-serves every batch above 16 rows (a workgroup owns the gate and the up projection of the
+serves every batch above 128 rows (a workgroup owns the gate and the up projection of the
 same 128 features, so the ``[M, 2 I]`` projection is never written); smaller batches run
-the streaming GEMM and the elementwise kernel. Both orders of work give the same bits.
+the GEMM for few tokens and the elementwise kernel. Both orders of work give the same bits.
 """
 
 from __future__ import annotations

@@ -137,6 +137,29 @@ def test_pingpong_and_staged_main_loops_give_the_same_bits(gemm, shape):
         assert _same_bits(gemm.mfma_gemm(a, w.t(), config=value | _lib.FORCE_STAGED), base), f"{name} staged"
 
 
+@pytest.mark.parametrize("m", (17, 31, 32, 33, 47, 48, 49, 64))
+@pytest.mark.parametrize("nk", ((4096, 12288), (40, 192), (16, 64), (250, 320), (72, 1088)))
+def test_streaming_kernel_for_17_to_64_tokens_gives_the_same_bits(gemm, native, m, nk):
+    """Two, three and four token tiles, panels past the N edge, stage counts that do not divide K / 64,
+    bf16 and fp32 output, against the one-wave 16x16 tile kernel; rows batch invariant."""
+    from rl_engine import _lib
+
+    n, k = nk
+    a = inputs.randn_bf16(2500 + m, m, k).to(DEV)
+    w = inputs.randn_bf16(2501 + n, n, k, 0.02).to(DEV)
+    base = gemm.mfma_gemm(a, w.t(), config="16x16")
+    got = gemm.mfma_gemm(a, w.t(), config="stream64")
+    assert _same_bits(got, base)
+    assert _same_bits(gemm.mfma_gemm(a, w.t(), config="stream64"), got)
+    f32 = torch.empty((m, n), dtype=torch.float32, device=DEV)
+    f32_base = torch.empty_like(f32)
+    native.gemm_strided(a, w.t(), f32, config=_lib.GEMM_CONFIGS["stream64"])
+    native.gemm_strided(a, w.t(), f32_base, config=_lib.GEMM_CONFIGS["16x16"])
+    assert torch.equal(f32.view(torch.int32), f32_base.view(torch.int32))
+    one = gemm.mfma_gemm(a[m - 1 :], w.t())
+    assert _same_bits(one, got[m - 1 :])
+
+
 # ---------------------------------------------------------------------------
 # Batch invariance (rows, cuts, strided views, chunked prefill, padding)
 # ---------------------------------------------------------------------------
