@@ -234,8 +234,8 @@ int pick_det_gemm_config(int M, int N, int K) {
   // Decode: many short panels keep the chip busy with one wave each; few long panels need
   // the streaming kernel's deep ring (one 16-feature panel per workgroup). Up to 32 / 64
   // tokens the same holds while there are at most 1.5 / 1 panels per CU: a 64-token tile
-  // kernel would run on N / 64 CUs only (down projection at 32 tokens: 38 -> 19 us). A CU's
-  // direct-to-LDS path moves about 31 bytes per clock, which bounds both kernels.
+  // kernel would run on N / 64 CUs only (down projection at 32 tokens: 38 -> 19 us, the time
+  // the 100 MB weight takes through the fabric).
   if (M <= 16) return N >= 64 * kCus ? RLK_GEMM_CFG_16x16 : RLK_GEMM_CFG_STREAM64;
   if (K >= 1024 && K % kTileK == 0 && ((M <= 32 && N <= 24 * kCus) || (M <= 64 && N <= 16 * kCus)))
     return RLK_GEMM_CFG_STREAM64;

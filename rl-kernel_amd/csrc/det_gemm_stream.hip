@@ -7,10 +7,12 @@
 // panel is the finest unit of work (N / 16 workgroups: 256 for the Qwen3-8B down projection,
 // one per CU). To keep enough bytes in flight with one workgroup per CU, four producer waves
 // issue direct-to-LDS loads several stages ahead; the consumer waves only read fragments and
-// issue the dependent MFMA chain, which is short (K/32 steps of ~21 cycles). The vector-memory
-// front end of a CU retires about one 1 KiB load per 33 cycles (about 31 bytes per clock), so
-// the loop is bound by the number of loads and the consumers issue none. Same instruction,
-// same ascending K order, same zero start as every other det_gemm kernel, so the bits match.
+// issue the dependent MFMA chain, which is short (K/32 steps of ~21 cycles). Measured on this
+// part: L2 hits feed a CU's direct-to-LDS path at 64 bytes per clock (135 GB/s, two issuing
+// waves suffice), data that comes through the fabric (infinity cache / HBM) arrives at about
+// 6 TB/s chip-wide, i.e. 23 GB/s per CU: the weight panel is the slow stream, the activations
+// (re-read by every workgroup, L2 hits) the wide one. Same instruction, same ascending K order,
+// same zero start as every other det_gemm kernel, so the bits match.
 #include "det_gemm_tile.h"
 #include "rlk_host.h"
 
