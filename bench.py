@@ -270,7 +270,7 @@ def main() -> int:
     # ---- every token count of the configuration
     if not args.no_shapes:
         shapes = []
-        for t in (1, 16, 256, 1024, 4096):
+        for t in (1, 16, 64, 256, 1024, 4096):
             for name, act, w, n, k, out in (("gate_up", x, w_gu, 2 * INTER, HIDDEN, out_gu), ("down", h, w_d, HIDDEN, INTER, out_d)):
                 a_t, o_t = act[:t], out[:t]
                 ms = _time_calls(lambda: gemm.mfma_gemm(a_t, w.t(), out=o_t), 30 if t <= 256 else 10, 10)
