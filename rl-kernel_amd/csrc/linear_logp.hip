@@ -108,30 +108,11 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_partial_kernel(LogpAr
 #pragma unroll
     for (int jm = 0; jm < S::TM; ++jm) {
       float y[16];
-      float tmax = kNegInf;
 #pragma unroll
-      for (int c = 0; c < 16; ++c) {
-        const float z = scaled_logit(acc[c >> 2][jm][c & 3], a.bias != nullptr, bias_run[c], col0 + c, a.vocab_limit,
-                                     a.temperature != nullptr, inv_t[jm]);
-        y[c] = z;
-        tmax = fmaxf(tmax, z);
-      }
-      const int tl = tgt[jm] - col0;
-      if (tl >= 0 && tl < 16) {
-        float sel = y[0];
-#pragma unroll
-        for (int c = 1; c < 16; ++c) sel = (tl == c) ? y[c] : sel;
-        run_zt[jm] = sel;
-      }
-      const float old_m = run_m[jm];
-      const float new_m = fmaxf(old_m, tmax);
-      float sum = pinned_exp(y[0] - new_m);
-#pragma unroll
-      for (int c = 1; c < 16; ++c) sum = sum + pinned_exp(y[c] - new_m);
-      const float scaled = run_s[jm] * pinned_exp(old_m - new_m);
-      const bool live = new_m > kNegInf;
-      run_s[jm] = live ? (scaled + sum) : run_s[jm];
-      run_m[jm] = new_m;
+      for (int c = 0; c < 16; ++c)
+        y[c] = scaled_logit(acc[c >> 2][jm][c & 3], a.bias != nullptr, bias_run[c], col0 + c, a.vocab_limit,
+                            a.temperature != nullptr, inv_t[jm]);
+      logp_fold_run(y, tgt[jm] - col0, run_m[jm], run_s[jm], run_zt[jm]);
     }
   }
 
@@ -151,17 +132,8 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_partial_kernel(LogpAr
   for (int tok = threadIdx.x; tok < S::BM; tok += S::kThreads) {
     const int m = m0 + tok;
     if (m >= a.T) continue;
-    float big = kNegInf;
-#pragma unroll
-    for (int j = 0; j < kLogpStreams; ++j) big = fmaxf(big, xm[j * S::BM + tok]);
-    float sum = 0.f, zt = 0.f;
-#pragma unroll
-    for (int j = 0; j < kLogpStreams; ++j) {
-      const float pm = xm[j * S::BM + tok];
-      const float term = xs[j * S::BM + tok] * pinned_exp(pm - big);
-      sum = sum + ((pm > kNegInf) ? term : 0.f);
-      zt = zt + xz[j * S::BM + tok];
-    }
+    float big, sum, zt;
+    logp_merge_streams(xm + tok, xs + tok, xz + tok, S::BM, big, sum, zt);
     const int64_t plane = (int64_t)a.n_split * a.T;
     const int64_t at = (int64_t)split * a.T + m;
     a.part[at] = big;
@@ -236,29 +208,12 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_streamgroup_kernel(Lo
           run_zt = sz[slot];
         }
         float y[16];
-        float tmax = kNegInf;
 #pragma unroll
-        for (int c = 0; c < 16; ++c) {
-          const float z = scaled_logit(acc[c >> 2][jm][c & 3], a.bias != nullptr, bias_run[c], col0 + c,
-                                       a.vocab_limit, a.temperature != nullptr, inv_t);
-          y[c] = z;
-          tmax = fmaxf(tmax, z);
-        }
-        const int tl = tgt - col0;
-        if (tl >= 0 && tl < 16) {
-          float sel = y[0];
-#pragma unroll
-          for (int c = 1; c < 16; ++c) sel = (tl == c) ? y[c] : sel;
-          run_zt = sel;
-        }
-        const float old_m = run_m;
-        const float new_m = fmaxf(old_m, tmax);
-        float sum = pinned_exp(y[0] - new_m);
-#pragma unroll
-        for (int c = 1; c < 16; ++c) sum = sum + pinned_exp(y[c] - new_m);
-        const float scaled = run_s * pinned_exp(old_m - new_m);
-        run_s = (new_m > kNegInf) ? (scaled + sum) : run_s;
-        sm[slot] = new_m;
+        for (int c = 0; c < 16; ++c)
+          y[c] = scaled_logit(acc[c >> 2][jm][c & 3], a.bias != nullptr, bias_run[c], col0 + c, a.vocab_limit,
+                              a.temperature != nullptr, inv_t);
+        logp_fold_run(y, tgt - col0, run_m, run_s, run_zt);
+        sm[slot] = run_m;
         ss[slot] = run_s;
         sz[slot] = run_zt;
       }
@@ -288,17 +243,8 @@ __global__ __launch_bounds__(256) void linear_logp_stream_merge_kernel(const flo
   const int split = idx / T;
   const int64_t splane = (int64_t)n_split * kLogpStreams * T;
   const float* xm = spart + (int64_t)split * kLogpStreams * T + m;
-  float big = kNegInf;
-#pragma unroll
-  for (int j = 0; j < kLogpStreams; ++j) big = fmaxf(big, xm[(int64_t)j * T]);
-  float sum = 0.f, zt = 0.f;
-#pragma unroll
-  for (int j = 0; j < kLogpStreams; ++j) {
-    const float pm = xm[(int64_t)j * T];
-    const float term = xm[splane + (int64_t)j * T] * pinned_exp(pm - big);
-    sum = sum + ((pm > kNegInf) ? term : 0.f);
-    zt = zt + xm[2 * splane + (int64_t)j * T];
-  }
+  float big, sum, zt;
+  logp_merge_streams(xm, xm + splane, xm + 2 * splane, T, big, sum, zt);
   const int64_t plane = (int64_t)n_split * T;
   const int64_t at = (int64_t)split * T + m;
   part[at] = big;

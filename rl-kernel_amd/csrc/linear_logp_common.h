@@ -27,4 +27,47 @@ __device__ __forceinline__ float scaled_logit(float z, bool has_bias, float bias
   return z;
 }
 
+// One step of a stream's online chain: the 16 scaled logits y of the stream's run in one
+// tile are folded into the running (max, sum), exponentials added in ascending column order;
+// `tl` is the target's position inside the run (outside [0, 16): not in this run). A run that
+// is all -inf (a fully padded tile) leaves the state unchanged.
+__device__ __forceinline__ void logp_fold_run(const float (&y)[16], int tl, float& run_m, float& run_s,
+                                              float& run_zt) {
+  float tmax = kNegInf;
+#pragma unroll
+  for (int c = 0; c < 16; ++c) tmax = fmaxf(tmax, y[c]);
+  if (tl >= 0 && tl < 16) {
+    float sel = y[0];
+#pragma unroll
+    for (int c = 1; c < 16; ++c) sel = (tl == c) ? y[c] : sel;
+    run_zt = sel;
+  }
+  const float old_m = run_m;
+  const float new_m = fmaxf(old_m, tmax);
+  float sum = pinned_exp(y[0] - new_m);
+#pragma unroll
+  for (int c = 1; c < 16; ++c) sum = sum + pinned_exp(y[c] - new_m);
+  const float scaled = run_s * pinned_exp(old_m - new_m);
+  run_s = (new_m > kNegInf) ? (scaled + sum) : run_s;
+  run_m = new_m;
+}
+
+// The 16 stream states of a (split, token), merged in ascending stream order. pm / ps / pz
+// point at stream 0; consecutive streams are `stride` floats apart.
+__device__ __forceinline__ void logp_merge_streams(const float* pm, const float* ps, const float* pz, int64_t stride,
+                                                   float& big, float& sum, float& zt) {
+  big = kNegInf;
+#pragma unroll
+  for (int j = 0; j < kLogpStreams; ++j) big = fmaxf(big, pm[j * stride]);
+  sum = 0.f;
+  zt = 0.f;
+#pragma unroll
+  for (int j = 0; j < kLogpStreams; ++j) {
+    const float m = pm[j * stride];
+    const float term = ps[j * stride] * pinned_exp(m - big);
+    sum = sum + ((m > kNegInf) ? term : 0.f);
+    zt = zt + pz[j * stride];
+  }
+}
+
 }  // namespace rlk

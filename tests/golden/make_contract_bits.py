@@ -1,0 +1,67 @@
+"""Writes tests/golden/contract_bits.json: SHA-256 of the raw output bytes of the GPU kernels
+on the stored fixture inputs, one entry per arithmetic contract id.
+
+The contracts promise bit-identical results for a given id across builds of the library; this
+file freezes the bits the first shipped build produced, so a change of arithmetic that forgets
+to bump the id fails tests/test_contract_bits_gpu.py. Needs an MI355X:
+
+    python tests/golden/make_contract_bits.py [output.json]
+"""
+
+from __future__ import annotations
+
+import hashlib
+import json
+import sys
+from pathlib import Path
+
+import numpy as np
+import torch
+
+HERE = Path(__file__).resolve().parent
+ROOT = HERE.parent.parent
+sys.path.insert(0, str(ROOT / "rl-kernel_amd"))
+sys.path.insert(0, str(ROOT / "tests"))
+
+import inputs  # noqa: E402
+
+
+def _sha(t: torch.Tensor) -> str:
+    raw = t.detach().contiguous().cpu()
+    raw = raw.view(torch.int16) if raw.dtype == torch.bfloat16 else raw
+    return hashlib.sha256(raw.numpy().tobytes()).hexdigest()
+
+
+def contract_bits() -> dict:
+    from rl_engine import _lib
+    from rl_engine.backends.rocm.gemm import det_gemm as gemm
+    from rl_engine.ops.logprob import deterministic_linear_logp
+
+    dev = "cuda"
+    lib = _lib.load()
+    a, b = inputs.config1()  # seeded; config1_det_gemm.npz holds the checksums of these operands
+    a, b = a.to(dev), b.to(dev)
+    out = {}
+    out[lib.rlk_contract_id().decode()] = {"config1_det_gemm": _sha(gemm.mfma_gemm(a, b))}
+    out[lib.rlk_det_gemm_tree_contract_id().decode()] = {"config1_det_gemm": _sha(gemm.tree_gemm(a, b))}
+    d = np.load(HERE / "small_linear_logp.npz")
+    h = inputs.from_bits(d["hidden_bits"], dev)
+    w = inputs.from_bits(d["weight_bits"], dev)
+    t = torch.from_numpy(d["target"]).to(dev)
+    logp, lse = deterministic_linear_logp(h, w, t)
+    logp2, lse2 = deterministic_linear_logp(
+        h, w, t % 1900, torch.from_numpy(d["bias"]).to(dev), temperature=torch.from_numpy(d["temperature"]).to(dev), real_vocab_size=1900
+    )
+    out[lib.rlk_linear_logp_contract_id().decode()] = {
+        "small_linear_logp.logp": _sha(logp),
+        "small_linear_logp.lse": _sha(lse),
+        "small_linear_logp.logp_bias_temp_pad": _sha(logp2),
+        "small_linear_logp.lse_bias_temp_pad": _sha(lse2),
+    }
+    return out
+
+
+if __name__ == "__main__":
+    target = Path(sys.argv[1]) if len(sys.argv) > 1 else HERE / "contract_bits.json"
+    target.write_text(json.dumps(contract_bits(), indent=2, sort_keys=True) + "\n")
+    print(target.read_text())
