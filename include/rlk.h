@@ -263,26 +263,29 @@ int rlk_logits_logp_backward(const void* logits, int dtype, int64_t row_stride, 
                              int64_t vocab_start, int64_t real_vocab, void* stream);
 
 /*
- * SwiGLU on bf16 rows: y[m, c] = bf16((g * sigmoid(g)) * u) with g = gate[m * ld_gate + c],
- * u = up[m * ld_up + c] widened to fp32 and sigmoid(g) = 1 / (1 + exp(-g)) (hardware
- * reciprocal and exponential, each within 1 ulp). A packed
- * [rows, 2 * cols] projection is the case up = gate + cols, ld_gate = ld_up = 2 * cols.
+ * SwiGLU on rows of element type `dtype` (rlk_dtype: bf16, fp16 or fp32; every tensor of a
+ * call has it; strides in elements): y[m, c] = round((g * sigmoid(g)) * u) with
+ * g = gate[m * ld_gate + c], u = up[m * ld_up + c] widened to fp32 and
+ * sigmoid(g) = 1 / (1 + exp(-g)) (hardware reciprocal and exponential, each within 1 ulp);
+ * one rounding to the element type. A packed [rows, 2 * cols] projection is the case
+ * up = gate + cols, ld_gate = ld_up = 2 * cols.
  *
  * Stands in for rl_engine._C.swiglu_forward / swiglu_packed_forward
  * (csrc/bindings/ops.cpp:400-413; csrc/cuda/activation/activation.cu:62-75, 97-112).
  */
 int rlk_swiglu_fwd(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, void* y, int64_t ld_y, int rows,
-                   int cols, void* stream);
+                   int cols, int dtype, void* stream);
 
 /*
- * Backward of rlk_swiglu_fwd: d_up = bf16(dy * silu(g)), d_gate = bf16(dy * u * silu'(g)),
+ * Backward of rlk_swiglu_fwd: d_up = round(dy * silu(g)), d_gate = round(dy * u * silu'(g)),
  * silu'(g) = s * (1 + g * (1 - s)), s = sigmoid(g).
  *
  * Stands in for rl_engine._C.swiglu_backward / swiglu_packed_backward
  * (csrc/bindings/ops.cpp:404-419; activation.cu:77-95, 114-135).
  */
 int rlk_swiglu_bwd(const void* dy, int64_t ld_dy, const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
-                   void* d_gate, int64_t ld_d_gate, void* d_up, int64_t ld_d_up, int rows, int cols, void* stream);
+                   void* d_gate, int64_t ld_d_gate, void* d_up, int64_t ld_d_up, int rows, int cols, int dtype,
+                   void* stream);
 
 /* Bytes of workspace rlk_det_gemm_swiglu_bf16 needs for these operands: 0 when the fused
  * kernel applies (unit K strides, 16-byte aligned rows, K % 64 == 0, M > 128), else the

@@ -556,6 +556,21 @@ def swiglu_backward(dy_bits, gate_bits, up_bits):
     return f32_to_bf16(d_gate), f32_to_bf16(d_up)
 
 
+def swiglu_values(gate, up, dy=None):
+    """The same formulas on fp32 arrays, unrounded fp32 results: ``y`` or, with ``dy``,
+    ``(d_gate, d_up)``. What the fp16 / fp32 instantiations of the reference kernels
+    compute before their cast to the element type (activation.cu:62-95)."""
+    g = np.asarray(gate, dtype=np.float32)
+    u = np.asarray(up, dtype=np.float32)
+    s = _sigmoid_f32(g)
+    if dy is None:
+        return ((g * s).astype(np.float32) * u).astype(np.float32)
+    d = np.asarray(dy, dtype=np.float32)
+    d_up = (d * (g * s)).astype(np.float32)
+    d_gate = ((d * u) * (s * (np.float32(1.0) + g * (np.float32(1.0) - s)))).astype(np.float32)
+    return d_gate, d_up
+
+
 def swiglu_packed(gate_up_bits) -> np.ndarray:
     """SwiGLU of a packed ``[rows, 2 I]`` projection: columns ``[0, I)`` gate, ``[I, 2 I)`` up
     (swiglu_packed_forward_kernel, activation.cu:97-112)."""

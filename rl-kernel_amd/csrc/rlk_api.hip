@@ -325,10 +325,18 @@ int rlk_logits_logp_backward(const void* logits, int dtype, int64_t row_stride, 
   return err == hipSuccess ? RLK_OK : device_error("rlk_logits_logp_backward", err);
 }
 
+static bool activation_dtype_ok(int dtype) {
+  return dtype == RLK_DTYPE_BF16 || dtype == RLK_DTYPE_FP16 || dtype == RLK_DTYPE_FP32;
+}
+
 int rlk_swiglu_fwd(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, void* y, int64_t ld_y, int rows,
-                   int cols, void* stream) {
+                   int cols, int dtype, void* stream) {
   if (rows < 0 || cols < 0) {
     set_last_error("rlk_swiglu_fwd: negative sizes");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (!activation_dtype_ok(dtype)) {
+    set_last_error("rlk_swiglu_fwd: unknown dtype %d", dtype);
     return RLK_ERR_INVALID_ARGUMENT;
   }
   if (rows == 0 || cols == 0) return RLK_OK;
@@ -336,15 +344,20 @@ int rlk_swiglu_fwd(const void* gate, int64_t ld_gate, const void* up, int64_t ld
     set_last_error("rlk_swiglu_fwd: null operand or row stride < cols");
     return RLK_ERR_INVALID_ARGUMENT;
   }
-  hipError_t err = swiglu_launch(gate, ld_gate, up, ld_up, nullptr, 0, y, ld_y, nullptr, 0, rows, cols, false,
+  hipError_t err = swiglu_launch(gate, ld_gate, up, ld_up, nullptr, 0, y, ld_y, nullptr, 0, rows, cols, false, dtype,
                                  reinterpret_cast<hipStream_t>(stream));
   return err == hipSuccess ? RLK_OK : device_error("rlk_swiglu_fwd", err);
 }
 
 int rlk_swiglu_bwd(const void* dy, int64_t ld_dy, const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
-                   void* d_gate, int64_t ld_d_gate, void* d_up, int64_t ld_d_up, int rows, int cols, void* stream) {
+                   void* d_gate, int64_t ld_d_gate, void* d_up, int64_t ld_d_up, int rows, int cols, int dtype,
+                   void* stream) {
   if (rows < 0 || cols < 0) {
     set_last_error("rlk_swiglu_bwd: negative sizes");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (!activation_dtype_ok(dtype)) {
+    set_last_error("rlk_swiglu_bwd: unknown dtype %d", dtype);
     return RLK_ERR_INVALID_ARGUMENT;
   }
   if (rows == 0 || cols == 0) return RLK_OK;
@@ -354,7 +367,7 @@ int rlk_swiglu_bwd(const void* dy, int64_t ld_dy, const void* gate, int64_t ld_g
     return RLK_ERR_INVALID_ARGUMENT;
   }
   hipError_t err = swiglu_launch(gate, ld_gate, up, ld_up, dy, ld_dy, d_gate, ld_d_gate, d_up, ld_d_up, rows, cols,
-                                 true, reinterpret_cast<hipStream_t>(stream));
+                                 true, dtype, reinterpret_cast<hipStream_t>(stream));
   return err == hipSuccess ? RLK_OK : device_error("rlk_swiglu_bwd", err);
 }
 

@@ -93,10 +93,11 @@ hipError_t linear_logp_bwd_launch(const MatView& H, const MatView& W, const int6
                                   int64_t gw_row_stride, float* grad_bias, void* workspace, int T, int D, int V,
                                   int64_t vocab_start, int vocab_limit, int config, hipStream_t stream);
 
-// SwiGLU on bf16 rows: forward writes y = out; backward writes d_gate = out, d_up = out2.
+// SwiGLU on rows of `dtype` (rlk_dtype; strides in elements): forward writes y = out; backward
+// writes d_gate = out, d_up = out2.
 hipError_t swiglu_launch(const void* gate, int64_t ld_g, const void* up, int64_t ld_u, const void* dy, int64_t ld_dy,
                          void* out, int64_t ld_out, void* out2, int64_t ld_out2, int rows, int cols, bool backward,
-                         hipStream_t stream);
+                         int dtype, hipStream_t stream);
 
 // Packed gate/up projection W[2 I, K] with the SwiGLU epilogue; workspace ([M, 2 I] bf16) is
 // only touched when det_gemm_swiglu_fused_supported() is false.

@@ -12,6 +12,8 @@
 //                                      e(x) = v_exp_f32(x * log2(e))
 //   y     = bf16((g * s) * u)
 //   d_up  = bf16(dy * (g * s));   d_gate = bf16((dy * u) * (s * (1 + g * (1 - s))))
+// The elementwise kernels also serve fp16 and fp32 tensors (the reference dispatches on the
+// element type, activation.cu:240-284): same fp32 arithmetic, one rounding to the element type.
 // The fused kernel rounds its two fp32 accumulators to bf16 before the activation, so it
 // returns exactly what the GEMM followed by the elementwise kernel returns.
 #include "linear_logp_common.h"
@@ -34,44 +36,75 @@ __device__ __forceinline__ float swiglu_f32(float g, float u) { return (g * sigm
 // ---------------------------------------------------------------------------
 
 struct SwigluArgs {
-  const bf16_bits* gate;
-  const bf16_bits* up;
-  const bf16_bits* dy;  // backward only
-  bf16_bits* y;         // forward: y; backward: d_gate
-  bf16_bits* y2;        // backward: d_up
-  int64_t ld_g, ld_u, ld_dy, ld_y, ld_y2;
+  const char* gate;
+  const char* up;
+  const char* dy;  // backward only
+  char* y;         // forward: y; backward: d_gate
+  char* y2;        // backward: d_up
+  int64_t ld_g, ld_u, ld_dy, ld_y, ld_y2;  // in elements
   int rows, cols;
 };
 
-__device__ __forceinline__ void load8(const bf16_bits* p, bool vec, int valid, float (&out)[8]) {
+// ELEM: rlk_dtype of the tensors. Arithmetic is fp32 for every type; results are rounded to
+// the element type once (round to nearest even), fp32 results are stored as they are.
+template <int ELEM>
+struct ActElem;
+template <>
+struct ActElem<RLK_DTYPE_BF16> {
+  typedef bf16_bits type;
+  static __device__ __forceinline__ float widen(bf16_bits v) { return bf16_to_f32(v); }
+  static __device__ __forceinline__ bf16_bits narrow(float v) { return to_bf16_bits(v); }
+};
+template <>
+struct ActElem<RLK_DTYPE_FP16> {
+  typedef _Float16 type;
+  static __device__ __forceinline__ float widen(_Float16 v) { return (float)v; }
+  static __device__ __forceinline__ _Float16 narrow(float v) { return (_Float16)v; }
+};
+template <>
+struct ActElem<RLK_DTYPE_FP32> {
+  typedef float type;
+  static __device__ __forceinline__ float widen(float v) { return v; }
+  static __device__ __forceinline__ float narrow(float v) { return v; }
+};
+
+template <int ELEM>
+__device__ __forceinline__ void load8(const char* base, int64_t index, bool vec, int valid, float (&out)[8]) {
+  typedef typename ActElem<ELEM>::type T;
+  const T* p = reinterpret_cast<const T*>(base) + index;
   if (vec && valid >= 8) {
-    const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(p);
-    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    T raw[8];
+    constexpr int kVecs = (int)sizeof(T) * 8 / 16;  // 16-byte accesses
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      out[2 * i] = bf16_to_f32(w[i] & 0xffffu);
-      out[2 * i + 1] = bf16_to_f32(w[i] >> 16);
-    }
+    for (int i = 0; i < kVecs; ++i)
+      reinterpret_cast<u32x4_t*>(raw)[i] = reinterpret_cast<const u32x4_t*>(p)[i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = ActElem<ELEM>::widen(raw[i]);
   } else {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) out[i] = i < valid ? bf16_to_f32(p[i]) : 0.f;
+    for (int i = 0; i < 8; ++i) out[i] = i < valid ? ActElem<ELEM>::widen(p[i]) : 0.f;
   }
 }
 
-__device__ __forceinline__ void store8(bf16_bits* p, bool vec, int valid, const float (&v)[8]) {
-  uint32_t w[4];
+template <int ELEM>
+__device__ __forceinline__ void store8(char* base, int64_t index, bool vec, int valid, const float (&v)[8]) {
+  typedef typename ActElem<ELEM>::type T;
+  T* p = reinterpret_cast<T*>(base) + index;
+  T raw[8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) w[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+  for (int i = 0; i < 8; ++i) raw[i] = ActElem<ELEM>::narrow(v[i]);
   if (vec && valid >= 8) {
-    *reinterpret_cast<u32x4_t*>(p) = u32x4_t{w[0], w[1], w[2], w[3]};
+    constexpr int kVecs = (int)sizeof(T) * 8 / 16;
+#pragma unroll
+    for (int i = 0; i < kVecs; ++i) reinterpret_cast<u32x4_t*>(p)[i] = reinterpret_cast<const u32x4_t*>(raw)[i];
   } else {
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-      if (i < valid) p[i] = (bf16_bits)((w[i >> 1] >> ((i & 1) * 16)) & 0xffffu);
+      if (i < valid) p[i] = raw[i];
   }
 }
 
-template <bool BACKWARD>
+template <bool BACKWARD, int ELEM>
 __global__ __launch_bounds__(256) void swiglu_kernel(SwigluArgs a, bool vec) {
   const int groups = (a.cols + 7) / 8;
   const int64_t total = (int64_t)a.rows * groups;
@@ -80,40 +113,52 @@ __global__ __launch_bounds__(256) void swiglu_kernel(SwigluArgs a, bool vec) {
     const int col = (int)(idx - (int64_t)row * groups) * 8;
     const int valid = a.cols - col;
     float g[8], u[8];
-    load8(a.gate + (int64_t)row * a.ld_g + col, vec, valid, g);
-    load8(a.up + (int64_t)row * a.ld_u + col, vec, valid, u);
+    load8<ELEM>(a.gate, (int64_t)row * a.ld_g + col, vec, valid, g);
+    load8<ELEM>(a.up, (int64_t)row * a.ld_u + col, vec, valid, u);
     if (!BACKWARD) {
       float y[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) y[i] = swiglu_f32(g[i], u[i]);
-      store8(a.y + (int64_t)row * a.ld_y + col, vec, valid, y);
+      store8<ELEM>(a.y, (int64_t)row * a.ld_y + col, vec, valid, y);
     } else {
       float dy[8], dg[8], du[8];
-      load8(a.dy + (int64_t)row * a.ld_dy + col, vec, valid, dy);
+      load8<ELEM>(a.dy, (int64_t)row * a.ld_dy + col, vec, valid, dy);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const float s = sigmoid_f32(g[i]);
         du[i] = dy[i] * (g[i] * s);
         dg[i] = (dy[i] * u[i]) * (s * (1.0f + g[i] * (1.0f - s)));
       }
-      store8(a.y + (int64_t)row * a.ld_y + col, vec, valid, dg);
-      store8(a.y2 + (int64_t)row * a.ld_y2 + col, vec, valid, du);
+      store8<ELEM>(a.y, (int64_t)row * a.ld_y + col, vec, valid, dg);
+      store8<ELEM>(a.y2, (int64_t)row * a.ld_y2 + col, vec, valid, du);
     }
   }
 }
 
-static bool aligned16(const void* p, int64_t ld) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0 && (ld % 8) == 0; }
+// Rows start on 16-byte boundaries and hold whole 16-byte vectors.
+static bool rows_aligned16(const void* p, int64_t ld, int elem_bytes) {
+  return (reinterpret_cast<uintptr_t>(p) & 15) == 0 && (ld * elem_bytes) % 16 == 0;
+}
+
+template <int ELEM>
+static void launch_swiglu_typed(const SwigluArgs& a, bool vec, bool backward, unsigned blocks, hipStream_t stream) {
+  if (backward) {
+    hipLaunchKernelGGL((swiglu_kernel<true, ELEM>), dim3(blocks), dim3(256), 0, stream, a, vec);
+  } else {
+    hipLaunchKernelGGL((swiglu_kernel<false, ELEM>), dim3(blocks), dim3(256), 0, stream, a, vec);
+  }
+}
 
 hipError_t swiglu_launch(const void* gate, int64_t ld_g, const void* up, int64_t ld_u, const void* dy, int64_t ld_dy,
                          void* out, int64_t ld_out, void* out2, int64_t ld_out2, int rows, int cols, bool backward,
-                         hipStream_t stream) {
+                         int dtype, hipStream_t stream) {
   if (rows == 0 || cols == 0) return hipSuccess;
   SwigluArgs a;
-  a.gate = reinterpret_cast<const bf16_bits*>(gate);
-  a.up = reinterpret_cast<const bf16_bits*>(up);
-  a.dy = reinterpret_cast<const bf16_bits*>(dy);
-  a.y = reinterpret_cast<bf16_bits*>(out);
-  a.y2 = reinterpret_cast<bf16_bits*>(out2);
+  a.gate = reinterpret_cast<const char*>(gate);
+  a.up = reinterpret_cast<const char*>(up);
+  a.dy = reinterpret_cast<const char*>(dy);
+  a.y = reinterpret_cast<char*>(out);
+  a.y2 = reinterpret_cast<char*>(out2);
   a.ld_g = ld_g;
   a.ld_u = ld_u;
   a.ld_dy = ld_dy;
@@ -121,15 +166,24 @@ hipError_t swiglu_launch(const void* gate, int64_t ld_g, const void* up, int64_t
   a.ld_y2 = ld_out2;
   a.rows = rows;
   a.cols = cols;
-  bool vec = aligned16(gate, ld_g) && aligned16(up, ld_u) && aligned16(out, ld_out);
-  if (backward) vec = vec && aligned16(dy, ld_dy) && aligned16(out2, ld_out2);
+  const int eb = dtype == RLK_DTYPE_FP32 ? 4 : 2;
+  bool vec = rows_aligned16(gate, ld_g, eb) && rows_aligned16(up, ld_u, eb) && rows_aligned16(out, ld_out, eb);
+  if (backward) vec = vec && rows_aligned16(dy, ld_dy, eb) && rows_aligned16(out2, ld_out2, eb);
   const int64_t total = (int64_t)rows * ((cols + 7) / 8);
   int64_t blocks = (total + 255) / 256;
   if (blocks > 256 * 32) blocks = 256 * 32;
-  if (backward) {
-    hipLaunchKernelGGL(swiglu_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, a, vec);
-  } else {
-    hipLaunchKernelGGL(swiglu_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, a, vec);
+  switch (dtype) {
+    case RLK_DTYPE_BF16:
+      launch_swiglu_typed<RLK_DTYPE_BF16>(a, vec, backward, (unsigned)blocks, stream);
+      break;
+    case RLK_DTYPE_FP16:
+      launch_swiglu_typed<RLK_DTYPE_FP16>(a, vec, backward, (unsigned)blocks, stream);
+      break;
+    case RLK_DTYPE_FP32:
+      launch_swiglu_typed<RLK_DTYPE_FP32>(a, vec, backward, (unsigned)blocks, stream);
+      break;
+    default:
+      return hipErrorInvalidValue;
   }
   return hipGetLastError();
 }
@@ -178,8 +232,8 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_swiglu_kernel(MatView W,
 #pragma unroll
       for (int q = 0; q < 4; ++q)
         y[h * 4 + q] = swiglu_f32(round_through_bf16(acc[h][jm][q]), round_through_bf16(acc[h + 2][jm][q]));
-    bf16_bits* dst = Y + (int64_t)m * ldy + f_run;
-    store8(dst, (reinterpret_cast<uintptr_t>(dst) & 15) == 0, I - f_run, y);
+    const int64_t at = (int64_t)m * ldy + f_run;
+    store8<RLK_DTYPE_BF16>(reinterpret_cast<char*>(Y), at, (reinterpret_cast<uintptr_t>(Y + at) & 15) == 0, I - f_run, y);
   }
 }
 
@@ -234,7 +288,8 @@ hipError_t det_gemm_swiglu_launch(const MatView& W, const MatView& X, void* Y, i
   hipError_t err = det_gemm_launch(W, X, workspace, 2 * (int64_t)I, M, 2 * I, K, false, RLK_GEMM_CFG_AUTO, stream);
   if (err != hipSuccess) return err;
   const bf16_bits* gu = reinterpret_cast<const bf16_bits*>(workspace);
-  return swiglu_launch(gu, 2 * (int64_t)I, gu + I, 2 * (int64_t)I, nullptr, 0, Y, ldy, nullptr, 0, M, I, false, stream);
+  return swiglu_launch(gu, 2 * (int64_t)I, gu + I, 2 * (int64_t)I, nullptr, 0, Y, ldy, nullptr, 0, M, I, false,
+                       RLK_DTYPE_BF16, stream);
 }
 
 }  // namespace rlk

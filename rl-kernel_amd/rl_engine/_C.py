@@ -579,16 +579,22 @@ def hip_deterministic_logp_backward(
 
 
 def _check_act(t: torch.Tensor, name: str) -> None:
-    """Checks of check_cuda_contig (csrc/cuda/activation/activation.cu:145-156); this build's
-    activation kernels serve bf16, the dtype of the GEMMs either side."""
+    """Checks of check_cuda_contig (csrc/cuda/activation/activation.cu:145-156)."""
     if not t.is_cuda:
         raise RuntimeError(f"{name} must be a CUDA tensor")
     if not t.is_contiguous():
         raise RuntimeError(f"{name} must be contiguous")
     if t.dtype not in (torch.float16, torch.bfloat16, torch.float32):
         raise RuntimeError(f"{name} must be fp16, bf16, or fp32, got {t.dtype}")
-    if t.dtype != _BF16:
-        raise RuntimeError(f"{name}: the gfx950 SwiGLU kernels serve bf16 only, got {t.dtype}")
+
+
+def _act_dtype_code(t: torch.Tensor) -> int:
+    return {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16, torch.float32: _lib.DTYPE_FP32}[t.dtype]
+
+
+def _same_act_dtype(first: torch.Tensor, first_name: str, other: torch.Tensor, other_name: str) -> None:
+    if other.dtype != first.dtype:
+        raise RuntimeError(f"{other_name} and {first_name} must share dtype")
 
 
 def _rows_cols(t: torch.Tensor) -> tuple:
@@ -604,13 +610,15 @@ def swiglu_forward(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
         raise RuntimeError(f"gate and up must be on the same CUDA device, got {gate.device} and {up.device}")
     if gate.shape != up.shape:
         raise RuntimeError("gate and up must share shape")
+    _same_act_dtype(gate, "gate", up, "up")
     y = torch.empty_like(gate)
     rows, cols = _rows_cols(gate)
     if gate.numel():
         with torch.cuda.device(gate.device):
             status = _lib.load().rlk_swiglu_fwd(
-                gate.data_ptr(), cols, up.data_ptr(), cols, y.data_ptr(), cols, rows, cols, _stream_handle(gate.device)
-            )
+                gate.data_ptr(), cols, up.data_ptr(), cols, y.data_ptr(), cols, rows, cols,
+                _act_dtype_code(gate), _stream_handle(gate.device),
+            )  # fmt: skip
         _lib.check(status, "rlk_swiglu_fwd failed")
     return y
 
@@ -624,13 +632,15 @@ def swiglu_backward(dy: torch.Tensor, gate: torch.Tensor, up: torch.Tensor) -> L
         raise RuntimeError("gate and up must share shape")
     if dy.shape != gate.shape:
         raise RuntimeError("dy and gate must share shape")
+    _same_act_dtype(gate, "gate", dy, "dy")
+    _same_act_dtype(gate, "gate", up, "up")
     d_gate, d_up = torch.empty_like(gate), torch.empty_like(up)
     rows, cols = _rows_cols(gate)
     if gate.numel():
         with torch.cuda.device(gate.device):
             status = _lib.load().rlk_swiglu_bwd(
                 dy.data_ptr(), cols, gate.data_ptr(), cols, up.data_ptr(), cols, d_gate.data_ptr(), cols,
-                d_up.data_ptr(), cols, rows, cols, _stream_handle(gate.device),
+                d_up.data_ptr(), cols, rows, cols, _act_dtype_code(gate), _stream_handle(gate.device),
             )  # fmt: skip
         _lib.check(status, "rlk_swiglu_bwd failed")
     return [d_gate, d_up]
@@ -650,8 +660,8 @@ def swiglu_packed_forward(gate_up: torch.Tensor) -> torch.Tensor:
         base = gate_up.data_ptr()
         with torch.cuda.device(gate_up.device):
             status = _lib.load().rlk_swiglu_fwd(
-                base, 2 * width, base + 2 * width, 2 * width, y.data_ptr(), width, rows, width,
-                _stream_handle(gate_up.device),
+                base, 2 * width, base + gate_up.element_size() * width, 2 * width, y.data_ptr(), width, rows, width,
+                _act_dtype_code(gate_up), _stream_handle(gate_up.device),
             )  # fmt: skip
         _lib.check(status, "rlk_swiglu_fwd failed")
     return y
@@ -669,14 +679,16 @@ def swiglu_packed_backward(dy: torch.Tensor, gate_up: torch.Tensor) -> List[torc
     rows, width = gate_up.size(0), gate_up.size(1) // 2
     if tuple(dy.shape) != (rows, width):
         raise RuntimeError("dy must be [rows, intermediate]")
+    _same_act_dtype(gate_up, "gate_up", dy, "dy")
     d_gate = torch.empty((rows, width), dtype=gate_up.dtype, device=gate_up.device)
     d_up = torch.empty_like(d_gate)
     if d_gate.numel():
         base = gate_up.data_ptr()
         with torch.cuda.device(gate_up.device):
             status = _lib.load().rlk_swiglu_bwd(
-                dy.data_ptr(), width, base, 2 * width, base + 2 * width, 2 * width, d_gate.data_ptr(), width,
-                d_up.data_ptr(), width, rows, width, _stream_handle(gate_up.device),
+                dy.data_ptr(), width, base, 2 * width, base + gate_up.element_size() * width, 2 * width,
+                d_gate.data_ptr(), width, d_up.data_ptr(), width, rows, width, _act_dtype_code(gate_up),
+                _stream_handle(gate_up.device),
             )  # fmt: skip
         _lib.check(status, "rlk_swiglu_bwd failed")
     return [d_gate, d_up]

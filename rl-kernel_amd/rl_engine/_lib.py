@@ -141,9 +141,9 @@ def load() -> ctypes.CDLL:
     lib.rlk_logits_logp_backward.argtypes = [vp, i32, i64, vp, vp, vp, vp, vp, vp, i64, i32, i64, i64, i64, vp]
 
     lib.rlk_swiglu_fwd.restype = i32
-    lib.rlk_swiglu_fwd.argtypes = [vp, i64, vp, i64, vp, i64, i32, i32, vp]
+    lib.rlk_swiglu_fwd.argtypes = [vp, i64, vp, i64, vp, i64, i32, i32, i32, vp]
     lib.rlk_swiglu_bwd.restype = i32
-    lib.rlk_swiglu_bwd.argtypes = [vp, i64, vp, i64, vp, i64, vp, i64, vp, i64, i32, i32, vp]
+    lib.rlk_swiglu_bwd.argtypes = [vp, i64, vp, i64, vp, i64, vp, i64, vp, i64, i32, i32, i32, vp]
     lib.rlk_det_gemm_swiglu_workspace_bytes.restype = sz
     lib.rlk_det_gemm_swiglu_workspace_bytes.argtypes = [vp, i64, vp, i64, i32, i32, i32]
     lib.rlk_det_gemm_swiglu_bf16.restype = i32

@@ -603,3 +603,20 @@ def test_grpo_hand_computed_2x2(oracle):
     assert kl == pytest.approx(sum(ks) / 3, rel=1e-4)
     assert loss == pytest.approx(sum(terms) / 3 + 0.01 * sum(ks) / 3, rel=1e-5)
     assert ratio[1, 0] == 0.0 and k3[1, 0] == 0.0
+
+
+def test_swiglu_values_is_the_unrounded_form_of_the_bf16_functions(oracle):
+    rng = np.random.default_rng(77)
+    g_bits = oracle.randn_bf16(rng, (9, 40), 2.0)
+    u_bits = oracle.randn_bf16(rng, (9, 40))
+    dy_bits = oracle.randn_bf16(rng, (9, 40))
+    g, u, dy = (oracle.bf16_to_f32(b) for b in (g_bits, u_bits, dy_bits))
+    assert np.array_equal(oracle.f32_to_bf16(oracle.swiglu_values(g, u)), oracle.swiglu(g_bits, u_bits))
+    d_gate, d_up = oracle.swiglu_values(g, u, dy)
+    ref_g, ref_u = oracle.swiglu_backward(dy_bits, g_bits, u_bits)
+    assert np.array_equal(oracle.f32_to_bf16(d_gate), ref_g) and np.array_equal(oracle.f32_to_bf16(d_up), ref_u)
+    # closed forms: silu(0) = 0, silu'(0) = 1/2, silu(x) -> x for large x
+    assert oracle.swiglu_values(np.zeros(3), np.ones(3)).tolist() == [0.0, 0.0, 0.0]
+    dg, du = oracle.swiglu_values(np.zeros(2), np.full(2, 3.0), np.full(2, 2.0))
+    assert dg.tolist() == [3.0, 3.0] and du.tolist() == [0.0, 0.0]
+    assert oracle.swiglu_values(np.full(1, 40.0), np.full(1, 0.5))[0] == 20.0

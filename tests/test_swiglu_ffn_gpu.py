@@ -147,6 +147,39 @@ def test_training_ffn_forward_and_backward(native, ffn_mod):
         assert _same_bits(a.grad, b.grad)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(64, 256), (37, 1000), (5, 7), (3, 4, 24)])
+def test_swiglu_fp16_and_fp32_tensors(native, oracle, dtype, shape):
+    """The reference's activation kernels dispatch on the element type (activation.cu:240-284): same
+    fp32 arithmetic, one rounding to the element type. fp32: within 4 fp32 ulp-scale of the oracle
+    (hardware exp and reciprocal); fp16: the oracle's value within half an fp16 ulp plus that."""
+    g = torch.Generator().manual_seed(8600 + len(shape))
+    gate = (torch.randn(shape, generator=g) * 2.0).to(dtype)
+    up = torch.randn(shape, generator=g).to(dtype)
+    dy = torch.randn(shape, generator=g).to(dtype)
+    y = native.swiglu_forward(gate.to(DEV), up.to(DEV))
+    d_gate, d_up = native.swiglu_backward(dy.to(DEV), gate.to(DEV), up.to(DEV))
+    assert y.dtype == dtype and y.shape == gate.shape and d_gate.dtype == dtype and d_up.shape == up.shape
+    want_y = oracle.swiglu_values(gate.float().numpy(), up.float().numpy())
+    want_g, want_u = oracle.swiglu_values(gate.float().numpy(), up.float().numpy(), dy.float().numpy())
+    eps = 2.0**-11 if dtype == torch.float16 else 0.0
+    floor = 2.0**-25 if dtype == torch.float16 else 0.0  # half an fp16 subnormal step
+    gf, uf, df = (np.abs(t.double().numpy()) for t in (gate, up, dy))
+    # the sigmoid is good to about 2 fp32 ulp; silu'(g) = s (1 + g (1 - s)) can cancel, so its error is
+    # absolute in (1 + |g|), not relative to the result
+    scales = (gf * uf, df * uf * (1.0 + gf), df * gf)
+    for got, want, scale in zip((y, d_gate, d_up), (want_y, want_g, want_u), scales):
+        err = np.abs(got.double().cpu().numpy() - want.astype(np.float64))
+        assert np.all(err <= eps * np.abs(want) + 2.0**-21 * scale + floor + 1e-30)
+    if len(shape) == 2:
+        packed = torch.cat([gate, up], dim=1).contiguous().to(DEV)
+        assert torch.equal(native.swiglu_packed_forward(packed), y)
+        pg, pu = native.swiglu_packed_backward(dy.to(DEV), packed)
+        assert torch.equal(pg, d_gate) and torch.equal(pu, d_up)
+    with pytest.raises(RuntimeError, match="must share dtype"):
+        native.swiglu_forward(gate.to(DEV), up.to(DEV).to(torch.bfloat16))
+
+
 def test_argument_errors(native, ffn_mod):
     x = torch.zeros((4, 64), dtype=torch.bfloat16, device=DEV)
     w = torch.zeros((32, 64), dtype=torch.bfloat16, device=DEV)
