@@ -267,6 +267,16 @@ def main() -> int:
         "roofline": roofline,
     }
 
+    # ---- orientation only: the vendor GEMM library on the same operands (not deterministic across
+    # batch shapes, not part of the product)
+    if not args.no_shapes:
+        ms_lib = _time_calls(lambda: torch.nn.functional.linear(x, w_gu), args.steps, args.warmup)
+        result["vendor_library_gemm"] = {
+            "what": "torch.nn.functional.linear (hipBLASLt) on the gate_up operands, same data, same process",
+            "ms": round(ms_lib, 4),
+            "tflops": round(flops_gu / ms_lib * 1e-9, 1),
+        }
+
     # ---- every token count of the configuration
     if not args.no_shapes:
         shapes = []
