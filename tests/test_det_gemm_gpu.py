@@ -160,6 +160,31 @@ def test_streaming_kernel_for_17_to_64_tokens_gives_the_same_bits(gemm, native, 
     assert _same_bits(one, got[m - 1 :])
 
 
+def test_seeded_random_shapes_layouts_and_offsets_match_the_element_loader(gemm):
+    """Whatever kernel the picker and the dispatch conditions choose for a shape, alignment and layout,
+    the bits are those of the one-wave tile kernel with the element-wise staged loader."""
+    from rl_engine import _lib
+
+    rng = np.random.default_rng(2600)
+    reference_config = _lib.GEMM_CONFIGS["16x16"] | _lib.FORCE_STAGED
+    for case in range(70):
+        m = int(rng.choice([1, 3, 8, 16, 17, 40, 64, 65, 130, 257]))
+        n = int(rng.choice([8, 16, 24, 72, 128, 200, 520]))
+        k = int(rng.choice([8, 64, 72, 128, 192, 320, 1024, 1088]))
+        a_layout, b_layout = rng.integers(0, 3, size=2)  # 0 native, 1 other axis contiguous, 2 padded rows + offset
+        a_full = inputs.randn_bf16(2601 + case, m + 1, k + 24).to(DEV)
+        w_full = inputs.randn_bf16(2801 + case, n + 1, k + 24, 0.05).to(DEV)
+        a = a_full[:m, :k] if a_layout != 2 else a_full[1:, 3 : k + 3]
+        w = w_full[:n, :k] if b_layout != 2 else w_full[1:, 5 : k + 5]
+        if a_layout == 1:
+            a = a.t().contiguous().t()  # token-contiguous activations
+        if b_layout == 1:
+            w = w.t().contiguous().t()  # B[K, N] with N contiguous
+        want = gemm.mfma_gemm(a.contiguous(), w.contiguous().t(), config=reference_config)
+        got = gemm.mfma_gemm(a, w.t())
+        assert _same_bits(got, want), (case, m, n, k, int(a_layout), int(b_layout))
+
+
 # ---------------------------------------------------------------------------
 # Batch invariance (rows, cuts, strided views, chunked prefill, padding)
 # ---------------------------------------------------------------------------
