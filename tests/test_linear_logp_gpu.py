@@ -140,6 +140,32 @@ def test_stream_group_split_keeps_the_bits(logp_mod, oracle, shape):
     assert np.abs(got[1].cpu().numpy() - ref_lse).max() <= TOL_NATS
 
 
+def test_seeded_random_shapes_match_the_smallest_tile_with_the_staged_loop(logp_mod):
+    """Whatever grid and tile the picker chooses for a token count, hidden size and vocabulary, with or
+    without bias, temperature and padding, logp and lse have the bits of the 16-token tile kernel."""
+    from rl_engine import _lib
+
+    rng = np.random.default_rng(4700)
+    reference_config = _lib.LOGP_CONFIGS["16"] | _lib.FORCE_STAGED
+    for case in range(40):
+        n = int(rng.choice([1, 5, 16, 33, 64, 65, 128, 129, 300, 700, 1025, 1300]))
+        v = int(rng.choice([40, 256, 1000, 1024, 2500, 4099, 6000]))
+        d = int(rng.choice([8, 64, 72, 128, 320, 512]))
+        h, w, target = inputs.logp_inputs(n, vocab=v, hidden=d, seed=4701 + case, rms_norm=False)
+        real = v if case % 3 else max(1, v - int(rng.integers(1, 30)))
+        target = target % real
+        extra = {}
+        if case % 2:
+            g = torch.Generator().manual_seed(4800 + case)
+            extra = {"bias": (torch.randn(v, generator=g) * 0.2).to(DEV), "temperature": (0.5 + torch.rand(n, generator=g)).to(DEV)}
+        if real != v:
+            extra["real_vocab_size"] = real
+        h_d, w_d, t_d = h.to(DEV), w.to(DEV), target.to(DEV)
+        want = logp_mod.deterministic_linear_logp(h_d, w_d, t_d, config=reference_config, **extra)
+        got = logp_mod.deterministic_linear_logp(h_d, w_d, t_d, **extra)
+        assert _same_bits(got[0], want[0]) and _same_bits(got[1], want[1]), (case, n, v, d, sorted(extra))
+
+
 def test_layout_packing_invariance(logp_mod):
     # Rows permuted across [2,3] / [3,2] / [1,6] layouts give the same per-row bits
     # (tests/ops/logprob/test_linear_logp.py:339-367).
