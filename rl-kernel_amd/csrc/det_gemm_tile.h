@@ -476,11 +476,18 @@ constexpr bool pingpong_supported() {
 // covers 64 * KS K values between two barriers: small tiles, whose phases would otherwise be
 // shorter than a barrier, stay on the matrix pipe. Needs K % (64 * KS) == 0 and
 // 2 * KS * S::kStageBytes of LDS; the MFMA chain is the same (K tiles ascending).
-template <class S, bool WK = false, bool XK = false, class Map = PlainRowMap<S>, int KS = 1>
+//
+// NS is the number of stages (K tiles in LDS): tile t lives in stage t % NS and the loads of
+// tile t + NS start as soon as tile t has been read, so NS - 1 tiles are in flight behind the
+// one being read. Two stages cover the latency of L2 hits; a weight tile that is used by one
+// workgroup only comes through the fabric and wants three. Needs NS * KS * S::kStageBytes of LDS.
+template <class S, bool WK = false, bool XK = false, class Map = PlainRowMap<S>, int KS = 1, int NS = 2>
 __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const MatView& X, int n0, int m0, int K,
                                                        char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
   static_assert(pingpong_supported<S>(), "two groups of four waves, 4 x 2 wave layout");
-  static_assert(KS >= 1 && KS * (DmaLoader<S, WK, XK, Map>::kLateLoads) <= 31, "loads in flight must fit vmcnt");
+  static_assert(KS >= 1 && NS >= 2 && (NS - 1) * KS * (DmaLoader<S, WK, XK, Map>::kLateLoads) <= 63 &&
+                    KS * (DmaLoader<S, WK, XK, Map>::kLateLoads) <= 31,
+                "loads in flight must fit vmcnt");
   using Loader = DmaLoader<S, WK, XK, Map>;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -510,7 +517,7 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
   // any more; that keeps the number of loads in flight (and so every s_waitcnt
   // immediate) the same in every iteration.
   auto tile_k = [&](int t) { return (t < nk ? t : nk - 1) * kStageK; };
-  auto stage = [&](int t) { return lds + (t & 1) * kStageSpan; };
+  auto stage = [&](int t) { return lds + (t % NS) * kStageSpan; };
   auto issue_early = [&](char* st, int k0) {
 #pragma unroll
     for (int s = 0; s < KS; ++s) loader.issue_early(st + s * S::kStageBytes, k0 + s * kTileK, wave);
@@ -611,8 +618,8 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
   // Phases are the intervals between consecutive workgroup barriers:
   //   phase 2t     : early group reads tile t        | late group computes tile t-1
   //   phase 2t + 1 : early group computes tile t     | late group reads tile t
-  // Tile t lives in stage t & 1, which is read in phases 2t and 2t + 1 and first
-  // read again (tile t + 2) in phase 2t + 4. Every wave waits for its own
+  // Tile t lives in stage t % NS, which is read in phases 2t and 2t + 1 and first
+  // read again (tile t + NS) in phase 2t + 2 NS. The notes below are for NS = 2. Every wave waits for its own
   // fragment reads before the barrier that ends its read phase.
   //   late wave, phase 2t + 1: starts its token rows of tile t + 2 at once (the early group
   //     read them one phase earlier) and its weight blocks as soon as its own weight
@@ -621,26 +628,27 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
   //   early wave, phase 2t + 2: starts its part of tile t + 2 (rows the late group read one
   //     phase earlier); confirms it at the end of phase 2t + 3.
   if (!late_group) {
-    issue_early(stage(0), 0);
-    issue_early(stage(1), tile_k(1));
-    __builtin_amdgcn_s_waitcnt(wait_vmcnt(KS * Loader::kEarlyLoads));  // my part of tile 0 has landed
+#pragma unroll
+    for (int i = 0; i < NS; ++i) issue_early(stage(i), tile_k(i));
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt((NS - 1) * KS * Loader::kEarlyLoads));  // my part of tile 0 has landed
     wg_barrier();
     for (int t = 0; t < nk; ++t) {
       read_tile(t);
-      if (t > 0) issue_early(stage(t + 1), tile_k(t + 1));
+      if (t > 0) issue_early(stage(t - 1 + NS), tile_k(t - 1 + NS));  // the stage tile t - 1 has left
       __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // my fragments are in registers
       wg_barrier();
       compute();
-      __builtin_amdgcn_s_waitcnt(kWaitVm0);  // my part of tile t+1 has landed
+      __builtin_amdgcn_s_waitcnt(wait_vmcnt((NS - 2) * KS * Loader::kEarlyLoads));  // my part of tile t+1 has landed
       wg_barrier();
     }
     wg_barrier();  // pairs with the late group's leading barrier
   } else {
-    issue_late_x(stage(0), 0);
-    issue_late_w(stage(0), 0);
-    issue_late_x(stage(1), tile_k(1));
-    issue_late_w(stage(1), tile_k(1));
-    __builtin_amdgcn_s_waitcnt(wait_vmcnt(KS * Loader::kLateLoads));  // my part of tile 0 has landed
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+      issue_late_x(stage(i), tile_k(i));
+      issue_late_w(stage(i), tile_k(i));
+    }
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt((NS - 1) * KS * Loader::kLateLoads));  // my part of tile 0 has landed
     wg_barrier();
     wg_barrier();  // half an iteration behind the early group
     // LDS reads return in order, so once at most kXReads of them are outstanding the weight
@@ -649,20 +657,20 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
     constexpr int kXReads = KS * S::TM * (XK ? 2 : 1);
     for (int t = 0; t < nk; ++t) {
       if constexpr (Loader::kSplitColumn && kXReads <= 15) {
-        issue_late_x(stage(t), tile_k(t + 2));  // token rows the early group read one phase ago
+        issue_late_x(stage(t), tile_k(t + NS));  // token rows the early group read one phase ago
         read_w(t);
         read_x(t, 0);
         __builtin_amdgcn_s_waitcnt(wait_lgkmcnt(kXReads));  // my weight fragments are in registers
-        issue_late_w(stage(t), tile_k(t + 2));
+        issue_late_w(stage(t), tile_k(t + NS));
         read_x(t, 1);
       } else {
         read_tile(t);
         __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
-        issue_late_w(stage(t), tile_k(t + 2));
-        issue_late_x(stage(t), tile_k(t + 2));
+        issue_late_w(stage(t), tile_k(t + NS));
+        issue_late_x(stage(t), tile_k(t + NS));
       }
       __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // all my fragments are in registers
-      __builtin_amdgcn_s_waitcnt(wait_vmcnt(KS * Loader::kLateLoads));  // my part of tile t+1 has landed
+      __builtin_amdgcn_s_waitcnt(wait_vmcnt((NS - 1) * KS * Loader::kLateLoads));  // my part of tile t+1 has landed
       wg_barrier();
       compute();
       wg_barrier();

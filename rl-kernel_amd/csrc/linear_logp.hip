@@ -151,7 +151,7 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_partial_kernel(LogpAr
 // columns into the state that column t - 1 left in LDS. Per-(split, stream) states go to
 // linear_logp_stream_merge_kernel, which repeats the in-kernel stream merge above. Same bits
 // as every other configuration.
-template <class S>
+template <class S, int NS>
 __global__ __launch_bounds__(S::kThreads) void linear_logp_streamgroup_kernel(LogpArgs a, float* __restrict__ spart) {
   static_assert(S::BN == kLogpTileCols && S::kRun == 16 && S::WN == 4, "wave column = tile of the split");
   constexpr int kGroups = kLogpStreams / 4;  // stream groups per split
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_streamgroup_kernel(Lo
   const int tok_local = wave_m * 16 * S::TM + l16;
 
   f32x4_t acc[S::TN][S::TM];
-  tile_mainloop_pingpong<S, false, false, StridedColumnRowMap<S, kLogpTileCols>>(a.W, a.H, n0, m0, a.D, lds, acc);
+  tile_mainloop_pingpong<S, false, false, StridedColumnRowMap<S, kLogpTileCols>, 1, NS>(a.W, a.H, n0, m0, a.D, lds, acc);
 
   const int v0 = split * kLogpSplitCols + tile * kLogpTileCols;
   const int col0 = v0 + (sg * 4 + grp) * 16;  // first column of this lane's run
@@ -363,15 +363,19 @@ static hipError_t launch_logp(LogpArgs a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// Up to 128 tokens every weight tile is used by one workgroup only: three stages for the
+// 64- and 128-token tiles (120 / 144 KiB); the 256-token tile has room for two.
 template <class S>
 static hipError_t launch_streamgroup(LogpArgs a, hipStream_t stream) {
-  auto kernel = linear_logp_streamgroup_kernel<S>;
+  constexpr int kStages = S::BM <= 128 ? 3 : 2;
+  auto kernel = linear_logp_streamgroup_kernel<S, kStages>;
+  constexpr int kLdsBytes = kStages * S::kStageBytes;
   static PerDeviceOnce once;
-  hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), S::kLdsBytes, once);
+  hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLdsBytes, once);
   if (err != hipSuccess) return err;
   a.tiles_m = (a.T + S::BM - 1) / S::BM;
   float* spart = a.part + (size_t)3 * a.n_split * a.T;  // behind the per-split partials
-  hipLaunchKernelGGL(kernel, dim3(a.tiles_m * a.n_split * (kLogpStreams / 4)), dim3(S::kThreads), S::kLdsBytes, stream,
+  hipLaunchKernelGGL(kernel, dim3(a.tiles_m * a.n_split * (kLogpStreams / 4)), dim3(S::kThreads), kLdsBytes, stream,
                      a, spart);
   err = hipGetLastError();
   if (err != hipSuccess) return err;
