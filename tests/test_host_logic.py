@@ -85,6 +85,15 @@ def test_argument_errors_are_reported_without_touching_the_gpu(rlk_lib):
     assert rc == -1 and b"null hidden" in rlk_lib.rlk_last_error()
     rc = rlk_lib.rlk_grpo_ratio_kl_loss(None, None, None, None, None, 2, 4, 0.2, 0.0, None, None, None, None, 0, None)
     assert rc == -1 and b"out3" in rlk_lib.rlk_last_error()
+    rc = rlk_lib.rlk_det_gemm_tree_bf16(None, 4, 1, None, 1, 4, None, 4, 2, 4, -4, None)
+    assert rc == -1 and b"negative size" in rlk_lib.rlk_last_error()
+    rc = rlk_lib.rlk_det_gemm_tree_bf16(None, 4, 1, None, 1, 4, None, 2, 2, 4, 4, None)
+    assert rc == -1 and b"ldc >= N" in rlk_lib.rlk_last_error()
+    assert rlk_lib.rlk_det_gemm_tree_bf16(None, 4, 1, None, 1, 4, None, 4, 2, 0, 4, None) == 0  # empty N: no-op
+    rc = rlk_lib.rlk_swiglu_fwd(None, 8, None, 8, None, 8, 2, 8, 7, None)
+    assert rc == -1 and b"unknown dtype" in rlk_lib.rlk_last_error()
+    rc = rlk_lib.rlk_swiglu_bwd(None, 8, None, 8, None, 8, None, 8, None, 8, 2, 8, 0, None)
+    assert rc == -1 and b"null operand" in rlk_lib.rlk_last_error()
 
 
 def test_missing_library_fails_loudly(tmp_path):
@@ -200,9 +209,12 @@ def test_linear_logp_python_validation():
 def test_ctypes_prototypes_cover_every_argument(rlk_lib):
     # A prototype with the wrong arity would corrupt the call; compare with the header.
     text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
-    for name in ("rlk_det_gemm_bf16", "rlk_linear_logp_fwd", "rlk_grpo_ratio_kl_loss"):
-        params = re.search(name + r"\s*\((.*?)\)\s*;", text, flags=re.S).group(1)
-        assert len(getattr(rlk_lib, name).argtypes) == params.count(",") + 1, name
+    from rl_engine import _lib
+
+    for name in _lib.EXPORTED_SYMBOLS:
+        params = re.search(r"\b" + name + r"\s*\((.*?)\)\s*;", text, flags=re.S).group(1).strip()
+        declared = 0 if params == "void" else params.count(",") + 1
+        assert len(getattr(rlk_lib, name).argtypes) == declared, name
     assert rlk_lib.rlk_linear_logp_workspace_bytes.restype is ctypes.c_size_t
 
 
