@@ -53,7 +53,7 @@ def _parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-logp", action="store_true", help="skip the linear-LogP leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-T table")
-    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|logp|logp_decode|logp_mid|logp_bwd|from_logits|ffn|tree|copy (used for profiling)")
+    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|down_t16|down_t64|logp|logp_decode|logp_mid|logp_bwd|from_logits|ffn|tree|copy (used for profiling)")
     return ap.parse_args()
 
 
@@ -173,6 +173,14 @@ def main() -> int:
         tgt = torch.randint(0, VOCAB, (tl,), generator=gen, device=dev)
         ms = _time_calls(lambda: deterministic_linear_logp(hid, w_lm, tgt), args.steps, args.warmup)
         print(json.dumps({"leg": args.only, "tokens": tl, "ms": ms, "weight_gbps": 2.0 * VOCAB * HIDDEN / ms * 1e-6,
+                          "launches": args.steps + args.warmup}))
+        return 0
+    if args.only in ("down_t16", "down_t64"):
+        # the streaming kernel: 16-feature weight panels against 16 / 64 tokens
+        ts = 16 if args.only == "down_t16" else 64
+        h_s, o_s = h[:ts], out_d[:ts]
+        ms = _time_calls(lambda: gemm.mfma_gemm(h_s, w_d.t(), out=o_s), args.steps, args.warmup)
+        print(json.dumps({"leg": args.only, "tokens": ts, "ms": ms, "gbps": _gemm_bytes(ts, HIDDEN, INTER) / ms * 1e-6,
                           "launches": args.steps + args.warmup}))
         return 0
     if args.only == "tree":
