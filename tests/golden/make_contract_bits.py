@@ -58,6 +58,21 @@ def contract_bits() -> dict:
         "small_linear_logp.logp_bias_temp_pad": _sha(logp2),
         "small_linear_logp.lse_bias_temp_pad": _sha(lse2),
     }
+    # gradients of the fused linear-LogP (same contract id: the backward is part of it)
+    from rl_engine import _C
+
+    g = torch.linspace(-1.0, 1.0, h.size(0), device=dev)
+    grad_h, grad_w, _ = _C.fused_linear_logp_bwd(h, w, t, lse, g, None)
+    out[lib.rlk_linear_logp_contract_id().decode()]["small_linear_logp.grad_hidden"] = _sha(grad_h)
+    out[lib.rlk_linear_logp_contract_id().decode()]["small_linear_logp.grad_weight"] = _sha(grad_w)
+    # gated FFN on the same hidden states: packed gate/up projection + SwiGLU, then down
+    from rl_engine.ops.ffn import qwen3_ffn_packed_inference
+
+    w_gu = inputs.randn_bf16(9901, 2 * 192, h.size(1), 0.1).to(dev)
+    w_d = inputs.randn_bf16(9902, h.size(1), 192, 0.1).to(dev)
+    out[lib.rlk_contract_id().decode()]["small_gated_ffn"] = _sha(qwen3_ffn_packed_inference(h, w_gu, w_d))
+    big = inputs.randn_bf16(9903, 200, h.size(1)).to(dev)  # above 128 tokens: the fused projection kernel
+    out[lib.rlk_contract_id().decode()]["gated_ffn_200_tokens"] = _sha(qwen3_ffn_packed_inference(big, w_gu, w_d))
     return out
 
 
