@@ -503,10 +503,12 @@ def test_weight_transpose_cache_refresh(gemm):
         gemm.prepare_det_gemm_linear_weight(w, out=w.view(32, 24))
 
 
-def test_hip_graph_capture_replays_bit_identically(gemm):
-    a = inputs.randn_bf16(131, 16, 4096).to(DEV)
+@pytest.mark.parametrize("rows", (16, 48, 300))
+def test_hip_graph_capture_replays_bit_identically(gemm, rows):
+    # 16 and 48 rows: the streaming kernel (one and three token tiles); 300: a tile kernel
+    a = inputs.randn_bf16(131, rows, 4096).to(DEV)
     w = inputs.randn_bf16(132, 4096, 4096, 0.02).to(DEV)
-    out = torch.empty((16, 4096), dtype=torch.bfloat16, device=DEV)
+    out = torch.empty((rows, 4096), dtype=torch.bfloat16, device=DEV)
     eager = gemm.det_gemm_linear(a, w)
     stream = torch.cuda.Stream()
     stream.wait_stream(torch.cuda.current_stream())

@@ -217,3 +217,24 @@ def test_tree_backend_routes_the_whole_facade(gemm, oracle, monkeypatch):
     assert np.array_equal(inputs.bits(b2.grad), oracle.k_tree_gemm(inputs.bits(x.t().contiguous()), inputs.bits(dy.t().contiguous())))
     monkeypatch.setattr(gemm, "_REQUESTED_BACKEND", "auto")
     assert gemm.det_gemm_backend() == "hip_mfma"
+
+
+def test_tree_gemm_is_graph_capturable(gemm):
+    a = inputs.randn_bf16(9900, 40, 1024).to(DEV)
+    w = inputs.randn_bf16(9901, 200, 1024, 0.02).to(DEV)
+    out = torch.empty((40, 200), dtype=torch.bfloat16, device=DEV)
+    eager = gemm.tree_gemm(a, w.t())
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        gemm.tree_gemm(a, w.t(), out=out)  # warm-up outside capture
+    torch.cuda.current_stream().wait_stream(stream)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        gemm.tree_gemm(a, w.t(), out=out)
+    for _ in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert _same_bits(out, eager)
