@@ -152,16 +152,17 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_partial_kernel(LogpAr
 // linear_logp_stream_merge_kernel, which repeats the in-kernel stream merge above. Same bits
 // as every other configuration.
 template <class S, int NS>
-__global__ __launch_bounds__(S::kThreads) void linear_logp_streamgroup_kernel(LogpArgs a, float* __restrict__ spart) {
+__global__ __launch_bounds__(S::kThreads) void linear_logp_streamgroup_kernel(LogpArgs a, float* __restrict__ spart,
+                                                                              int split_first, int split_count) {
   static_assert(S::BN == kLogpTileCols && S::kRun == 16 && S::WN == 4, "wave column = tile of the split");
   constexpr int kGroups = kLogpStreams / 4;  // stream groups per split
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
-  const int total = a.tiles_m * a.n_split * kGroups;
+  const int total = a.tiles_m * split_count * kGroups;  // this launch covers splits [split_first, + split_count)
   const int id = xcd_compact_id(blockIdx.x, total);
   const int tile_m = id % a.tiles_m;
   const int unit = id / a.tiles_m;
-  const int split = unit / kGroups;
+  const int split = split_first + unit / kGroups;
   const int sg = unit % kGroups;
   const int m0 = tile_m * S::BM;
   const int n0 = split * kLogpSplitCols + sg * 64;
@@ -366,7 +367,8 @@ static hipError_t launch_logp(LogpArgs a, hipStream_t stream) {
 // Up to 128 tokens every weight tile is used by one workgroup only: three stages for the
 // 64- and 128-token tiles (120 / 144 KiB); the 256-token tile has room for two.
 template <class S>
-static hipError_t launch_streamgroup(LogpArgs a, hipStream_t stream) {
+static hipError_t launch_streamgroup_range(LogpArgs a, float* spart, int split_first, int split_count,
+                                           hipStream_t stream) {
   constexpr int kStages = S::BM <= 128 ? 3 : 2;
   auto kernel = linear_logp_streamgroup_kernel<S, kStages>;
   constexpr int kLdsBytes = kStages * S::kStageBytes;
@@ -374,11 +376,34 @@ static hipError_t launch_streamgroup(LogpArgs a, hipStream_t stream) {
   hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLdsBytes, once);
   if (err != hipSuccess) return err;
   a.tiles_m = (a.T + S::BM - 1) / S::BM;
+  hipLaunchKernelGGL(kernel, dim3(a.tiles_m * split_count * (kLogpStreams / 4)), dim3(S::kThreads), kLdsBytes, stream,
+                     a, spart, split_first, split_count);
+  return hipGetLastError();
+}
+
+// `balance`: with the 256-token tile, a last round that would fill at most half of the chip
+// runs as 128-token tiles instead (twice the workgroups, each about 0.57 of the time): for
+// 256 tokens and V = 151936, 596 workgroups are 2.33 rounds of 256; 512 of them plus 168
+// half-height ones are two rounds and a short one (350 -> 290 us). Same bits: the tile height
+// is not part of the contract.
+template <class S>
+static hipError_t launch_streamgroup(LogpArgs a, bool balance, hipStream_t stream) {
+  constexpr int kCus = 256;
   float* spart = a.part + (size_t)3 * a.n_split * a.T;  // behind the per-split partials
-  hipLaunchKernelGGL(kernel, dim3(a.tiles_m * a.n_split * (kLogpStreams / 4)), dim3(S::kThreads), kLdsBytes, stream,
-                     a, spart);
-  err = hipGetLastError();
+  const int tiles_m = (a.T + S::BM - 1) / S::BM;
+  const int per_split = tiles_m * (kLogpStreams / 4);
+  int main_splits = a.n_split;
+  if (balance && S::BM == 256 && per_split <= kCus && kCus % per_split == 0) {
+    const int per_round = kCus / per_split;
+    const int tail = a.n_split % per_round;
+    if (tail * per_split * 2 <= kCus && a.n_split > tail) main_splits = a.n_split - tail;
+  }
+  hipError_t err = launch_streamgroup_range<S>(a, spart, 0, main_splits, stream);
   if (err != hipSuccess) return err;
+  if (main_splits < a.n_split) {
+    err = launch_streamgroup_range<LogpShape128>(a, spart, main_splits, a.n_split - main_splits, stream);
+    if (err != hipSuccess) return err;
+  }
   const int threads = a.T * a.n_split;
   hipLaunchKernelGGL(linear_logp_stream_merge_kernel, dim3((threads + 255) / 256), dim3(256), 0, stream, spart,
                      a.part, a.T, a.n_split);
@@ -419,6 +444,7 @@ hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t*
                    (reinterpret_cast<uintptr_t>(H.ptr) & 15) == 0 && (D % kChunkElems) == 0;
   const bool force_staged = (config & RLK_LOGP_CFG_FORCE_STAGED) != 0;
   config &= ~RLK_LOGP_CFG_FORCE_STAGED;
+  const int requested = config;
   if (config == RLK_LOGP_CFG_AUTO) config = pick_linear_logp_config(T, V);
   if (!vec && config == RLK_LOGP_CFG_256) config = RLK_LOGP_CFG_128;
   const int loop = !vec ? 0 : (D % kTileK == 0 && !force_staged) ? 2 : 1;
@@ -431,13 +457,13 @@ hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t*
   hipError_t err;
   switch (config) {
     case RLK_LOGP_CFG_64_STREAMS:
-      err = launch_streamgroup<LogpShape64>(a, stream);
+      err = launch_streamgroup<LogpShape64>(a, false, stream);
       break;
     case RLK_LOGP_CFG_128_STREAMS:
-      err = launch_streamgroup<LogpShape128>(a, stream);
+      err = launch_streamgroup<LogpShape128>(a, false, stream);
       break;
     case RLK_LOGP_CFG_256_STREAMS:
-      err = launch_streamgroup<LogpShape256>(a, stream);
+      err = launch_streamgroup<LogpShape256>(a, requested == RLK_LOGP_CFG_AUTO, stream);
       break;
     case RLK_LOGP_CFG_256:
       err = loop == 2 ? launch_logp<LogpShape256, 2>(a, stream) : launch_logp<LogpShape256, 1>(a, stream);
