@@ -53,7 +53,7 @@ def _parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-logp", action="store_true", help="skip the linear-LogP leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-T table")
-    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|gate_up_tN|down_tN|logp|logp_decode|logp_mid|logp_bwd|from_logits|ffn|tree|copy (used for profiling)")
+    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|gate_up_tN|down_tN|logp|logp_decode|logp_mid|logp_bwd|from_logits|ffn|tree|copy|power (used for profiling)")
     return ap.parse_args()
 
 
@@ -188,6 +188,41 @@ def main() -> int:
         ms = _time_calls(lambda: gemm.mfma_gemm(a_s, w_s.t(), out=o_s), args.steps, args.warmup)
         print(json.dumps({"leg": args.only, "tokens": ts, "ms": ms, "gbps": _gemm_bytes(ts, n_s, k_s) / ms * 1e-6,
                           "launches": args.steps + args.warmup}))
+        return 0
+    if args.only == "power":
+        # Board power (hwmon, microwatts) while the gate_up GEMM loops on the benchmark's random
+        # operands and on all-zero operands: the same instruction stream at two data-toggle rates.
+        import glob
+
+        def hwmon(name):
+            vals = []
+            for f in glob.glob(f"/sys/class/drm/card*/device/hwmon/hwmon*/{name}"):
+                try:
+                    vals.append(int(open(f).read()) / 1e6)
+                except (OSError, ValueError):
+                    pass
+            return max(vals) if vals else None
+
+        def looped(a_op, w_op, seconds=3.0):
+            for _ in range(50):
+                gemm.mfma_gemm(a_op, w_op.t(), out=out_gu)
+            torch.cuda.synchronize()
+            t0, n, watts = time.perf_counter(), 0, []
+            while time.perf_counter() - t0 < seconds:
+                for _ in range(200):
+                    gemm.mfma_gemm(a_op, w_op.t(), out=out_gu)
+                n += 200
+                watts.append(hwmon("power1_average") or hwmon("power1_input"))  # sampled while the queue is busy
+                torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            watts = sorted(w for w in watts if w is not None)
+            return {"tflops": round(2.0 * T * 2 * INTER * HIDDEN * n / dt * 1e-12, 1),
+                    "watts": watts[len(watts) // 2] if watts else None}
+
+        idle = hwmon("power1_average") or hwmon("power1_input")
+        res = {"leg": "power", "cap_watts": hwmon("power1_cap"), "idle_watts": idle,
+               "random_operands": looped(x, w_gu), "zero_operands": looped(torch.zeros_like(x), torch.zeros_like(w_gu))}
+        print(json.dumps(res))
         return 0
     if args.only == "tree":
         ms = _time_calls(lambda: gemm.tree_gemm(x, w_gu.t(), out=out_gu), args.steps, args.warmup)
