@@ -143,3 +143,112 @@ def test_gated_projection_and_k_tree_rows():
         alone = torch.empty(1, inter, device=DEV, dtype=torch.bfloat16)
         _C.gemm_tree_strided(a[row : row + 1], w[:inter].t(), alone)
         assert _same(tree[row : row + 1], alone), (case, m, inter, k, row)
+
+
+def test_linear_logp_backward_configurations_rows_and_values():
+    from rl_engine import _C, _lib
+
+    d = _Draw(9400)
+    for case in range(80):
+        t = int(d.rng.integers(1, 400)) if d.rng.random() < 0.85 else int(d.rng.integers(400, 1400))
+        v, hidden = int(d.rng.integers(1, 5000)), 32 * int(d.rng.integers(1, 16))
+        h, w = d.bf16(t, hidden), d.bf16(v, hidden, scale=0.1)
+        real = v if d.rng.random() < 0.5 else int(d.rng.integers(1, v + 1))
+        start = 0 if d.rng.random() < 0.6 else int(d.rng.integers(0, 100000))
+        tgt = torch.randint(max(start - 3, 0), start + real + 3, (t,), device=DEV, generator=d.gen)
+        bias = torch.randn(v, device=DEV, generator=d.gen) if d.rng.random() < 0.4 else None
+        temp = (torch.rand(t, device=DEV, generator=d.gen) + 0.5) if d.rng.random() < 0.4 else None
+        g_logp = torch.randn(t, device=DEV, generator=d.gen) if d.rng.random() < 0.8 else None
+        g_lse = torch.randn(t, device=DEV, generator=d.gen) if (d.rng.random() < 0.4 or g_logp is None) else None
+        where = (case, t, v, hidden, real, start, bias is not None, temp is not None, g_logp is None, g_lse is None)
+        _, lse = _C.fused_linear_logp(h, w, tgt, bias, temp, False, real, vocab_start_index=start)
+        base = None
+        for name, code in _lib.LOGP_CONFIGS.items():
+            for staged in (0, _lib.FORCE_STAGED):
+                if staged and d.rng.random() < 0.6:
+                    continue
+                out = _C.fused_linear_logp_bwd(
+                    h, w, tgt, lse, g_logp, g_lse, bias, temp, real, vocab_start_index=start,
+                    need_grad_bias=bias is not None, config=code | staged,
+                )  # fmt: skip
+                if base is None:
+                    base = out
+                for got, want in zip(out, base):
+                    assert (got is None) == (want is None), where + (name, staged)
+                    assert got is None or _same(got, want), where + (name, staged)
+        row = int(d.rng.integers(0, t))
+        cut = slice(row, row + 1)
+        alone = _C.fused_linear_logp_bwd(
+            h[cut].contiguous(), w, tgt[cut].contiguous(), lse[cut].contiguous(),
+            None if g_logp is None else g_logp[cut].contiguous(), None if g_lse is None else g_lse[cut].contiguous(),
+            bias, None if temp is None else temp[cut].contiguous(), real, vocab_start_index=start, need_grad_weight=False,
+        )  # fmt: skip
+        assert _same(alone[0], base[0][cut]), where + (row,)
+        # values: fp64 gradients of the bf16-rounded d(logits)
+        z = h.double() @ w.double().t()
+        if bias is not None:
+            z = z + bias.double()
+        z[:, real:] = float("-inf")
+        if temp is not None:
+            z = z / temp.double()[:, None]
+        p = torch.exp(z - lse.double()[:, None])
+        gl = torch.zeros(t, device=DEV, dtype=torch.float64) if g_logp is None else g_logp.double()
+        gs = torch.zeros(t, device=DEV, dtype=torch.float64) if g_lse is None else g_lse.double()
+        dz = p * (gs - gl)[:, None]
+        local = tgt - start
+        owned = (local >= 0) & (local < real)
+        dz[torch.arange(t, device=DEV)[owned], local[owned]] += gl[owned]
+        if temp is not None:
+            dz = dz / temp.double()[:, None]
+        dz = dz.to(torch.bfloat16).double()
+        for got, ref in ((base[0], dz @ w.double()), (base[1], dz.t() @ h.double())):
+            scale = max(ref.abs().max().item(), 1e-6)
+            assert (got.double() - ref).abs().max().item() <= 2.0**-6 * scale, where
+
+
+def test_logits_side_kernels_dtypes_pitches_and_rows():
+    from rl_engine import _C
+
+    d = _Draw(9500)
+    for case in range(150):
+        rows, tiles = int(d.rng.integers(1, 300)), int(d.rng.choice([1, 2, 8, 64]))
+        v = tiles * int(d.rng.integers(1, 120))
+        dtype = [torch.bfloat16, torch.float16, torch.float32][int(d.rng.integers(0, 3))]
+        pad = int(d.rng.choice([0, 0, 8, 5]))
+        logits = (torch.randn(rows, v + pad, device=DEV, generator=d.gen) * 3).to(dtype)[:, :v]
+        real = int(d.rng.integers(1, v + 1)) if d.rng.random() < 0.5 else v
+        start = 0 if d.rng.random() < 0.6 else int(d.rng.integers(0, 100000))
+        tgt = torch.randint(start, start + real, (rows,), device=DEV, generator=d.gen)
+        temp = (torch.rand(rows, device=DEV, generator=d.gen) + 0.5) if d.rng.random() < 0.4 else None
+        where = (case, rows, v, tiles, real, start, str(dtype), pad, temp is not None)
+        logp, lse = _C.hip_deterministic_logp_from_logits(logits, tgt, start, start + real, tiles, temperature=temp)
+        z = logits.double()[:, :real]
+        if temp is not None:
+            z = z / temp.double()[:, None]
+        lse64 = torch.logsumexp(z, -1)
+        zt = z.gather(1, (tgt - start)[:, None])[:, 0]
+        tol = 1e-3 if dtype == torch.float32 else 2e-3
+        assert (lse.double() - lse64).abs().max().item() <= tol, where
+        assert (logp.double() - (zt - lse64)).abs().max().item() <= tol, where
+        row = int(d.rng.integers(0, rows))
+        cut = slice(row, row + 1)
+        lp1, lse1 = _C.hip_deterministic_logp_from_logits(
+            logits[cut], tgt[cut].contiguous(), start, start + real, tiles,
+            temperature=None if temp is None else temp[cut].contiguous(),
+        )  # fmt: skip
+        assert _same(lp1, logp[cut]) and _same(lse1, lse[cut]), where + (row,)
+        c_logp = torch.randn(rows, device=DEV, generator=d.gen)
+        c_lse = torch.randn(rows, device=DEV, generator=d.gen)
+        with_lse = bool(d.rng.random() < 0.5)
+        grad = _C.hip_deterministic_logp_backward(
+            logits, lse, c_logp, c_lse, (tgt - start).contiguous(), start, start + real, with_lse, temperature=temp
+        )
+        p = torch.exp(z - lse.double()[:, None])
+        ref = torch.zeros(rows, v, device=DEV, dtype=torch.float64)
+        ref[:, :real] = p * ((c_lse.double() if with_lse else 0.0) - c_logp.double())[:, None]
+        ref[torch.arange(rows, device=DEV), tgt - start] += c_logp.double()
+        if temp is not None:
+            ref = ref / temp.double()[:, None]
+        eps = {torch.bfloat16: 2.0**-7, torch.float16: 2.0**-9, torch.float32: 1e-4}[dtype]
+        scale = max(ref.abs().max().item(), c_logp.abs().max().item(), c_lse.abs().max().item())
+        assert (grad.double() - ref).abs().max().item() <= eps * scale + 1e-6, where
