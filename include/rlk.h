@@ -51,7 +51,8 @@ typedef enum rlk_gemm_config {
   RLK_GEMM_CFG_128x64_DEEP = 12,  /* 128x64 tile, 128 K values per barrier pair */
   RLK_GEMM_CFG_128x128_DEEP = 13, /* 128x128 tile, 128 K values per barrier pair */
   RLK_GEMM_CFG_STREAM64 = 14,     /* M <= 64: 16-feature panels streamed through an LDS ring, one consumer wave per 16 tokens */
-  RLK_GEMM_CFG_COUNT = 15,
+  RLK_GEMM_CFG_256x256_SOLO = 15, /* 256 x 256 tile on four waves (one per SIMD, 128 x 128 each) */
+  RLK_GEMM_CFG_COUNT = 16,
   /* OR-ed into a configuration: use the register-staged main loop even where the
    * direct-to-LDS ping-pong loop applies. Bit-neutral; exists so tests can
    * compare the two loops. */

@@ -21,7 +21,8 @@ enum : int {
   kLoopPingPong = 2,
   kLoopPingPongKMajor = 3,   // weight K-major
   kLoopPingPongXKMajor = 4,  // activation K-major
-  kLoopPingPongBothKMajor = 5
+  kLoopPingPongBothKMajor = 5,
+  kLoopSolo = 6  // four waves, one per SIMD
 };
 constexpr bool loop_weight_kmajor(int loop) { return loop == kLoopPingPongKMajor || loop == kLoopPingPongBothKMajor; }
 constexpr bool loop_act_kmajor(int loop) { return loop == kLoopPingPongXKMajor || loop == kLoopPingPongBothKMajor; }
@@ -47,7 +48,9 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
   const int m0 = tile_m * S::BM;
 
   f32x4_t acc[S::TN][S::TM];
-  if constexpr (LOOP >= kLoopPingPongKMajor) {
+  if constexpr (LOOP == kLoopSolo) {
+    tile_mainloop_solo<S>(W, X, n0, m0, K, lds, acc);
+  } else if constexpr (LOOP >= kLoopPingPongKMajor) {
     tile_mainloop_pingpong<S, loop_weight_kmajor(LOOP), loop_act_kmajor(LOOP)>(W, X, n0, m0, K, lds, acc);
   } else if constexpr (LOOP == kLoopPingPong) {
     tile_mainloop_pingpong<S, false, false, PlainRowMap<S>, KS, NS>(W, X, n0, m0, K, lds, acc);
@@ -212,6 +215,7 @@ static hipError_t launch_deep(const MatView& W, const MatView& X, void* C, int64
 
 // Tile shapes. Which one runs is a pure performance choice (see det_gemm_tile.h).
 using Shape256x256 = TileShape<256, 256, 4, 2>;
+using Shape256x256Solo = TileShape<256, 256, 2, 2>;
 using Shape256x128 = TileShape<256, 128, 4, 2>;
 using Shape256x64 = TileShape<256, 64, 4, 2>;
 using Shape128x128 = TileShape<128, 128, 4, 2>;
@@ -345,6 +349,11 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
   // flight; the largest shapes would spill registers with it.
   if (!vec && (config == RLK_GEMM_CFG_256x256 || config == RLK_GEMM_CFG_256x128 || config == RLK_GEMM_CFG_256x64))
     config = RLK_GEMM_CFG_128x128;
+  if (config == RLK_GEMM_CFG_256x256_SOLO) {
+    if (vec && allow_pingpong && K % kTileK == 0)
+      return launch_loop<Shape256x256Solo, kLoopSolo>(W, X, C, ldc, M, N, K, out_f32, stream);
+    config = RLK_GEMM_CFG_256x256;
+  }
   switch (config) {
     case RLK_GEMM_CFG_256x256:
       return launch_shape<Shape256x256>(W, X, C, ldc, M, N, K, vec, 0, allow_pingpong, out_f32, stream);

@@ -445,6 +445,17 @@ struct DmaLoader {
     __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + (kBlocksW + xb) * 1024), 16, 0, 0);
   }
 
+  // The same for a native-layout tile that lies inside both matrices: no clamping.
+  __device__ __forceinline__ void load_w_block_inside(char* stage, int k0, int b) const {
+    const bf16_bits* src = w_base + (int64_t)(Map::block_half(b) * n_rows + Map::block_offset(b)) * ldw + k0 +
+                           w_lane_off[b & 1];
+    __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + b * 1024), 16, 0, 0);
+  }
+  __device__ __forceinline__ void load_x_block_inside(char* stage, int k0, int xb) const {
+    const bf16_bits* src = x_base + (int64_t)(xb * 8) * ldx + k0 + x_lane_off;
+    __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + (kBlocksW + xb) * 1024), 16, 0, 0);
+  }
+
   // `wave` is the workgroup wave index 0..7.
   __device__ __forceinline__ void issue_early(char* stage, int k0, int wave) const {
 #pragma unroll
@@ -678,6 +689,183 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
   }
   __builtin_amdgcn_s_waitcnt(kWaitAll0);
   wg_barrier();  // callers reuse the LDS after the loop
+}
+
+// ---------------------------------------------------------------------------
+// One wave per SIMD: four waves, each a 128 x 128 quarter of a 256 x 256 tile.
+//
+// A square wave tile reads 16 fragments from LDS per 64 MFMAs (the 64 x 128 wave tiles of
+// the ping-pong loop: 12 per 32). Its 256 accumulator registers and two sets of 16
+// fragments need the whole unified register file of a SIMD, so a wave has no partner to
+// hide its stalls: fragment reads of K step s + 1 and the direct-to-LDS loads of K tile
+// t + 2 are issued under the MFMAs of step s, and there is one barrier per K tile.
+//
+//   iteration t (tile t in stage t & 1; F0 = fragments of its first K step, already in registers)
+//     read F1 (second K step of tile t)           | MFMAs on F0
+//     wait: F1 in registers, my loads of tile t + 1 landed; barrier
+//     start the loads of tile t + 2 into stage t & 1, read F0 of tile t + 1 | MFMAs on F1
+//
+// Same MFMA chain per output element as every other loop. Needs the native layouts,
+// 16-byte aligned rows and K % 64 == 0.
+// ---------------------------------------------------------------------------
+template <class S>
+constexpr bool solo_supported() {
+  return S::WN == 2 && S::WM == 2 && S::BN == 256 && S::BM == 256;
+}
+
+template <bool V>
+struct BoolTag {
+  static constexpr bool value = V;
+};
+
+template <class S, bool INSIDE>
+__device__ __forceinline__ void tile_mainloop_solo_impl(const MatView& W, const MatView& X, int n0, int m0, int K,
+                                                        char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
+  static_assert(solo_supported<S>(), "four waves of 128 x 128");
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave_n = wave % S::WN;
+  const int wave_m = wave / S::WN;
+  const int l16 = lane & 15;
+  const int grp = lane >> 4;
+
+  using Loader = DmaLoader<S>;
+  Loader loader;
+  loader.init(W, X, n0, m0, lane);
+  constexpr int kBlocksW = S::BN / 8, kBlocksX = S::BM / 8;
+  constexpr int kLoads = (kBlocksW + kBlocksX) / 4;  // blocks (load instructions) per wave and K tile
+  static_assert(kBlocksW == 2 * kLoads && kBlocksX == 2 * kLoads, "waves 0, 1 load weight rows, waves 2, 3 token rows");
+  // Inside the matrices a block's 64 addresses are a uniform base (operand, 128-row half of
+  // the tile, block) plus one of two lane offsets, the same for every K tile.
+  const bool loads_weights = wave < 2;
+  const bf16_bits* my_base = (loads_weights ? loader.w_base : loader.x_base);
+  const int64_t my_ld = loads_weights ? loader.ldw : loader.ldx;
+  const uint32_t my_off[2] = {loads_weights ? loader.w_lane_off[0] : loader.x_lane_off,
+                              loads_weights ? loader.w_lane_off[1] : loader.x_lane_off};
+  my_base += (int64_t)((wave & 1) * (kLoads * 8)) * my_ld;
+  auto issue_tile = [&](char* st, int k0) {
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+      const int b = wave * kLoads + j;
+      if constexpr (INSIDE) {
+        // weight block j of a 128-row wave column holds features 4 (j >> 1) + (lane part); token block j rows 8 j ..
+        const int rows = loads_weights ? 4 * (j >> 1) : 8 * j;
+        const bf16_bits* src = my_base + (int64_t)rows * my_ld + k0 + my_off[j & 1];
+        __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(st + b * 1024), 16, 0, 0);
+      } else if (loads_weights) {
+        loader.load_w_block(st, k0, b);
+      } else {
+        loader.load_x_block(st, k0, b - kBlocksW);
+      }
+    }
+  };
+
+#pragma unroll
+  for (int jn = 0; jn < S::TN; ++jn)
+#pragma unroll
+    for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const int frag_lo = (grp ^ (l16 & 7)) << 4;
+  const int w_row_base = (wave_n * 16 * S::TN + l16) * kRowBytes;
+  const int x_row_base = S::BN * kRowBytes + (wave_m * 16 * S::TM + l16) * kRowBytes;
+  u32x4_t w0[S::TN], x0[S::TM], w1[S::TN], x1[S::TM];
+  auto read_step = [&](const char* st, int step, u32x4_t (&wf)[S::TN], u32x4_t (&xf)[S::TM]) {
+    const int frag = frag_lo ^ (step << 6);
+#pragma unroll
+    for (int jn = 0; jn < S::TN; ++jn)
+      wf[jn] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + jn * 16 * kRowBytes + frag);
+#pragma unroll
+    for (int jm = 0; jm < S::TM; ++jm)
+      xf[jm] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + jm * 16 * kRowBytes + frag);
+  };
+  auto mfma_step = [&](const u32x4_t (&wf)[S::TN], const u32x4_t (&xf)[S::TM]) {
+#pragma unroll
+    for (int jn = 0; jn < S::TN; ++jn)
+#pragma unroll
+      for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = mfma_16x16x32(wf[jn], xf[jm], acc[jn][jm]);
+  };
+  constexpr int kReads = S::TN + S::TM;    // fragment reads per K step
+  constexpr int kMfmas = S::TN * S::TM;    // MFMAs per K step
+  static_assert(kMfmas % kReads == 0 && kMfmas % (2 * kLoads) == 0, "whole interleave groups");
+
+  const int nk = K / kTileK;
+  char* const st0 = lds;
+  char* const st1 = lds + S::kStageBytes;
+  issue_tile(st0, 0);
+  if (nk > 1) issue_tile(st1, kTileK);
+  if (nk > 1) {
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt(kLoads));  // my part of tile 0 has landed
+  } else {
+    __builtin_amdgcn_s_waitcnt(kWaitVm0);
+  }
+  wg_barrier();
+  read_step(st0, 0, w0, x0);
+  __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
+
+  // One K tile. LOAD: tile t + 2 exists; READ: tile t + 1 exists. Written in issue order, one
+  // row of MFMA tiles at a time with its share of the reads and loads in front; the fences keep
+  // the compiler from regrouping them.
+  static_assert(S::TN == S::TM && kLoads == 2 * S::TN, "one weight and one token fragment, two loads per MFMA row");
+  auto read_one = [&](const char* st, int step, int j, u32x4_t (&wf)[S::TN], u32x4_t (&xf)[S::TM]) {
+    const int frag = frag_lo ^ (step << 6);
+    wf[j] = *reinterpret_cast<const u32x4_t*>(st + w_row_base + j * 16 * kRowBytes + frag);
+    xf[j] = *reinterpret_cast<const u32x4_t*>(st + x_row_base + j * 16 * kRowBytes + frag);
+  };
+  auto issue_two = [&](char* st, int k0, int jn) {
+#pragma unroll
+    for (int j = 2 * jn; j < 2 * jn + 2; ++j) {
+      const int b = wave * kLoads + j;
+      if constexpr (INSIDE) {
+        const int rows = loads_weights ? 4 * (j >> 1) : 8 * j;
+        const bf16_bits* src = my_base + (int64_t)rows * my_ld + k0 + my_off[j & 1];
+        __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(st + b * 1024), 16, 0, 0);
+      } else if (loads_weights) {
+        loader.load_w_block(st, k0, b);
+      } else {
+        loader.load_x_block(st, k0, b - kBlocksW);
+      }
+    }
+  };
+  auto iteration = [&](int t, auto load_tag, auto read_tag) {
+    constexpr bool LOAD = decltype(load_tag)::value, READ = decltype(read_tag)::value;
+    char* cur = (t & 1) ? st1 : st0;
+    char* nxt = (t & 1) ? st0 : st1;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int jn = 0; jn < S::TN; ++jn) {
+      read_one(cur, 1, jn, w1, x1);
+#pragma unroll
+      for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = mfma_16x16x32(w0[jn], x0[jm], acc[jn][jm]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitAll0);  // F1 in registers, my part of tile t + 1 landed
+    wg_barrier();
+#pragma unroll
+    for (int jn = 0; jn < S::TN; ++jn) {
+      if constexpr (LOAD) issue_two(cur, (t + 2) * kTileK, jn);
+      if constexpr (READ) read_one(nxt, 0, jn, w0, x0);
+#pragma unroll
+      for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = mfma_16x16x32(w1[jn], x1[jm], acc[jn][jm]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (READ) __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // F0 of tile t + 1 in registers
+  };
+  int t = 0;
+  for (; t + 2 < nk; ++t) iteration(t, BoolTag<true>{}, BoolTag<true>{});
+  if (t + 1 < nk) iteration(t++, BoolTag<false>{}, BoolTag<true>{});
+  iteration(t, BoolTag<false>{}, BoolTag<false>{});
+  __builtin_amdgcn_s_waitcnt(kWaitAll0);
+  wg_barrier();  // callers reuse the LDS after the loop
+}
+
+template <class S>
+__device__ __forceinline__ void tile_mainloop_solo(const MatView& W, const MatView& X, int n0, int m0, int K,
+                                                   char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
+  if (n0 + S::BN <= W.rows && m0 + S::BM <= X.rows) {
+    tile_mainloop_solo_impl<S, true>(W, X, n0, m0, K, lds, acc);
+  } else {
+    tile_mainloop_solo_impl<S, false>(W, X, n0, m0, K, lds, acc);
+  }
 }
 
 }  // namespace rlk

@@ -37,6 +37,7 @@ GEMM_CONFIGS = {
     "128x64_deep": 12,
     "128x128_deep": 13,
     "stream64": 14,
+    "256x256_solo": 15,
 }
 # OR-ed into a GEMM or LogP configuration: register-staged main loop (bit-neutral).
 FORCE_STAGED = 0x100
