@@ -524,3 +524,50 @@ def test_hip_graph_capture_replays_bit_identically(gemm, rows):
         graph.replay()
         torch.cuda.synchronize()
         assert _same_bits(out, eager)
+
+
+def test_host_threads_on_their_own_streams(gemm):
+    """Four host threads, each with its own stream and shapes (so each reaches other kernels),
+    launch concurrently; every result equals the one the main thread computed alone. The library
+    keeps no state between calls except the per-device 'attribute set' flags and a per-thread
+    error string."""
+    import threading
+
+    from rl_engine.ops import logprob
+
+    shapes = ((5, 1536, 4096), (48, 4096, 4096), (300, 1024, 2048), (1024, 2048, 1024))
+    cases = []
+    for i, (m, n, k) in enumerate(shapes):
+        a = inputs.randn_bf16(141 + i, m, k).to(DEV)
+        w = inputs.randn_bf16(151 + i, n, k, 0.02).to(DEV)
+        tgt = torch.randint(0, n, (m,), device=DEV, generator=torch.Generator(device=DEV).manual_seed(161 + i))
+        cases.append((a, w, tgt, gemm.det_gemm_linear(a, w), logprob.deterministic_linear_logp(a, w, tgt)))
+    torch.cuda.synchronize()
+    results: list = [None] * len(cases)
+    errors: list = []
+
+    def worker(i):
+        try:
+            a, w, tgt, _, _ = cases[i]
+            stream = torch.cuda.Stream()
+            got = []
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    got.append((gemm.det_gemm_linear(a, w), logprob.deterministic_linear_logp(a, w, tgt)))
+            stream.synchronize()
+            results[i] = got
+        except Exception as exc:  # surfaced in the main thread
+            errors.append((i, repr(exc)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(cases))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    for i, (_, _, _, want, (want_logp, want_lse)) in enumerate(cases):
+        assert results[i] is not None and len(results[i]) == 20
+        for out, (logp, lse) in results[i]:
+            assert _same_bits(out, want), i
+            assert torch.equal(logp.view(torch.int32), want_logp.view(torch.int32)), i
+            assert torch.equal(lse.view(torch.int32), want_lse.view(torch.int32)), i
