@@ -235,14 +235,13 @@ static int64_t tile_count(int M, int N, int bm, int bn) {
 
 int pick_det_gemm_config(int M, int N, int K) {
   constexpr int kCus = 256;
-  // Decode: many short panels keep the chip busy with one wave each; few long
-  // panels need the streaming kernel's deep ring.
-  // Decode: many short panels keep the chip busy with one wave each; few long panels need
-  // the streaming kernel's deep ring (one 16-feature panel per workgroup). Up to 32 / 64
-  // tokens the same holds while there are at most 1.5 / 1 panels per CU: a 64-token tile
-  // kernel would run on N / 64 CUs only (down projection at 32 tokens: 38 -> 19 us, the time
-  // the 100 MB weight takes through the fabric).
-  if (M <= 16) return N >= 64 * kCus ? RLK_GEMM_CFG_16x16 : RLK_GEMM_CFG_STREAM64;
+  // Decode (weights fitted while they rotate through 1.3 GB, i.e. come from HBM as in a model with
+  // many layers, not from the 256 MB memory-side cache): up to 16 tokens the streaming kernel with
+  // two workgroups per CU is the fastest or equal for every Qwen3-8B projection (gate_up 52 -> 38 us,
+  // qkv 14 -> 12 us against the one-wave tile kernel, which wins only when the weight is cache
+  // resident). Up to 32 / 64 tokens it holds while there are at most 1.5 / 1 panels per CU: a
+  // 64-token tile kernel would run on N / 64 CUs only.
+  if (M <= 16) return (K >= 1024 && K % kTileK == 0) ? RLK_GEMM_CFG_STREAM16 : RLK_GEMM_CFG_16x16;
   if (K >= 1024 && K % kTileK == 0 && ((M <= 32 && N <= 24 * kCus) || (M <= 64 && N <= 16 * kCus)))
     return RLK_GEMM_CFG_STREAM64;
   // Problems that give the chip at most one small tile per CU: the deep-stage variants
