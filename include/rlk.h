@@ -289,8 +289,8 @@ int rlk_swiglu_bwd(const void* dy, int64_t ld_dy, const void* gate, int64_t ld_g
                    void* stream);
 
 /* Bytes of workspace rlk_det_gemm_swiglu_bf16 needs for these operands: 0 when the fused
- * kernel applies (unit K strides, 16-byte aligned rows, K % 64 == 0, M > 128), else the
- * bf16 [M, 2 I] projection. */
+ * kernels apply (unit K strides, 16-byte aligned rows, K % 64 == 0, and M > 128 or M <= 16 with
+ * K >= 1024), else the bf16 [M, 2 I] projection. */
 size_t rlk_det_gemm_swiglu_workspace_bytes(const void* a, int64_t a_row_stride, const void* w_packed,
                                            int64_t w_row_stride, int M, int I, int K);
 

@@ -13,7 +13,7 @@
 // 6 TB/s chip-wide, i.e. 23 GB/s per CU: the weight panel is the slow stream, the activations
 // (re-read by every workgroup, L2 hits) the wide one. Same instruction, same ascending K order,
 // same zero start as every other det_gemm kernel, so the bits match.
-#include "det_gemm_tile.h"
+#include "linear_logp_common.h"
 #include "rlk_host.h"
 
 namespace rlk {
@@ -24,10 +24,17 @@ namespace rlk {
 // fetches the same 8-row half (producer & 1) of the (tile, sub-tile) pairs
 // (producer >> 1) + 2 j. Rows past M or N are clamped to the last valid row: computed, never
 // stored (MFMA columns and rows are independent).
-template <int KT, int RING, int MT, bool OUT_F32>
+//
+// GATED: W is a packed gate/up weight [2 I, K] (N = 2 I). The panel of workgroup b holds the gate
+// rows of features 8 b .. 8 b + 7 in its first half and their up rows in the second, so gate and
+// up of an output element sit 32 lanes apart in one accumulator; the epilogue brings them
+// together, rounds both to bf16 as the unfused projection would, and stores swiglu(gate, up) into
+// C[M, I] (bf16).
+template <int KT, int RING, int MT, bool OUT_F32, bool GATED = false>
 __global__ __launch_bounds__(64 * (MT + 4)) void det_gemm_stream_kernel(MatView W, MatView X,
                                                                               void* __restrict__ C, int64_t ldc, int M,
                                                                               int N, int K) {
+  static_assert(!(GATED && OUT_F32), "the gated projection stores bf16");
   constexpr int kSubBytes = 16 * kRowBytes;
   constexpr int kPairs = KT * (1 + MT);
   constexpr int kStageBytes = kPairs * kSubBytes;
@@ -39,7 +46,7 @@ __global__ __launch_bounds__(64 * (MT + 4)) void det_gemm_stream_kernel(MatView 
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // [0, MT): consumers, then 4 producers
   const int producer = wave - MT;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * (GATED ? 8 : 16);  // GATED: first feature of the workgroup
   const int nsub = K / kTileK;  // K % 64 == 0 on this path
   const int nstage = (nsub + KT - 1) / KT;
 
@@ -48,7 +55,12 @@ __global__ __launch_bounds__(64 * (MT + 4)) void det_gemm_stream_kernel(MatView 
   const int chunk_elems = ((lane & 7) ^ rib) * kChunkElems;
   const int half = producer & 1;
   const int r16 = half * 8 + rib;
-  const int wr = n0 + r16 < N ? n0 + r16 : N - 1;  // rows past an edge are computed, never stored
+  int wr = n0 + r16 < N ? n0 + r16 : N - 1;  // rows past an edge are computed, never stored
+  if constexpr (GATED) {
+    const int features = N / 2;
+    const int f = n0 + rib < features ? n0 + rib : features - 1;
+    wr = half * features + f;  // producers with half == 0 fetch gate rows, the others up rows
+  }
   const bf16_bits* w_base = W.ptr + (int64_t)wr * W.row_stride + chunk_elems;
   const bf16_bits* x_base[MT];
 #pragma unroll
@@ -114,6 +126,33 @@ __global__ __launch_bounds__(64 * (MT + 4)) void det_gemm_stream_kernel(MatView 
   wg_barrier();
 
   const int m = wave * 16 + l16;
+  if constexpr (GATED) {
+    if (wave < MT) {
+      // accumulator rows 4 grp + q: lane groups 0, 1 hold gate features n0 + 4 grp + q, groups 2, 3
+      // the up projection of features n0 + 4 (grp - 2) + q
+      float up[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        up[q] = __int_as_float(__builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __float_as_int(acc[q])));
+      const int f = n0 + grp * 4;
+      if (grp < 2 && m < M) {
+        bf16_bits* row = reinterpret_cast<bf16_bits*>(C) + (int64_t)m * ldc;
+        uint32_t packed[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          packed[h] = pack_bf16x2(swiglu_f32(round_through_bf16(acc[2 * h]), round_through_bf16(up[2 * h])),
+                                  swiglu_f32(round_through_bf16(acc[2 * h + 1]), round_through_bf16(up[2 * h + 1])));
+        if (f + 4 <= N / 2 && (reinterpret_cast<uintptr_t>(row + f) & 7) == 0) {
+          *reinterpret_cast<u32x2_t*>(row + f) = u32x2_t{packed[0], packed[1]};
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (f + q < N / 2) row[f + q] = (bf16_bits)((packed[q >> 1] >> ((q & 1) * 16)) & 0xffffu);
+        }
+      }
+    }
+    return;
+  }
   if (wave < MT && m < M) {
     const int n = n0 + grp * 4;
     if (OUT_F32) {
@@ -147,6 +186,19 @@ static hipError_t launch_stream(const MatView& W, const MatView& X, void* C, int
   hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLds, once);
   if (err != hipSuccess) return err;
   hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(64 * (MT + 4)), kLds, stream, W, X, C, ldc, M, N, K);
+  return hipGetLastError();
+}
+
+// Packed gate/up projection with the SwiGLU epilogue for up to 16 tokens (W.rows = 2 I, Y[M, I]):
+// the two-workgroups-per-CU geometry, I / 8 workgroups.
+hipError_t det_gemm_stream_gated_launch(const MatView& W, const MatView& X, void* Y, int64_t ldy, int M, int I, int K,
+                                        hipStream_t stream) {
+  auto kernel = det_gemm_stream_kernel<2, 8, 1, false, true>;
+  constexpr int kLds = 8 * 2 * 2 * 16 * kRowBytes;
+  static PerDeviceOnce once;
+  hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLds, once);
+  if (err != hipSuccess) return err;
+  hipLaunchKernelGGL(kernel, dim3((I + 7) / 8), dim3(64 * 5), kLds, stream, W, X, Y, ldy, M, 2 * I, K);
   return hipGetLastError();
 }
 

@@ -1,5 +1,6 @@
 // Pieces of the fused linear-LogP reduction contract shared by its forward and
-// backward kernels: the vocabulary tiling and the pinned exponential.
+// backward kernels (the vocabulary tiling and the pinned exponential), and the SwiGLU
+// arithmetic built on the same exponential.
 #pragma once
 
 #include "det_gemm_tile.h"
@@ -16,6 +17,13 @@ constexpr float kNegInf = -__builtin_huge_valf();
 __device__ __forceinline__ float pinned_exp(float x) {
   return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
 }
+
+// SwiGLU arithmetic shared by the elementwise kernels and the fused projections: s = rcp(1 + e(-g))
+// (v_rcp_f32), y = (g * s) * u, on the bf16-rounded gate and up values.
+__device__ __forceinline__ float bf16_to_f32(uint32_t bits) { return __uint_as_float(bits << 16); }
+__device__ __forceinline__ float round_through_bf16(float v) { return bf16_to_f32(pack_bf16x2(v, 0.f) & 0xffffu); }
+__device__ __forceinline__ float sigmoid_f32(float x) { return __builtin_amdgcn_rcpf(1.0f + pinned_exp(-x)); }
+__device__ __forceinline__ float swiglu_f32(float g, float u) { return (g * sigmoid_f32(g)) * u; }
 
 // The scaled logit y of the contract for accumulator value z at column `col`:
 // bias added, padded lanes -inf, then the temperature scaling.

@@ -48,6 +48,9 @@ hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int
 // two workgroups per CU.
 hipError_t det_gemm_stream_launch(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
                                   bool out_f32, bool shallow, hipStream_t stream);
+// The same kernel on a packed gate/up weight [2 I, K] with the SwiGLU epilogue, M <= 16: Y[M, I].
+hipError_t det_gemm_stream_gated_launch(const MatView& W, const MatView& X, void* Y, int64_t ldy, int M, int I, int K,
+                                        hipStream_t stream);
 
 hipError_t fill_zero_launch(void* dst, int64_t rows, int64_t cols, int64_t ld, int elem_bytes,
                             hipStream_t stream);

@@ -21,14 +21,6 @@
 
 namespace rlk {
 
-__device__ __forceinline__ float bf16_to_f32(uint32_t bits) { return __uint_as_float(bits << 16); }
-
-__device__ __forceinline__ float round_through_bf16(float v) { return bf16_to_f32(pack_bf16x2(v, 0.f) & 0xffffu); }
-
-__device__ __forceinline__ float sigmoid_f32(float x) { return __builtin_amdgcn_rcpf(1.0f + pinned_exp(-x)); }
-
-__device__ __forceinline__ float swiglu_f32(float g, float u) { return (g * sigmoid_f32(g)) * u; }
-
 // ---------------------------------------------------------------------------
 // Elementwise kernels: eight features per thread, 16-byte accesses.
 // gate[m * ld_g + c], up[m * ld_u + c]: a packed [T, 2 I] buffer is the case
@@ -256,11 +248,17 @@ static hipError_t launch_gated(const MatView& W, const MatView& X, void* Y, int6
   return hipGetLastError();
 }
 
+// Up to 16 tokens the streaming kernel serves the packed projection (the same panels of 16 weight
+// rows, eight gate and eight up), from 129 tokens on the gated tile kernels; between them the
+// projection and the activation run as two kernels (the weight read bounds the time there and the
+// GEMM kernels for few tokens spread it over more CUs than a gated 128-feature tile).
+static bool streams_gated(int M, int K) { return M <= 16 && K >= 1024; }
+
 bool det_gemm_swiglu_fused_supported(const MatView& W, const MatView& X, int M, int K) {
   auto native = [](const MatView& v) {
     return v.k_stride == 1 && (v.row_stride % kChunkElems) == 0 && (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0;
   };
-  return native(W) && native(X) && (K % kTileK) == 0 && M > 128;
+  return native(W) && native(X) && (K % kTileK) == 0 && (M > 128 || streams_gated(M, K));
 }
 
 // Y[M, I] = swiglu(X @ W[0:I]^T, X @ W[I:2I]^T). `workspace` ([M, 2 I] bf16) is used only when
@@ -270,6 +268,7 @@ bool det_gemm_swiglu_fused_supported(const MatView& W, const MatView& X, int M, 
 hipError_t det_gemm_swiglu_launch(const MatView& W, const MatView& X, void* Y, int64_t ldy, void* workspace, int M,
                                   int I, int K, hipStream_t stream) {
   if (det_gemm_swiglu_fused_supported(W, X, M, K)) {
+    if (streams_gated(M, K)) return det_gemm_stream_gated_launch(W, X, Y, ldy, M, I, K, stream);
     const int64_t t256 = (int64_t)((M + 255) / 256) * ((I + 127) / 128);
     const int64_t t128 = (int64_t)((M + 127) / 128) * ((I + 127) / 128);
     // Rounds of 256 workgroups x tokens per tile / relative throughput, as in pick_det_gemm_config:

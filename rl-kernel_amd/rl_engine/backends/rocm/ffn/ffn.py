@@ -93,7 +93,7 @@ def _packed_ffn(hidden_2d: Tensor, fused_gate_up_weight: Tensor, down_weight: Te
 
 @torch.library.custom_op("rl_kernel::qwen3_ffn_packed_inference", mutates_args=())
 def _qwen3_ffn_packed_inference(rmsnorm_output: Tensor, fused_gate_up_weight: Tensor, down_weight: Tensor) -> Tensor:
-    """Graph-safe compute of the strict rollout FFN (no host sync, no workspace for M > 128)."""
+    """Graph-safe compute of the strict rollout FFN (no host sync; no workspace for M > 128 or M <= 16)."""
     shape = rmsnorm_output.shape
     hidden_2d = rmsnorm_output.reshape(-1, shape[-1]).contiguous()
     output = _packed_ffn(hidden_2d, fused_gate_up_weight, down_weight, None)

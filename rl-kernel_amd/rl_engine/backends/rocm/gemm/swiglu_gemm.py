@@ -1,10 +1,12 @@
 """Packed gate/up projection with the SwiGLU activation in the GEMM epilogue (gfx950).
 
 Stands in for rl_engine/backends/rocm/gemm/swiglu_gemm.py:36-86 of the reference, whose
-fused path serves decode-sized batches through split-K partials. Here one MFMA kernel
+fused path serves decode-sized batches through split-K partials. Here one MFMA tile kernel
 serves every batch above 128 rows (a workgroup owns the gate and the up projection of the
-same 128 features, so the ``[M, 2 I]`` projection is never written); smaller batches run
-the GEMM for few tokens and the elementwise kernel. Both orders of work give the same bits.
+same 128 features, so the ``[M, 2 I]`` projection is never written), the streaming kernel
+serves up to 16 rows the same way (eight gate and eight up rows per weight panel), and the
+batches between run the GEMM for few tokens and the elementwise kernel. All three orders of
+work give the same bits.
 """
 
 from __future__ import annotations

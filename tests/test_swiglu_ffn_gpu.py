@@ -68,7 +68,9 @@ def test_elementwise_special_values(native):
 
 @pytest.mark.parametrize(
     "shape",
-    [(300, 256, 256), (1024, 1000, 128), (17, 128, 64), (64, 136, 4096), (513, 3000, 512), (4096, 1536, 1024), (16, 512, 256), (1, 256, 4096), (40, 256, 72), (129, 4096, 128), (128, 4096, 128), (200, 136, 64)],
+    [(300, 256, 256), (1024, 1000, 128), (17, 128, 64), (64, 136, 4096), (513, 3000, 512), (4096, 1536, 1024), (16, 512, 256), (1, 256, 4096), (40, 256, 72), (129, 4096, 128), (128, 4096, 128), (200, 136, 64),
+     # up to 16 rows with K >= 1024: the streaming kernel with the gated panel (edges: I % 8, one feature)
+     (16, 12288, 4096), (5, 13, 1024), (9, 100, 2048), (16, 1, 1088), (2, 8, 12288)],
 )
 def test_fused_projection_equals_gemm_then_activation(native, shape):
     m, inter, k = shape
