@@ -38,6 +38,7 @@ GEMM_CONFIGS = {
     "128x128_deep": 13,
     "stream64": 14,
     "256x256_solo": 15,
+    "192x256": 16,
 }
 # OR-ed into a GEMM or LogP configuration: register-staged main loop (bit-neutral).
 FORCE_STAGED = 0x100
