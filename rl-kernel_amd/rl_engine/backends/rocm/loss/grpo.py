@@ -4,7 +4,10 @@ Mirrors, on the GPU, the log-prob form of the reference loss:
 ``compute_policy_ratio`` / ``compute_reference_kl`` / ``masked_mean``
 (rl_engine/reference/definitions.py:50-106) composed as in
 tests/e2e/test_rl_kernel_loss_step.py:18-39 and NativeGRPOLossOp.apply
-(rl_engine/reference/loss/grpo_loss.py:96-125). Forward only.
+(rl_engine/reference/loss/grpo_loss.py:96-125). The three scalars are differentiable
+with respect to the current log-probs, with the gradients torch's autograd gives the
+reference's formula (``torch.minimum`` / ``torch.clamp`` conventions), so the loss
+can sit on top of the differentiable fused linear-LogP in a training step.
 """
 
 from __future__ import annotations
@@ -26,6 +29,43 @@ class GrpoLossOutput(NamedTuple):
 
 def _as_2d(t: torch.Tensor) -> torch.Tensor:
     return t.reshape(1, -1) if t.dim() == 1 else t
+
+
+class _GrpoLossAutograd(torch.autograd.Function):
+    """Forward on the HIP kernel; backward elementwise on the saved per-token outputs.
+
+    With ``r = exp(logp - old)``, ``d = ref - logp``, ``n = max(active, 1e-8)``:
+    ``d policy_i / d logp_i = -A r_i`` where the unclipped branch is the minimum or ties it
+    (inside the clip range, or outside it on the side the clip does not bind), else 0;
+    ``d k3_i / d logp_i = 1 - exp(d_i)``; both times ``mask_i / n``.
+    """
+
+    @staticmethod
+    def forward(ctx, cur, old, ref, adv, mask, clip_eps, beta):
+        out3, ratio, k3 = _C.grpo_ratio_kl_loss(cur, old, ref, adv, mask, clip_eps, beta)
+        ctx.save_for_backward(cur, old, ref, adv, mask if mask is not None else torch.empty(0, device=cur.device))
+        ctx.has_mask = mask is not None
+        ctx.clip_eps, ctx.beta = float(clip_eps), float(beta)
+        ctx.mark_non_differentiable(ratio, k3)
+        return out3[0], out3[1], out3[2], ratio, k3
+
+    @staticmethod
+    def backward(ctx, g_loss, g_policy, g_kl, _g_ratio, _g_k3):
+        cur, old, ref, adv, mask = ctx.saved_tensors
+        keep = mask.to(torch.float32) if ctx.has_mask else torch.ones_like(cur)
+        count = torch.clamp(keep.sum(), min=1e-8)
+        a = adv.reshape(-1, 1)
+        r = torch.exp(cur - old)
+        lo, hi = 1.0 - ctx.clip_eps, 1.0 + ctx.clip_eps
+        flows = ((r >= lo) & (r <= hi)) | ((r > hi) & (a < 0)) | ((r < lo) & (a > 0))
+        d_policy = -(a * r) * flows.to(torch.float32)
+        d_kl = 1.0 - torch.exp(ref - cur)
+        zero = torch.zeros((), dtype=torch.float32, device=cur.device)
+        g_loss = zero if g_loss is None else g_loss
+        w_policy = g_loss + (zero if g_policy is None else g_policy)
+        w_kl = ctx.beta * g_loss + (zero if g_kl is None else g_kl)
+        grad = (w_policy * d_policy + w_kl * d_kl) * keep / count
+        return grad, None, None, None, None, None, None
 
 
 def grpo_ratio_kl_loss(
@@ -60,6 +100,11 @@ def grpo_ratio_kl_loss(
         mask = _as_2d(completion_mask)
         if mask.shape != cur.shape:
             raise ValueError("completion_mask must match the log-prob shape")
+    if torch.is_grad_enabled() and cur.requires_grad:
+        loss, policy, kl, ratio, k3 = _GrpoLossAutograd.apply(
+            cur, old.detach(), ref.detach(), adv.detach(), mask, float(clip_eps), float(beta)
+        )
+        return GrpoLossOutput(loss, policy, kl, ratio.reshape(shape), k3.reshape(shape))
     out3, ratio, k3 = _C.grpo_ratio_kl_loss(cur, old, ref, adv, mask, clip_eps, beta)
     return GrpoLossOutput(out3[0], out3[1], out3[2], ratio.reshape(shape), k3.reshape(shape))
 

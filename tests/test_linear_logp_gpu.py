@@ -317,6 +317,89 @@ def test_grpo_closed_forms(loss_mod):
     assert bool((loss_mod.compute_reference_kl(logp, logp + 0.01) >= 0).all())
 
 
+def _reference_rl_loss(logp, old, ref, adv, mask, eps, beta):
+    """The reference's minimal RL loss in torch (tests/e2e/test_rl_kernel_loss_step.py:18-39 on
+    rl_engine/reference/definitions.py:50-106): differentiable through torch's own autograd."""
+    keep = mask.to(logp.dtype)
+    ratio = torch.exp(logp - old) * keep
+    a = adv.reshape(-1, 1).to(logp.dtype)
+    policy = -torch.minimum(ratio * a, torch.clamp(ratio, 1.0 - eps, 1.0 + eps) * a)
+    d = (ref - logp) * keep
+    kl = (torch.exp(d) - d - 1.0) * keep
+    count = torch.clamp(keep.sum(), min=1e-8)
+    policy_loss, kl_mean = (policy * keep).sum() / count, kl.sum() / count
+    return policy_loss + beta * kl_mean, policy_loss, kl_mean
+
+
+def test_grpo_loss_gradients_match_torch_autograd(loss_mod):
+    g = torch.Generator().manual_seed(5300)
+    rollouts, tokens = 9, 70
+    base = -torch.randn((rollouts, tokens), generator=g).abs()
+    old = (base + 0.3 * torch.randn((rollouts, tokens), generator=g)).to(DEV)  # ratios on both sides of the clip range
+    ref = (base + 0.2 * torch.randn((rollouts, tokens), generator=g)).to(DEV)
+    adv = torch.randn(rollouts, generator=g).to(DEV)
+    adv[3] = 0.0
+    mask = (torch.rand((rollouts, tokens), generator=g) < 0.75).to(DEV)
+    for which, beta in ((0, 0.01), (0, 0.0), (1, 0.3), (2, 0.3)):
+        cur = base.to(DEV).clone().requires_grad_(True)
+        out = loss_mod.grpo_ratio_kl_loss(cur, old, ref, adv, mask, clip_eps=0.2, beta=beta)
+        assert out.loss.requires_grad and not out.ratio.requires_grad
+        (out.loss, out.policy_loss, out.kl)[which].backward()
+        cur64 = base.to(DEV).double().requires_grad_(True)
+        want = _reference_rl_loss(cur64, old.double(), ref.double(), adv.double(), mask, 0.2, beta)
+        want[which].backward()
+        assert float(out.loss.detach()) == pytest.approx(float(want[0].detach()), rel=1e-5, abs=1e-7)
+        assert (cur.grad.double() - cur64.grad).abs().max().item() <= 1e-6 * max(1.0, cur64.grad.abs().max().item())
+        assert bool((cur.grad[~mask] == 0).all())
+    # the forward values under autograd are the inference values, bit for bit
+    cur = base.to(DEV).clone().requires_grad_(True)
+    a = loss_mod.grpo_ratio_kl_loss(cur, old, ref, adv, mask, beta=0.01)
+    b = loss_mod.grpo_ratio_kl_loss(cur.detach(), old, ref, adv, mask, beta=0.01)
+    assert _same_bits(a.loss.detach().reshape(1), b.loss.reshape(1)) and _same_bits(a.k3, b.k3)
+
+
+def test_rl_loss_step_end_to_end(logp_mod, loss_mod):
+    """hidden, lm_head -> fused linear-LogP -> GRPO loss -> backward: the training step of
+    tests/e2e/test_rl_kernel_loss_step.py on this path, against fp64 autograd of the same formula."""
+    rollouts, tokens, hidden, vocab = 8, 40, 128, 3000
+    g = torch.Generator().manual_seed(5400)
+    h0 = inputs.randn_bf16(5401, rollouts * tokens, hidden).to(DEV)
+    w0 = inputs.randn_bf16(5402, vocab, hidden, 0.1).to(DEV)
+    target = torch.randint(0, vocab, (rollouts, tokens), generator=g).to(DEV)
+    mask = (torch.rand((rollouts, tokens), generator=g) < 0.75).to(DEV)
+    adv = torch.randn(rollouts, generator=g).to(DEV)
+    with torch.no_grad():
+        logp0, _ = logp_mod.deterministic_linear_logp(h0, w0, target.reshape(-1))
+    old = logp0.view(rollouts, tokens) + 0.15 * torch.randn((rollouts, tokens), generator=g).to(DEV)
+    ref = logp0.view(rollouts, tokens) + 0.15 * torch.randn((rollouts, tokens), generator=g).to(DEV)
+
+    h = h0.clone().requires_grad_(True)
+    w = w0.clone().requires_grad_(True)
+    logp, _ = logp_mod.deterministic_linear_logp(h.view(rollouts, tokens, hidden), w, target)
+    out = loss_mod.grpo_ratio_kl_loss(logp, old, ref, adv, mask, clip_eps=0.2, beta=0.01)
+    out.loss.backward()
+    assert torch.isfinite(out.loss) and h.grad.dtype == torch.bfloat16 and w.grad.shape == w.shape
+    assert bool((out.ratio[~mask] == 0).all()) and bool((out.k3[~mask] == 0).all())
+
+    h64 = h0.double().requires_grad_(True)
+    w64 = w0.double().requires_grad_(True)
+    logp64 = torch.log_softmax(h64 @ w64.t(), dim=-1).gather(1, target.reshape(-1, 1)).view(rollouts, tokens)
+    want = _reference_rl_loss(logp64, old.double(), ref.double(), adv.double(), mask, 0.2, 0.01)
+    want[0].backward()
+    assert float(out.loss.detach()) == pytest.approx(float(want[0].detach()), rel=1e-4, abs=1e-6)
+    for got, exact in ((h.grad, h64.grad), (w.grad, w64.grad)):
+        scale = exact.abs().max().item()
+        assert (got.double() - exact).abs().max().item() <= 2.0**-6 * scale  # d(logits) and the gradients are bf16
+    masked_rows = (~mask).reshape(-1)
+    assert bool((h.grad[masked_rows] == 0).all())  # masked tokens do not reach the hidden states
+
+    # masked positions do not affect the loss, whatever they hold (reference test, :94-131)
+    wild_old, wild_ref = old.clone(), ref.clone()
+    wild_old[~mask], wild_ref[~mask] = -1000.0, 500.0
+    again = loss_mod.grpo_ratio_kl_loss(logp.detach(), wild_old, wild_ref, adv, mask, clip_eps=0.2, beta=0.01)
+    assert _same_bits(again.loss.reshape(1), out.loss.detach().reshape(1))
+
+
 def test_config5_rollout_scale(logp_mod, loss_mod, oracle, config4):
     """64 rollouts x 1024 tokens through linear-LogP then the GRPO epilogue."""
     rollouts, per = 64, 1024
