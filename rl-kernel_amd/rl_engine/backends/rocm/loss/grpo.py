@@ -109,6 +109,57 @@ def grpo_ratio_kl_loss(
     return GrpoLossOutput(out3[0], out3[1], out3[2], ratio.reshape(shape), k3.reshape(shape))
 
 
+def group_advantages(
+    rewards: torch.Tensor,
+    *,
+    samples_per_prompt: Optional[int] = None,
+    group_boundaries=None,
+    eps: float = 1e-6,
+) -> torch.Tensor:
+    """Per-sequence rewards normalised inside each generation group:
+    ``(r - mean_g) / sqrt(max(E_g[r^2] - mean_g^2, eps^2))``, fp32, one value per sequence.
+
+    Same arguments, checks and messages as ``NativeGRPOLossOp.group_advantages``
+    (rl_engine/reference/loss/grpo_loss.py:53-84, 170-206). The group sums are plain
+    reductions over each group's slice (no atomics), so the result is the same from run to run.
+    """
+    flat = rewards.reshape(-1).float()
+    n = flat.numel()
+    if (samples_per_prompt is not None) + (group_boundaries is not None) != 1:
+        raise ValueError("Provide exactly one of samples_per_prompt or group_boundaries.")
+    if samples_per_prompt is not None:
+        if samples_per_prompt < 2:
+            raise ValueError("samples_per_prompt must be at least 2 for group normalization.")
+        if n % samples_per_prompt != 0:
+            raise ValueError(f"num_sequences ({n}) must be divisible by samples_per_prompt ({samples_per_prompt}).")
+        bounds = list(range(0, n + 1, int(samples_per_prompt)))
+    else:
+        b = torch.as_tensor(group_boundaries, dtype=torch.long).cpu()
+        if b.ndim != 1 or b.numel() < 2:
+            raise ValueError("group_boundaries must be a 1D tensor of length num_groups + 1.")
+        bounds = [int(v) for v in b.tolist()]
+        sizes = [hi - lo for lo, hi in zip(bounds[:-1], bounds[1:])]
+        if sum(sizes) != n:
+            raise ValueError(f"group sizes sum to {sum(sizes)} but there are {n} sequences.")
+        if any(size < 1 for size in sizes):
+            raise ValueError("each group must contain at least one sequence.")
+    out = torch.empty_like(flat)
+    uniform = len(bounds) > 1 and len({hi - lo for lo, hi in zip(bounds[:-1], bounds[1:])}) == 1 and bounds[0] == 0
+    groups = list(zip(bounds[:-1], bounds[1:]))
+    if uniform and n:
+        size = bounds[1] - bounds[0]
+        g = flat.view(-1, size)
+        mean = g.sum(dim=1, keepdim=True) / size
+        var = (g * g).sum(dim=1, keepdim=True) / size - mean * mean
+        return ((g - mean) / var.clamp_min(eps**2).sqrt()).reshape(-1)
+    for lo, hi in groups:
+        g = flat[lo:hi]
+        mean = g.sum() / (hi - lo)
+        var = (g * g).sum() / (hi - lo) - mean * mean
+        out[lo:hi] = (g - mean) / var.clamp_min(eps**2).sqrt()
+    return out
+
+
 def compute_policy_ratio(current_logps, old_logps, mask=None) -> torch.Tensor:
     """``exp(current - old)`` with masked entries set to zero."""
     zeros = torch.zeros(_as_2d(current_logps).size(0), dtype=torch.float32, device=current_logps.device)
@@ -121,4 +172,4 @@ def compute_reference_kl(current_logps, ref_logps, mask=None) -> torch.Tensor:
     return grpo_ratio_kl_loss(current_logps, current_logps, ref_logps, zeros, mask).k3
 
 
-__all__ = ["GrpoLossOutput", "compute_policy_ratio", "compute_reference_kl", "grpo_ratio_kl_loss"]
+__all__ = ["GrpoLossOutput", "compute_policy_ratio", "compute_reference_kl", "group_advantages", "grpo_ratio_kl_loss"]

@@ -240,3 +240,28 @@ def test_linear_logp_wrapper_contract_errors_without_a_gpu():
     with pytest.raises(TypeError, match="integer dtype"):
         LinearLogpWrapper._validate_targets(torch.tensor([0.0, 1.0]), rows=2, real_vocab_size=4)
     assert wrapper.provenance == {}
+
+
+def test_group_advantages_known_answers_and_errors():
+    """Host-side reward normalisation: the reference's own known answer and argument checks
+    (tests/ops/loss/test_grpo_loss.py:94-128), and equality with the oracle."""
+    from oracle import reference_math as oracle
+    from rl_engine.ops.loss import group_advantages
+
+    got = group_advantages(torch.tensor([1.0, 3.0, 10.0, 20.0, 30.0]), group_boundaries=[0, 2, 5])
+    g1 = (torch.tensor([10.0, 20.0, 30.0]) - 20.0) / (200.0 / 3.0) ** 0.5
+    assert torch.allclose(got, torch.cat([torch.tensor([-1.0, 1.0]), g1]), atol=1e-5)
+    rewards = torch.randn(12, generator=torch.Generator().manual_seed(61))
+    uniform = group_advantages(rewards.view(3, 4), samples_per_prompt=4)
+    assert uniform.shape == (12,) and uniform.dtype == torch.float32
+    assert torch.allclose(uniform, group_advantages(rewards, group_boundaries=[0, 4, 8, 12]), atol=1e-6)
+    assert torch.allclose(uniform, torch.from_numpy(oracle.group_advantages(rewards.numpy(), samples_per_prompt=4)), atol=1e-6)
+    ragged = group_advantages(rewards, group_boundaries=torch.tensor([0, 1, 5, 12]))
+    assert torch.allclose(ragged, torch.from_numpy(oracle.group_advantages(rewards.numpy(), group_boundaries=[0, 1, 5, 12])), atol=1e-5)
+    assert float(ragged[0]) == 0.0  # a group of one: zero variance is floored at eps, the numerator is zero
+    assert torch.equal(group_advantages(torch.full((4,), 2.5), samples_per_prompt=2), torch.zeros(4))
+    for kwargs in ({}, {"samples_per_prompt": 4, "group_boundaries": [0, 4, 8, 12]}, {"samples_per_prompt": 1},
+                   {"samples_per_prompt": 5}, {"group_boundaries": [0, 4, 8]}, {"group_boundaries": [0, 4, 4, 12]},
+                   {"group_boundaries": [12]}):  # fmt: skip
+        with pytest.raises(ValueError):
+            group_advantages(rewards, **kwargs)
