@@ -1,4 +1,5 @@
-"""Buffers of more than 2**31 elements, through the C ABI, on a real MI355X.
+"""Both ends of the size range, through the C ABI, on a real MI355X: buffers of more than
+2**31 elements, and empty inputs.
 
 The reference sizes its rollout case at 65536 tokens x 151936 vocabulary columns
 (9.96e9 logits); every kernel that walks a [rows, columns] buffer must index it
@@ -149,3 +150,31 @@ def test_linear_logp_backward_over_2g_elements(C):
         ref = dz.to(torch.bfloat16).double().t() @ h.double()
         scale = ref.abs().max().item()
         assert (gw[cols].double() - ref).abs().max().item() <= 2.0**-7 * scale
+
+
+def test_empty_inputs_through_every_entry(C):
+    """The other end of the size range: zero rows (and zero columns where the shape allows it)
+    return empty tensors of the right shape and dtype without a launch."""
+    from rl_engine.ops import logprob, loss
+
+    w = _randn((64, 128), 41, 0.1)
+    none = torch.empty((0, 128), dtype=torch.bfloat16, device=DEV)
+    no_ids = torch.empty((0,), dtype=torch.int64, device=DEV)
+    assert C.det_gemm_fwd_rhs_transposed(none, w).shape == (0, 64)
+    assert C.det_gemm_fwd_out_fp32(none, w.t()).dtype == torch.float32
+    tree = torch.empty((0, 64), dtype=torch.bfloat16, device=DEV)
+    assert C.gemm_tree_strided(none, w.t(), tree).shape == (0, 64)
+    logp, lse = C.fused_linear_logp(none, w, no_ids)
+    assert logp.shape == (0,) and lse.shape == (0,) and logp.dtype == torch.float32
+    logp, lse = logprob.deterministic_linear_logp(none.view(0, 3, 128), w, no_ids.view(0, 3))
+    assert logp.shape == (0, 3)
+    assert C.det_gemm_swiglu(none, w).shape == (0, 32)
+    assert C.swiglu_packed_forward(torch.empty((0, 64), dtype=torch.bfloat16, device=DEV)).shape == (0, 32)
+    logits = torch.empty((0, 64), dtype=torch.bfloat16, device=DEV)
+    a, b = C.hip_deterministic_logp_from_logits(logits, no_ids, 0, 64, 8)
+    assert a.shape == (0,) and b.shape == (0,)
+    stats = C.hip_deterministic_logp_tile_stats(logits, 0, 64, 8)
+    assert stats[0].shape == (0, 8)
+    out = loss.grpo_ratio_kl_loss(torch.empty((0, 5), device=DEV), torch.empty((0, 5), device=DEV),
+                                  torch.empty((0, 5), device=DEV), torch.empty((0,), device=DEV))
+    assert float(out.loss) == 0.0 and out.ratio.shape == (0, 5)
