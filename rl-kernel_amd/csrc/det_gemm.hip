@@ -51,7 +51,8 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
   if constexpr (LOOP == kLoopSolo) {
     tile_mainloop_solo<S>(W, X, n0, m0, K, lds, acc);
   } else if constexpr (LOOP >= kLoopPingPongKMajor) {
-    tile_mainloop_pingpong<S, loop_weight_kmajor(LOOP), loop_act_kmajor(LOOP)>(W, X, n0, m0, K, lds, acc);
+    tile_mainloop_pingpong<S, loop_weight_kmajor(LOOP), loop_act_kmajor(LOOP), PlainRowMap<S>, KS, NS>(W, X, n0, m0, K,
+                                                                                                        lds, acc);
   } else if constexpr (LOOP == kLoopPingPong) {
     tile_mainloop_pingpong<S, false, false, PlainRowMap<S>, KS, NS>(W, X, n0, m0, K, lds, acc);
   } else {
@@ -177,11 +178,20 @@ static hipError_t launch_tile(const MatView& W, const MatView& X, void* C, int64
   return hipGetLastError();
 }
 
-template <class S, int LOOP>
+template <class S, int LOOP, int NS = 2>
 static hipError_t launch_loop(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
                               bool out_f32, hipStream_t stream) {
-  return out_f32 ? launch_tile<S, LOOP, true>(W, X, C, ldc, M, N, K, stream)
-                 : launch_tile<S, LOOP, false>(W, X, C, ldc, M, N, K, stream);
+  return out_f32 ? launch_tile<S, LOOP, true, 1, NS>(W, X, C, ldc, M, N, K, stream)
+                 : launch_tile<S, LOOP, false, 1, NS>(W, X, C, ldc, M, N, K, stream);
+}
+
+// LDS stages of the native ping-pong loop: 256 x 128 and 256 x 64 run three (144 / 120 KiB). With
+// weights that come from HBM the extra K tile of lead is worth 8 % (gate_up at 256 tokens:
+// 73 -> 68 us); on cache-resident operands it changes nothing. The smaller shapes have their
+// deep-stage variants; the K-major loops measured no gain from a third stage and keep two.
+template <class S>
+constexpr int pingpong_stages() {
+  return (S::BN == 256 && S::BM <= 128) ? 3 : 2;
 }
 
 // kmajor_loop: 0, or the K-major ping-pong variant the operand layouts call for.
@@ -201,12 +211,7 @@ static hipError_t launch_shape(const MatView& W, const MatView& X, void* C, int6
   if (kmajor_loop != 0) return hipErrorInvalidValue;
   if constexpr (pingpong_supported<S>()) {
     if (vec && allow_pingpong && K % kTileK == 0) {
-      // 256 x 128 and 256 x 64 run three stages (144 / 120 KiB): with weights that come from HBM the
-      // extra K tile of lead is worth 8 % (gate_up at 256 tokens: 73 -> 68 us); on cache-resident
-      // operands it changes nothing. The smaller shapes have their deep-stage variants.
-      constexpr int kStages = (S::BN == 256 && S::BM <= 128) ? 3 : 2;
-      return out_f32 ? launch_tile<S, kLoopPingPong, true, 1, kStages>(W, X, C, ldc, M, N, K, stream)
-                     : launch_tile<S, kLoopPingPong, false, 1, kStages>(W, X, C, ldc, M, N, K, stream);
+      return launch_loop<S, kLoopPingPong, pingpong_stages<S>()>(W, X, C, ldc, M, N, K, out_f32, stream);
     }
   }
   if (vec) return launch_loop<S, kLoopStaged>(W, X, C, ldc, M, N, K, out_f32, stream);
@@ -323,10 +328,29 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
     // Only the shapes with 64-feature wave columns have the transposing loop, and a K-major
     // activation needs at least 128 tokens per tile.
     if (config == RLK_GEMM_CFG_AUTO) {
-      const int64_t t256 = tile_count(M, N, 256, 256), t128 = tile_count(M, N, 128, 256);
-      config = (M > 128 && t256 >= 256) ? RLK_GEMM_CFG_256x256
-               : (t128 >= 128 || M > 64 || x_kmajor) ? RLK_GEMM_CFG_256x128
-                                                     : RLK_GEMM_CFG_256x64;
+      // The same estimate as pick_det_gemm_config over the three shapes that have the loop: rounds of
+      // 256 workgroups (a partly filled one costs at least 0.9) x tile area / relative throughput. With
+      // few token tiles against a long reduction (grad_hidden of the LogP backward at 1024 tokens:
+      // N = 4096, K = 151936) the 64-token tile doubles the workgroups (2.15 -> 2.0 ms: every
+      // workgroup of a feature tile still streams the whole 78 MB weight panel).
+      struct Shape {
+        int config, bm;
+        double quality;
+      };
+      const Shape shapes[] = {{RLK_GEMM_CFG_256x256, 256, 1.00}, {RLK_GEMM_CFG_256x128, 128, 0.65},
+                              {RLK_GEMM_CFG_256x64, 64, 0.50}};
+      double best = 1e300;
+      for (const Shape& c : shapes) {
+        if (c.config == RLK_GEMM_CFG_256x64 && x_kmajor) continue;
+        const int64_t tiles = tile_count(M, N, c.bm, 256);
+        const int64_t full = tiles / 256;
+        const double part = (double)(tiles - full * 256) / 256.0;
+        const double t = ((double)full + (part > 0.0 ? (part > 0.9 ? part : 0.9) : 0.0)) * (256.0 * c.bm) / c.quality;
+        if (t < best * 0.999) {
+          best = t;
+          config = c.config;
+        }
+      }
     }
     switch (config) {
       case RLK_GEMM_CFG_256x256:
