@@ -10,13 +10,16 @@ H[4096,12288] x W[4096,12288]^T, inputs resident in HBM. The JSON line also carr
                      on the launch stream;
 * ``cpu_baseline`` - the CPU oracle (``oracle/reference_math.det_gemm_ref``) timed on
                      this box's host cores on the same step;
-* ``shapes``       - every token count of the configuration (T = 1, 16, 256, 4096)
-                     with its own MFMA or HBM fraction;
+* ``shapes``       - every token count of the configuration (T = 1, 16, 64, 256, 1024, 4096)
+                     with its own MFMA or HBM fraction; up to 1024 tokens also over copies of
+                     the weight that rotate through 1.3 GB, so that it is read from HBM and
+                     not from the 256 MB memory-side cache (``weights_from_hbm``);
 * ``linear_logp``  - the fused linear-LogP at T=8192, V=151936, D=4096 in tokens/s, with its
                      backward and the from-logits stage;
 * ``ffn``          - the gated FFN (fused gate/up + SwiGLU, then down) at T=4096.
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-logp]
+       python bench.py --only LEG [--rotate-weights]   (one leg, for profiling; see --help)
 """
 
 from __future__ import annotations
