@@ -177,6 +177,27 @@ int rlk_linear_logp_fwd(const void* hidden, int64_t h_row_stride, const void* we
                         float* lse, void* workspace, size_t workspace_bytes, int T, int D, int V,
                         int64_t vocab_start, int real_vocab_end, int config, void* stream);
 
+/*
+ * The same pass for one shard of a vocabulary split over ranks: `weight` holds rows
+ * [vocab_start, vocab_start + V) of the lm_head, `target` stays in global ids, and the
+ * outputs are the two terms a caller merges across shards,
+ *   target_logit [T] fp32 out (may be NULL): the scaled logit y_target (bias and
+ *                temperature applied, not clamped) when this shard owns the target, else 0
+ *   lse          [T] fp32 out (may be NULL): log-sum-exp over this shard's real columns
+ * so that logp = sum_shards(target_logit) - log(sum_shards(exp(lse))). With one shard,
+ * min(target_logit - lse, 0) is bit-for-bit rlk_linear_logp_fwd's logp. Workspace, configs,
+ * order of summation and errors are those of rlk_linear_logp_fwd.
+ *
+ * Stands in for rl_engine._C.fused_linear_logp_sm90_global_target
+ * (csrc/bindings/ops.cpp:522-526; csrc/cuda/logprob/fused_linear_logp_sm90.cu:2169-2176),
+ * whose caller merges the pair in _merge_tp_local_logp
+ * (rl_engine/backends/cuda/logprob/linear_logp.py:711-740).
+ */
+int rlk_linear_logp_fwd_shard(const void* hidden, int64_t h_row_stride, const void* weight, int64_t w_row_stride,
+                              const int64_t* target, const float* bias, const float* temperature,
+                              float* target_logit, float* lse, void* workspace, size_t workspace_bytes, int T,
+                              int D, int V, int64_t vocab_start, int real_vocab_end, int config, void* stream);
+
 /* Bytes of workspace rlk_linear_logp_bwd needs: the bf16 d(logits) [T, V rounded up to 64]
  * plus, when a bias gradient is wanted, fp32 block sums [ceil(T / 256), V]. */
 size_t rlk_linear_logp_bwd_workspace_bytes(int T, int V, int with_bias);

@@ -265,7 +265,8 @@ constexpr int kMergeThreads = kMergeTokens * kMergeLanes;  // 256
 
 __global__ __launch_bounds__(kMergeThreads) void linear_logp_merge_kernel(const float* __restrict__ part,
                                                                           float* __restrict__ logp,
-                                                                          float* __restrict__ lse, int T,
+                                                                          float* __restrict__ lse,
+                                                                          float* __restrict__ target_logit, int T,
                                                                           int n_split, bool clamp) {
   __shared__ float red[kMergeLanes][kMergeTokens];
   __shared__ float terms[kMergeChunk][kMergeTokens];
@@ -320,13 +321,14 @@ __global__ __launch_bounds__(kMergeThreads) void linear_logp_merge_kernel(const 
     const float l = big + logf(sum);
     if (lse) lse[m] = l;
     if (logp) logp[m] = clamp ? fminf(zt - l, 0.f) : zt - l;
+    if (target_logit) target_logit[m] = zt;
   }
 }
 
-hipError_t linear_logp_merge_launch(const float* part, float* logp, float* lse, int T, int n_split, bool clamp,
-                                    hipStream_t stream) {
+hipError_t linear_logp_merge_launch(const float* part, float* logp, float* lse, float* target_logit, int T,
+                                    int n_split, bool clamp, hipStream_t stream) {
   hipLaunchKernelGGL(linear_logp_merge_kernel, dim3((T + kMergeTokens - 1) / kMergeTokens), dim3(kMergeThreads), 0,
-                     stream, part, logp, lse, T, n_split, clamp);
+                     stream, part, logp, lse, target_logit, T, n_split, clamp);
   return hipGetLastError();
 }
 
@@ -422,8 +424,9 @@ int pick_linear_logp_config(int T, int V) {
 }
 
 hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t* target, const float* bias,
-                              const float* temperature, float* logp, float* lse, float* workspace, int T, int D,
-                              int V, int64_t vocab_start, int vocab_limit, int config, hipStream_t stream) {
+                              const float* temperature, float* logp, float* lse, float* target_logit,
+                              float* workspace, int T, int D, int V, int64_t vocab_start, int vocab_limit, int config,
+                              hipStream_t stream) {
   LogpArgs a;
   a.W = W;
   a.H = H;
@@ -485,7 +488,7 @@ hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t*
       return hipErrorInvalidValue;
   }
   if (err != hipSuccess) return err;
-  return linear_logp_merge_launch(workspace, logp, lse, T, a.n_split, true, stream);
+  return linear_logp_merge_launch(workspace, logp, lse, target_logit, T, a.n_split, true, stream);
 }
 
 }  // namespace rlk

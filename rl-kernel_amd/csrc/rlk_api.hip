@@ -136,42 +136,61 @@ size_t rlk_linear_logp_workspace_bytes(int T, int V) {
   return linear_logp_workspace_bytes(T, V);
 }
 
-int rlk_linear_logp_fwd(const void* hidden, int64_t h_row_stride, const void* weight, int64_t w_row_stride,
-                        const int64_t* target, const float* bias, const float* temperature, float* logp,
-                        float* lse, void* workspace, size_t workspace_bytes, int T, int D, int V,
-                        int64_t vocab_start, int real_vocab_end, int config, void* stream) {
+static int linear_logp_fwd_checked(const char* who, const void* hidden, int64_t h_row_stride, const void* weight,
+                                   int64_t w_row_stride, const int64_t* target, const float* bias,
+                                   const float* temperature, float* logp, float* lse, float* target_logit,
+                                   void* workspace, size_t workspace_bytes, int T, int D, int V, int64_t vocab_start,
+                                   int real_vocab_end, int config, void* stream) {
   if (T < 0 || D <= 0 || V <= 0) {
-    set_last_error("rlk_linear_logp_fwd: bad sizes T=%d D=%d V=%d", T, D, V);
+    set_last_error("%s: bad sizes T=%d D=%d V=%d", who, T, D, V);
     return RLK_ERR_INVALID_ARGUMENT;
   }
   if (real_vocab_end <= 0 || real_vocab_end > V) {
-    set_last_error("rlk_linear_logp_fwd: real_vocab_end must be in [1, %d], got %d", V, real_vocab_end);
+    set_last_error("%s: real_vocab_end must be in [1, %d], got %d", who, V, real_vocab_end);
     return RLK_ERR_INVALID_ARGUMENT;
   }
   if (config < 0 || (config & ~RLK_LOGP_CFG_FORCE_STAGED) >= RLK_LOGP_CFG_COUNT) {
-    set_last_error("rlk_linear_logp_fwd: unknown config %d", config);
+    set_last_error("%s: unknown config %d", who, config);
     return RLK_ERR_INVALID_ARGUMENT;
   }
   if (T == 0) return RLK_OK;
   if (hidden == nullptr || weight == nullptr || target == nullptr) {
-    set_last_error("rlk_linear_logp_fwd: null hidden / weight / target");
+    set_last_error("%s: null hidden / weight / target", who);
     return RLK_ERR_INVALID_ARGUMENT;
   }
   if (h_row_stride < D || w_row_stride < D) {
-    set_last_error("rlk_linear_logp_fwd: row strides must be >= D");
+    set_last_error("%s: row strides must be >= D", who);
     return RLK_ERR_INVALID_ARGUMENT;
   }
   const size_t need = linear_logp_workspace_bytes(T, V);
   if (workspace == nullptr || workspace_bytes < need) {
-    set_last_error("rlk_linear_logp_fwd: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    set_last_error("%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
     return RLK_ERR_INVALID_ARGUMENT;
   }
   MatView H{reinterpret_cast<const bf16_bits*>(hidden), h_row_stride, 1, T};
   MatView W{reinterpret_cast<const bf16_bits*>(weight), w_row_stride, 1, V};
-  hipError_t err = linear_logp_launch(H, W, target, bias, temperature, logp, lse, reinterpret_cast<float*>(workspace),
-                                      T, D, V, vocab_start, real_vocab_end, config,
-                                      reinterpret_cast<hipStream_t>(stream));
-  return err == hipSuccess ? RLK_OK : device_error("rlk_linear_logp_fwd", err);
+  hipError_t err = linear_logp_launch(H, W, target, bias, temperature, logp, lse, target_logit,
+                                      reinterpret_cast<float*>(workspace), T, D, V, vocab_start, real_vocab_end,
+                                      config, reinterpret_cast<hipStream_t>(stream));
+  return err == hipSuccess ? RLK_OK : device_error(who, err);
+}
+
+int rlk_linear_logp_fwd(const void* hidden, int64_t h_row_stride, const void* weight, int64_t w_row_stride,
+                        const int64_t* target, const float* bias, const float* temperature, float* logp,
+                        float* lse, void* workspace, size_t workspace_bytes, int T, int D, int V,
+                        int64_t vocab_start, int real_vocab_end, int config, void* stream) {
+  return linear_logp_fwd_checked("rlk_linear_logp_fwd", hidden, h_row_stride, weight, w_row_stride, target, bias,
+                                 temperature, logp, lse, nullptr, workspace, workspace_bytes, T, D, V, vocab_start,
+                                 real_vocab_end, config, stream);
+}
+
+int rlk_linear_logp_fwd_shard(const void* hidden, int64_t h_row_stride, const void* weight, int64_t w_row_stride,
+                              const int64_t* target, const float* bias, const float* temperature,
+                              float* target_logit, float* lse, void* workspace, size_t workspace_bytes, int T,
+                              int D, int V, int64_t vocab_start, int real_vocab_end, int config, void* stream) {
+  return linear_logp_fwd_checked("rlk_linear_logp_fwd_shard", hidden, h_row_stride, weight, w_row_stride, target,
+                                 bias, temperature, nullptr, lse, target_logit, workspace, workspace_bytes, T, D, V,
+                                 vocab_start, real_vocab_end, config, stream);
 }
 
 size_t rlk_linear_logp_bwd_workspace_bytes(int T, int V, int with_bias) {
@@ -304,7 +323,7 @@ int rlk_logp_from_logits(const void* logits, int dtype, int64_t row_stride, cons
   const int64_t plane = (int64_t)num_tiles * T;
   hipError_t err = logits_tile_stats_launch(logits, dtype, row_stride, target, temperature, T, V, vocab_start,
                                             real_vocab, num_tiles, part, part + plane, part + 2 * plane, 1, T, s);
-  if (err == hipSuccess) err = linear_logp_merge_launch(part, logp, lse, T, num_tiles, false, s);
+  if (err == hipSuccess) err = linear_logp_merge_launch(part, logp, lse, nullptr, T, num_tiles, false, s);
   return err == hipSuccess ? RLK_OK : device_error("rlk_logp_from_logits", err);
 }
 

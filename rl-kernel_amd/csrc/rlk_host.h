@@ -60,15 +60,18 @@ int linear_logp_split_count(int V);
 size_t linear_logp_workspace_bytes(int T, int V);
 
 // H[T,D] hidden states, W[V,D] lm_head weight; workspace holds
-// linear_logp_workspace_bytes(T, V) bytes of fp32 partials.
+// linear_logp_workspace_bytes(T, V) bytes of fp32 partials. logp, lse and target_logit
+// (the unclamped scaled logit of a target this weight owns, else 0) may each be null.
 hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t* target, const float* bias,
-                              const float* temperature, float* logp, float* lse, float* workspace, int T, int D,
-                              int V, int64_t vocab_start, int vocab_limit, int config, hipStream_t stream);
+                              const float* temperature, float* logp, float* lse, float* target_logit,
+                              float* workspace, int T, int D, int V, int64_t vocab_start, int vocab_limit, int config,
+                              hipStream_t stream);
 
 // Ascending merge of (max, sum, target logit) partials laid out [3][n_split][T] into
-// lse = M + log(S) and logp = target - lse (clamped at 0 when `clamp`).
-hipError_t linear_logp_merge_launch(const float* part, float* logp, float* lse, int T, int n_split, bool clamp,
-                                    hipStream_t stream);
+// lse = M + log(S), logp = target - lse (clamped at 0 when `clamp`) and the merged target
+// logit itself (0 for a target no partial owns); each output may be null.
+hipError_t linear_logp_merge_launch(const float* part, float* logp, float* lse, float* target_logit, int T,
+                                    int n_split, bool clamp, hipStream_t stream);
 
 // Per-row, per-tile (max, sum of exp relative to it[, target logit]) of materialised logits
 // of element type `dtype` (rlk_dtype); element (row, tile) of each output sits at

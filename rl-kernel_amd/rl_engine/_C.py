@@ -223,6 +223,82 @@ def linear_logp_split_count(vocab: int) -> int:
     return int(_lib.load().rlk_linear_logp_split_count(int(vocab)))
 
 
+def _linear_logp_forward(
+    who: str,
+    entry: str,
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    target: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    temperature: Optional[torch.Tensor],
+    real_vocab_size: int,
+    vocab_start_index: int,
+    config: int,
+):
+    """Checks shared by the fused linear-LogP entries, then one call of ``entry`` in the C ABI.
+
+    Returns ``(first, lse, bias_f32, real_vocab)``; ``first`` is logp or the target
+    logit, whichever ``entry`` writes."""
+    if not hidden.is_cuda or not weight.is_cuda or not target.is_cuda:
+        raise RuntimeError(f"{who}: hidden, weight and target must be CUDA tensors")
+    if hidden.dtype != _BF16 or weight.dtype != _BF16:
+        raise RuntimeError(f"{who}: hidden and weight must be bf16")
+    if hidden.dim() != 2 or weight.dim() != 2:
+        raise RuntimeError(f"{who}: expect hidden [N,D] and weight [V,D]")
+    if not hidden.is_contiguous() or not weight.is_contiguous():
+        raise RuntimeError(f"{who}: hidden and weight must be contiguous")
+    n, d = hidden.shape
+    v = weight.size(0)
+    if weight.size(1) != d:
+        raise RuntimeError(f"{who}: hidden dim must match weight dim")
+    if target.numel() != n:
+        raise RuntimeError(f"{who}: target must have one id per row")
+    real_vocab = v if int(real_vocab_size) < 0 else int(real_vocab_size)
+    if not 0 < real_vocab <= v:
+        raise RuntimeError(f"{who}: real_vocab_size must be in [1, {v}]")
+    target_i64 = target.reshape(-1).to(torch.int64).contiguous()
+    bias_f32 = None
+    if bias is not None:
+        if bias.numel() != v:
+            raise RuntimeError(f"{who}: bias must have V elements")
+        bias_f32 = bias.to(device=hidden.device, dtype=torch.float32).contiguous()
+    temp_f32 = None
+    if temperature is not None:
+        if temperature.dtype != torch.float32 or temperature.numel() != n:
+            raise RuntimeError(f"{who}: temperature must be fp32 with one value per row")
+        temp_f32 = temperature.to(hidden.device).contiguous()
+
+    lib = _lib.load()
+    first = torch.empty((n,), dtype=torch.float32, device=hidden.device)
+    lse = torch.empty((n,), dtype=torch.float32, device=hidden.device)
+    ws_bytes = int(lib.rlk_linear_logp_workspace_bytes(n, v))
+    workspace = torch.empty((max(ws_bytes, 4) // 4,), dtype=torch.float32, device=hidden.device)
+    if n > 0:
+        with torch.cuda.device(hidden.device):
+            status = getattr(lib, entry)(
+                hidden.data_ptr(),
+                hidden.stride(0),
+                weight.data_ptr(),
+                weight.stride(0),
+                target_i64.data_ptr(),
+                bias_f32.data_ptr() if bias_f32 is not None else None,
+                temp_f32.data_ptr() if temp_f32 is not None else None,
+                first.data_ptr(),
+                lse.data_ptr(),
+                workspace.data_ptr(),
+                ws_bytes,
+                n,
+                d,
+                v,
+                int(vocab_start_index),
+                real_vocab,
+                config,
+                _stream_handle(hidden.device),
+            )
+        _lib.check(status, f"{entry} failed")
+    return first, lse, bias_f32, real_vocab
+
+
 def fused_linear_logp(
     hidden: torch.Tensor,
     weight: torch.Tensor,
@@ -243,65 +319,13 @@ def fused_linear_logp(
     applied, padded lanes -inf) computed by the same MFMA chain through
     rlk_det_gemm_bf16 with fp32 output; it does not change logp / lse.
     """
-    if not hidden.is_cuda or not weight.is_cuda or not target.is_cuda:
-        raise RuntimeError("fused_linear_logp: hidden, weight and target must be CUDA tensors")
-    if hidden.dtype != _BF16 or weight.dtype != _BF16:
-        raise RuntimeError("fused_linear_logp: hidden and weight must be bf16")
-    if hidden.dim() != 2 or weight.dim() != 2:
-        raise RuntimeError("fused_linear_logp: expect hidden [N,D] and weight [V,D]")
-    if not hidden.is_contiguous() or not weight.is_contiguous():
-        raise RuntimeError("fused_linear_logp: hidden and weight must be contiguous")
-    n, d = hidden.shape
-    v = weight.size(0)
-    if weight.size(1) != d:
-        raise RuntimeError("fused_linear_logp: hidden dim must match weight dim")
-    if target.numel() != n:
-        raise RuntimeError("fused_linear_logp: target must have one id per row")
-    real_vocab = v if int(real_vocab_size) < 0 else int(real_vocab_size)
-    if not 0 < real_vocab <= v:
-        raise RuntimeError(f"fused_linear_logp: real_vocab_size must be in [1, {v}]")
-    target_i64 = target.reshape(-1).to(torch.int64).contiguous()
-    bias_f32 = None
-    if bias is not None:
-        if bias.numel() != v:
-            raise RuntimeError("fused_linear_logp: bias must have V elements")
-        bias_f32 = bias.to(device=hidden.device, dtype=torch.float32).contiguous()
-    temp_f32 = None
-    if temperature is not None:
-        if temperature.dtype != torch.float32 or temperature.numel() != n:
-            raise RuntimeError("fused_linear_logp: temperature must be fp32 with one value per row")
-        temp_f32 = temperature.to(hidden.device).contiguous()
-
-    lib = _lib.load()
-    logp = torch.empty((n,), dtype=torch.float32, device=hidden.device)
-    lse = torch.empty((n,), dtype=torch.float32, device=hidden.device)
-    ws_bytes = int(lib.rlk_linear_logp_workspace_bytes(n, v))
-    workspace = torch.empty((max(ws_bytes, 4) // 4,), dtype=torch.float32, device=hidden.device)
-    if n > 0:
-        with torch.cuda.device(hidden.device):
-            status = lib.rlk_linear_logp_fwd(
-                hidden.data_ptr(),
-                hidden.stride(0),
-                weight.data_ptr(),
-                weight.stride(0),
-                target_i64.data_ptr(),
-                bias_f32.data_ptr() if bias_f32 is not None else None,
-                temp_f32.data_ptr() if temp_f32 is not None else None,
-                logp.data_ptr(),
-                lse.data_ptr(),
-                workspace.data_ptr(),
-                ws_bytes,
-                n,
-                d,
-                v,
-                int(vocab_start_index),
-                real_vocab,
-                config,
-                _stream_handle(hidden.device),
-            )
-        _lib.check(status, "rlk_linear_logp_fwd failed")
+    logp, lse, bias_f32, real_vocab = _linear_logp_forward(
+        "fused_linear_logp", "rlk_linear_logp_fwd", hidden, weight, target, bias, temperature,
+        real_vocab_size, vocab_start_index, config,
+    )  # fmt: skip
     outputs = [logp, lse]
     if return_logits:
+        n, v = hidden.size(0), weight.size(0)
         logits = torch.empty((n, v), dtype=torch.float32, device=hidden.device)
         gemm_strided(hidden, weight.t(), logits)
         if bias_f32 is not None:
@@ -310,6 +334,37 @@ def fused_linear_logp(
             logits[:, real_vocab:] = float("-inf")
         outputs.append(logits)
     return outputs
+
+
+# The name the reference's CUDA build binds the same function under (csrc/bindings/ops.cpp:514).
+fused_linear_logp_sm90 = fused_linear_logp
+
+
+def fused_linear_logp_sm90_global_target(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    target: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    vocab_start_index: int = 0,
+    temperature: Optional[torch.Tensor] = None,
+    real_vocab_size: int = -1,
+    *,
+    config: int = 0,
+) -> List[torch.Tensor]:
+    """One vocabulary shard's ``[target_logit, lse]`` for targets given in global ids.
+
+    ``weight`` holds lm_head rows ``[vocab_start_index, vocab_start_index + V)``.
+    ``target_logit`` is the scaled, unclamped logit of a target this shard owns and 0
+    otherwise; ``lse`` covers the shard's real columns. The caller merges both across
+    shards (_merge_tp_local_logp, rl_engine/backends/cuda/logprob/linear_logp.py:711-740).
+    Argument order and return convention of ``_C.fused_linear_logp_sm90_global_target``
+    (csrc/bindings/ops.cpp:522-526; csrc/cuda/logprob/fused_linear_logp_sm90.cu:2169-2176).
+    """
+    target_logit, lse, _, _ = _linear_logp_forward(
+        "fused_linear_logp_sm90_global_target", "rlk_linear_logp_fwd_shard", hidden, weight, target, bias,
+        temperature, real_vocab_size, vocab_start_index, config,
+    )  # fmt: skip
+    return [target_logit, lse]
 
 
 def fused_linear_logp_bwd(
@@ -420,6 +475,41 @@ def fused_linear_logp_bwd(
         )
     _lib.check(status, "rlk_linear_logp_bwd failed")
     return [grad_hidden, grad_weight, grad_bias]
+
+
+def fused_linear_logp_sm90_backward(
+    grad_logp: torch.Tensor,
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    target: torch.Tensor,
+    lse: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    vocab_start_index: int,
+    compute_grad_hidden: bool,
+    compute_grad_weight: bool,
+    compute_grad_bias: bool,
+    use_global_lse: bool,
+) -> List[torch.Tensor]:
+    """:func:`fused_linear_logp_bwd` under the reference's CUDA name and argument order
+    (csrc/bindings/ops.cpp:33-43, 527-528): ``[grad_hidden, grad_weight, grad_bias]`` with an
+    empty fp32 tensor in place of a gradient that was not asked for
+    (csrc/cuda/logprob/fused_linear_logp_sm90.cu:2185-2215, 2307).
+
+    ``target`` is in global ids and ``lse`` is the value to differentiate against: the
+    shard-merged one when ``use_global_lse``, else this weight's own. The reference
+    recomputes the latter from its backward logits; here the forward's ``lse`` is already
+    the value of the same MFMA chain, so it is used as given in both cases.
+    """
+    del use_global_lse
+    if grad_logp.numel() != hidden.size(0):
+        raise RuntimeError("fused_linear_logp_sm90_backward: grad_logp must have one value per token")
+    grads = fused_linear_logp_bwd(
+        hidden, weight, target, lse, grad_logp.reshape(-1), None, bias,
+        vocab_start_index=int(vocab_start_index), need_grad_hidden=bool(compute_grad_hidden),
+        need_grad_weight=bool(compute_grad_weight), need_grad_bias=bool(compute_grad_bias),
+    )  # fmt: skip
+    empty = torch.empty((0,), dtype=torch.float32, device=hidden.device)
+    return [empty if g is None else g for g in grads]
 
 
 def _logits_dtype_code(logits: torch.Tensor) -> int:

@@ -59,6 +59,7 @@ EXPORTED_SYMBOLS = (
     "rlk_linear_logp_split_count",
     "rlk_linear_logp_workspace_bytes",
     "rlk_linear_logp_fwd",
+    "rlk_linear_logp_fwd_shard",
     "rlk_linear_logp_bwd_workspace_bytes",
     "rlk_linear_logp_bwd",
     "rlk_logits_tile_stats",
@@ -125,6 +126,8 @@ def load() -> ctypes.CDLL:
     lib.rlk_linear_logp_workspace_bytes.argtypes = [i32, i32]
     lib.rlk_linear_logp_fwd.restype = i32
     lib.rlk_linear_logp_fwd.argtypes = [vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, sz, i32, i32, i32, i64, i32, i32, vp]
+    lib.rlk_linear_logp_fwd_shard.restype = i32
+    lib.rlk_linear_logp_fwd_shard.argtypes = lib.rlk_linear_logp_fwd.argtypes
 
     lib.rlk_linear_logp_bwd_workspace_bytes.restype = sz
     lib.rlk_linear_logp_bwd_workspace_bytes.argtypes = [i32, i32, i32]

@@ -24,7 +24,7 @@ def _declared_functions() -> list[str]:
 
 def test_header_declares_the_expected_entry_points():
     names = _declared_functions()
-    for required in ("rlk_det_gemm_bf16", "rlk_linear_logp_fwd", "rlk_grpo_ratio_kl_loss", "rlk_contract_id"):
+    for required in ("rlk_det_gemm_bf16", "rlk_linear_logp_fwd", "rlk_linear_logp_fwd_shard", "rlk_grpo_ratio_kl_loss", "rlk_contract_id"):
         assert required in names
 
 
@@ -153,7 +153,13 @@ def test_ops_gemm_exports_the_reference_names():
 def test_native_module_has_the_reference_function_names():
     from rl_engine import _C
 
-    for name in ("det_gemm_sm90_compiled", "det_gemm_fwd", "det_gemm_fwd_rhs_transposed", "det_gemm_da", "det_gemm_db", "det_gemm_db_transposed", "fused_linear_logp"):
+    names = (
+        "det_gemm_sm90_compiled", "det_gemm_fwd", "det_gemm_fwd_rhs_transposed", "det_gemm_da", "det_gemm_db",
+        "det_gemm_db_transposed", "fused_linear_logp", "fused_linear_logp_sm90", "fused_linear_logp_sm90_global_target",
+        "fused_linear_logp_sm90_backward", "hip_deterministic_logp_tile_stats", "hip_deterministic_logp_backward",
+        "swiglu_forward", "swiglu_backward", "swiglu_packed_forward", "swiglu_packed_backward",
+    )  # fmt: skip
+    for name in names:
         assert callable(getattr(_C, name))
     assert _C.det_gemm_sm90_compiled() is False
 

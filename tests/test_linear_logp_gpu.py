@@ -212,6 +212,74 @@ def test_vocab_start_index_offsets_targets(logp_mod):
     assert _same_bits(base, shifted)
 
 
+@pytest.mark.parametrize("tokens", [5, 300, 1500])
+def test_shard_entry_returns_the_terms_a_vocabulary_split_merges(tokens):
+    """``fused_linear_logp_sm90_global_target`` against the whole-vocabulary entry and the dense
+    formula: one shard reproduces logp bit for bit; three uneven shards (the last one padded,
+    with bias and per-token temperature) merge to the whole vocabulary's logp within 1e-3 nats,
+    and each target logit is owned by exactly one shard."""
+    from rl_engine import _C
+
+    vocab, hidden = 5000, 192
+    h, w, target = inputs.logp_inputs(tokens, vocab=vocab, hidden=hidden, seed=4700 + tokens, rms_norm=False)
+    g = torch.Generator().manual_seed(4701)
+    bias = torch.randn((vocab,), generator=g) * 0.5
+    temp = torch.rand((tokens,), generator=g) + 0.5
+    h_d, w_d, t_d, b_d, temp_d = (x.to(DEV) for x in (h, w, target, bias, temp))
+
+    logp, lse = _C.fused_linear_logp_sm90(h_d, w_d, t_d, b_d, temp_d)
+    zt, lse1 = _C.fused_linear_logp_sm90_global_target(h_d, w_d, t_d, b_d, 0, temp_d)
+    assert _same_bits(lse, lse1)
+    assert _same_bits(logp, torch.clamp(zt - lse1, max=0.0))
+    dense = (h.double() @ w.double().t() + bias.double()) / temp.double()[:, None]
+    want_zt = dense.gather(1, target[:, None])[:, 0]
+    assert (zt.cpu().double() - want_zt).abs().max().item() <= 2e-3 * max(1.0, want_zt.abs().max().item())
+
+    bounds = [0, 1111, 3200, vocab]
+    zts, lses = [], []
+    for lo, hi in zip(bounds[:-1], bounds[1:]):
+        rows = w_d[lo:hi]
+        shard_bias = b_d[lo:hi]
+        real = hi - lo
+        if hi == vocab:  # the last shard carries 40 rows of padding that must not count
+            rows = torch.cat([rows, torch.full((40, hidden), 3.0, dtype=torch.bfloat16, device=DEV)])
+            shard_bias = torch.cat([shard_bias, torch.full((40,), 9.0, device=DEV)])
+        a, b = _C.fused_linear_logp_sm90_global_target(h_d, rows.contiguous(), t_d, shard_bias, lo, temp_d, real)
+        zts.append(a)
+        lses.append(b)
+        owned = (target >= lo) & (target < hi)
+        assert torch.equal(a.cpu() != 0, owned & (want_zt != 0).cpu())
+    owners = torch.stack([z != 0 for z in zts]).sum(0)
+    assert int(owners.max()) <= 1
+    merged = torch.stack(zts).double().sum(0) - torch.logsumexp(torch.stack(lses).double(), dim=0)
+    want = torch.log_softmax(dense, dim=-1).gather(1, target[:, None])[:, 0]
+    assert (merged.cpu() - want).abs().max().item() <= TOL_NATS
+    assert (logp.cpu().double() - want).abs().max().item() <= TOL_NATS
+
+
+def test_backward_under_the_reference_name_and_argument_order():
+    from rl_engine import _C
+
+    h, w, target = inputs.logp_inputs(70, vocab=1300, hidden=128, seed=4800, rms_norm=False)
+    h_d, w_d, t_d = h.to(DEV), w.to(DEV), target.to(DEV)
+    grad = torch.randn((70,), generator=torch.Generator().manual_seed(4801)).to(DEV)
+    _, lse = _C.fused_linear_logp_sm90(h_d, w_d, t_d)
+    gh, gw, gb = _C.fused_linear_logp_sm90_backward(grad, h_d, w_d, t_d, lse, None, 0, True, True, False, False)
+    ours = _C.fused_linear_logp_bwd(h_d, w_d, t_d, lse, grad, None)
+    assert torch.equal(gh, ours[0]) and torch.equal(gw, ours[1])
+    assert gb.numel() == 0 and gb.dtype == torch.float32
+    only_w = _C.fused_linear_logp_sm90_backward(grad, h_d, w_d, t_d, lse, None, 0, False, True, False, False)
+    assert only_w[0].numel() == 0 and torch.equal(only_w[1], gw)
+    # a shard's backward takes global ids and the shard's first row
+    lo = 400
+    half = _C.fused_linear_logp_sm90_backward(grad, h_d, w_d[lo:].contiguous(), t_d, lse, None, lo, False, True, False, True)
+    zf = h.double() @ w.double().t()
+    dz = -torch.exp(zf - lse.cpu().double()[:, None]) * grad.cpu().double()[:, None]
+    dz[torch.arange(70), target] += grad.cpu().double()
+    ref = dz[:, lo:].to(torch.bfloat16).double().t() @ h.double()
+    assert (half[1].cpu().double() - ref).abs().max().item() <= 2.0**-7 * ref.abs().max().item()
+
+
 # ---------------------------------------------------------------------------
 # Config 4 at full size: T=8192, V=151936, D=4096
 # ---------------------------------------------------------------------------
