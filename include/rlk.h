@@ -102,7 +102,8 @@ int rlk_det_gemm_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stride, c
  * Rounding points depend on K only: rows are batch invariant, and a K range that is a subtree
  * (the contiguous half, quarter, ... of a K-sharded rank) evaluates to exactly that node.
  * Strides as in rlk_det_gemm_bf16; any non-negative strides are accepted (no fast layout:
- * this is a vector-ALU kernel, about 20 times slower than the MFMA contract). bf16 output only.
+ * a leaf is a chain of single fp32 multiply-adds, which runs on the fp32 matrix pipe one k at a
+ * time or on the vector ALU, about ten times slower than the bf16 MFMA contract). bf16 output only.
  *
  * Stands in for the reference's "triton_tree" backend: _triton_tree_gemm and its tree plan
  * (rl_engine/backends/shared/triton/gemm/det_gemm.py:218-258, 355-417, 514-546), the CUDA
@@ -112,6 +113,20 @@ int rlk_det_gemm_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stride, c
 int rlk_det_gemm_tree_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stride, const void* b,
                            int64_t b_k_stride, int64_t b_n_stride, void* c, int64_t ldc, int M, int N, int K,
                            void* stream);
+
+/* Leaf loops of the k-tree kernel. Both compute every bit of the contract; exposed so tests can
+ * prove that. No counterpart in the reference. */
+typedef enum rlk_tree_config {
+  RLK_TREE_CFG_AUTO = 0,
+  RLK_TREE_CFG_VALU = 1,     /* one v_fma_f32 per term */
+  RLK_TREE_CFG_MFMA_F32 = 2, /* one v_mfma_f32_32x32x1_2b_f32 per k (reduction length one: a single fused step) */
+  RLK_TREE_CFG_COUNT = 3
+} rlk_tree_config;
+
+/* rlk_det_gemm_tree_bf16 with an explicit leaf loop (rlk_tree_config). */
+int rlk_det_gemm_tree_bf16_config(const void* a, int64_t a_row_stride, int64_t a_k_stride, const void* b,
+                                  int64_t b_k_stride, int64_t b_n_stride, void* c, int64_t ldc, int M, int N,
+                                  int K, int config, void* stream);
 
 /* Contract id of rlk_det_gemm_tree_bf16 (the reference reports
  * "rlkernel.det_gemm.triton_tree_rocm.v1", rl_engine/backends/rocm/gemm/det_gemm.py:101-104). */

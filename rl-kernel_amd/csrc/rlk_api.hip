@@ -94,6 +94,17 @@ const char* rlk_det_gemm_tree_contract_id(void) { return "rlkernel.det_gemm.hip_
 int rlk_det_gemm_tree_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stride, const void* b,
                            int64_t b_k_stride, int64_t b_n_stride, void* c, int64_t ldc, int M, int N, int K,
                            void* stream) {
+  return rlk_det_gemm_tree_bf16_config(a, a_row_stride, a_k_stride, b, b_k_stride, b_n_stride, c, ldc, M, N, K,
+                                       RLK_TREE_CFG_AUTO, stream);
+}
+
+int rlk_det_gemm_tree_bf16_config(const void* a, int64_t a_row_stride, int64_t a_k_stride, const void* b,
+                                  int64_t b_k_stride, int64_t b_n_stride, void* c, int64_t ldc, int M, int N,
+                                  int K, int config, void* stream) {
+  if (config < 0 || config >= RLK_TREE_CFG_COUNT) {
+    set_last_error("rlk_det_gemm_tree_bf16: unknown configuration %d", config);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
   if (M < 0 || N < 0 || K < 0) {
     set_last_error("rlk_det_gemm_tree_bf16: negative size M=%d N=%d K=%d", M, N, K);
     return RLK_ERR_INVALID_ARGUMENT;
@@ -123,7 +134,7 @@ int rlk_det_gemm_tree_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stri
   }
   MatView A{reinterpret_cast<const bf16_bits*>(a), a_row_stride, a_k_stride, M};
   MatView B{reinterpret_cast<const bf16_bits*>(b), b_n_stride, b_k_stride, N};
-  hipError_t err = det_gemm_tree_launch(A, B, c, ldc, M, N, K, s);
+  hipError_t err = det_gemm_tree_launch(A, B, c, ldc, M, N, K, config, s);
   return err == hipSuccess ? RLK_OK : device_error("rlk_det_gemm_tree_bf16", err);
 }
 

@@ -42,7 +42,7 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
 // one row per output column (B.rows == N); any strides. K <= det_gemm_tree_max_k().
 int det_gemm_tree_max_k();
 hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int64_t ldc, int M, int N, int K,
-                                hipStream_t stream);
+                                int config, hipStream_t stream);
 
 // Up to 64 tokens, unit K stride, 16-byte aligned rows, K % 64 == 0. `shallow`: M <= 16 with
 // two workgroups per CU.

@@ -81,15 +81,18 @@ def gemm_strided(
     return out
 
 
-def gemm_tree_strided(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """``out[M,N] = a[M,K] @ b[K,N]`` under the k-tree contract, arbitrary non-negative strides."""
+def gemm_tree_strided(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor, config: int = 0) -> torch.Tensor:
+    """``out[M,N] = a[M,K] @ b[K,N]`` under the k-tree contract, arbitrary non-negative strides.
+
+    ``config``: 0 picks the leaf loop, 1 forces the vector-ALU loop, 2 the fp32 matrix-pipe loop
+    (``rlk_tree_config``; the same bits either way)."""
     m, k = a.shape
     n = b.shape[1]
     if m == 0 or n == 0:
         return out
     lib = _lib.load()
     with torch.cuda.device(a.device):
-        status = lib.rlk_det_gemm_tree_bf16(
+        status = lib.rlk_det_gemm_tree_bf16_config(
             a.data_ptr(),
             a.stride(0),
             a.stride(1),
@@ -101,6 +104,7 @@ def gemm_tree_strided(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> to
             m,
             n,
             k,
+            int(config),
             _stream_handle(a.device),
         )
     _lib.check(status, "rlk_det_gemm_tree_bf16 failed")

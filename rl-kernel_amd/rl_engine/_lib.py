@@ -54,6 +54,7 @@ EXPORTED_SYMBOLS = (
     "rlk_det_gemm_bf16",
     "rlk_det_gemm_pick_config",
     "rlk_det_gemm_tree_bf16",
+    "rlk_det_gemm_tree_bf16_config",
     "rlk_det_gemm_tree_contract_id",
     "rlk_linear_logp_contract_id",
     "rlk_linear_logp_split_count",
@@ -113,6 +114,8 @@ def load() -> ctypes.CDLL:
     lib.rlk_det_gemm_bf16.argtypes = [vp, i64, i64, vp, i64, i64, vp, i64, i32, i32, i32, i32, i32, vp]
     lib.rlk_det_gemm_tree_bf16.restype = i32
     lib.rlk_det_gemm_tree_bf16.argtypes = [vp, i64, i64, vp, i64, i64, vp, i64, i32, i32, i32, vp]
+    lib.rlk_det_gemm_tree_bf16_config.restype = i32
+    lib.rlk_det_gemm_tree_bf16_config.argtypes = [vp, i64, i64, vp, i64, i64, vp, i64, i32, i32, i32, i32, vp]
     lib.rlk_det_gemm_tree_contract_id.restype = c.c_char_p
     lib.rlk_det_gemm_tree_contract_id.argtypes = []
     lib.rlk_det_gemm_pick_config.restype = i32

@@ -146,6 +146,41 @@ def test_tree_special_values(gemm, oracle):
     assert bool(torch.isfinite(got[0]).all()) and bool(torch.isinf(got[1]).all()) and bool(torch.isnan(got[2]).all())
 
 
+def test_both_leaf_loops_compute_the_same_bits(oracle):
+    # The fp32 matrix-pipe leaf (one v_mfma_f32_32x32x1 per k) against the vector-ALU leaf (one
+    # v_fma_f32 per term): every shape of the oracle test, special values (signed zeros, bf16
+    # denormals whose products are fp32 denormals, the largest finite values), strided operands.
+    from rl_engine import _C
+
+    def run(a_d, b_kn, config):
+        out = torch.empty((a_d.size(0), b_kn.size(1)), dtype=torch.bfloat16, device=DEV)
+        return _C.gemm_tree_strided(a_d, b_kn, out, config)
+
+    for m, k, n in TREE_SHAPES + [(300, 4096, 384), (130, 12288, 260), (64, 40000, 128)]:
+        a = inputs.randn_bf16(9700 + k, m, k).to(DEV)
+        w = inputs.randn_bf16(9701 + k, n, k, 0.02).to(DEV)
+        for b_kn in (w.t(), w.t().contiguous()):
+            valu, mfma = run(a, b_kn, 1), run(a, b_kn, 2)
+            assert _same_bits(valu, mfma), (m, k, n)
+            assert _same_bits(run(a, b_kn, 0), mfma)
+    finite = np.array([0x0000, 0x8000, 0x3F80, 0xBF80, 0x0080, 0x8080, 0x0001, 0x8001, 0x7F7F, 0xFF7F, 0x4000, 0x3F00, 0x0040], dtype=np.uint16)
+    small = np.array([0x0000, 0x8000, 0x3F80, 0xBF80, 0x0080, 0x0001, 0x3F00, 0x3E80, 0x0040], dtype=np.uint16)
+    rng = np.random.default_rng(9710)
+    for k in (1, 31, 32, 33, 64, 200, 4096):
+        a_bits = rng.choice(finite, size=(37, k))
+        w_bits = rng.choice(small, size=(70, k))
+        a_d, w_d = inputs.from_bits(a_bits, DEV), inputs.from_bits(w_bits, DEV)
+        valu, mfma = run(a_d, w_d.t(), 1), run(a_d, w_d.t(), 2)
+        nan = torch.isnan(valu.float())
+        assert torch.equal(nan, torch.isnan(mfma.float())), k
+        assert torch.equal(valu.view(torch.int16)[~nan], mfma.view(torch.int16)[~nan]), k
+        want = oracle.k_tree_gemm(a_bits, w_bits)
+        want_nan = (want & 0x7FFF) > 0x7F80
+        assert np.array_equal(inputs.bits(mfma)[~want_nan], want[~want_nan]), k
+    with pytest.raises(ValueError, match="unknown configuration"):
+        run(a_d, w_d.t(), 7)
+
+
 def test_tree_out_argument_empty_shapes_and_errors(gemm):
     a = inputs.randn_bf16(9600, 20, 256).to(DEV)
     w = inputs.randn_bf16(9601, 48, 256, 0.02).to(DEV)
