@@ -58,7 +58,7 @@ def _parse():
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-T table")
     ap.add_argument("--rotate-weights", action="store_true",
                     help="gate_up_tN / down_tN legs: launch over copies of the weight (~1.3 GB in rotation) so that it is read from HBM")
-    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|gate_up_tN|down_tN|logp|logp_decode|logp_mid|logp_bwd|from_logits|ffn|tree|copy|power (used for profiling)")
+    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|gate_up_tN|down_tN|logp|logp_decode|logp_mid|logp_bwd|from_logits|ffn|tree|tree_down|copy|power (used for profiling)")
     return ap.parse_args()
 
 
@@ -243,9 +243,14 @@ def main() -> int:
                "random_operands": looped(x, w_gu), "zero_operands": looped(torch.zeros_like(x), torch.zeros_like(w_gu))}
         print(json.dumps(res))
         return 0
-    if args.only == "tree":
-        ms = _time_calls(lambda: gemm.tree_gemm(x, w_gu.t(), out=out_gu), args.steps, args.warmup)
-        print(json.dumps({"leg": "tree", "ms": ms, "tflops": 2.0 * T * 2 * INTER * HIDDEN / ms * 1e-9,
+    if args.only in ("tree", "tree_down"):
+        if args.only == "tree":
+            ms = _time_calls(lambda: gemm.tree_gemm(x, w_gu.t(), out=out_gu), args.steps, args.warmup)
+            flops = 2.0 * T * 2 * INTER * HIDDEN
+        else:
+            ms = _time_calls(lambda: gemm.tree_gemm(h, w_d.t(), out=out_d), args.steps, args.warmup)
+            flops = 2.0 * T * INTER * HIDDEN
+        print(json.dumps({"leg": args.only, "ms": ms, "tflops": flops / ms * 1e-9,
                           "launches": args.steps + args.warmup}))
         return 0
     if args.only in ("logp_bwd", "from_logits"):
@@ -406,14 +411,19 @@ def main() -> int:
         result["attention_projections"] = proj
         del xa
 
-    # ---- the k-tree contract (vector-ALU kernel) on the same gate_up step
+    # ---- the k-tree contract (leaves on the fp32 matrix pipe, one 32x32x1 MFMA per k) on the same two GEMMs
     if not args.no_shapes:
         ms_tree = _time_calls(lambda: gemm.tree_gemm(x, w_gu.t(), out=out_gu), 3, 1)
+        ms_tree_down = _time_calls(lambda: gemm.tree_gemm(h, w_d.t(), out=out_d), 3, 1)
         result["det_gemm_tree"] = {
             "workload": "gate_up X[4096,4096]xW[24576,4096]^T under the k-tree contract (fp32 FMA leaves of 32, bf16 midpoint tree)",
             "ms": round(ms_tree, 3),
             "tflops": round(flops_gu / ms_tree * 1e-9, 1),
-            "bound": "fp32 vector FMA",
+            "bound": "fp32 mfma",
+            "frac_of_fp32_mfma_peak": round(flops_gu / ms_tree * 1e-9 / 157.3, 4),
+            "down": {"workload": "H[4096,12288]xW[4096,12288]^T, leaves of 24", "ms": round(ms_tree_down, 3),
+                     "tflops": round(flops_d / ms_tree_down * 1e-9, 1),
+                     "frac_of_fp32_mfma_peak": round(flops_d / ms_tree_down * 1e-9 / 157.3, 4)},
             "contract": _lib.load().rlk_det_gemm_tree_contract_id().decode(),
         }
 
