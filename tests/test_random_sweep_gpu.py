@@ -145,6 +145,35 @@ def test_gated_projection_and_k_tree_rows():
         assert _same(tree[row : row + 1], alone), (case, m, inter, k, row)
 
 
+def test_k_tree_leaf_loops_over_layouts_and_depths(oracle):
+    # The matrix-pipe leaf loop (16-byte chunks where the layout allows, elements elsewhere) against
+    # the vector-ALU one over contiguous, transposed, offset and padded operands; small cases also
+    # bit for bit against the CPU oracle.
+    from rl_engine import _C
+
+    d = _Draw(9350)
+    for case in range(90):
+        m, n, k = d.dim(), d.dim(), d.depth()
+        if case % 9 == 0:
+            k = int(d.rng.integers(1, 9)) * 4096 + (0 if case % 2 else 8 * int(d.rng.integers(0, 5)))
+            m, n = min(m, 200), min(n, 200)
+        a = d.view(m, k, int(d.rng.integers(0, 4)), 1.0)
+        w = d.view(n, k, int(d.rng.integers(0, 4)), 0.1)
+        outs = []
+        for config in (1, 2, 0):
+            out = torch.full((m, n + 3), 7.0, device=DEV, dtype=torch.bfloat16)[:, :n]
+            outs.append(_C.gemm_tree_strided(a, w.t(), out, config))
+            assert bool((out.as_strided((m, 3), (n + 3, 1), n) == 7.0).all()), (case, "wrote past N")
+        assert _same(outs[0], outs[1]) and _same(outs[0], outs[2]), (case, m, n, k, a.stride(), w.stride())
+        if m * n * k <= 4_000_000:
+            want = oracle.k_tree_gemm(
+                a.contiguous().view(torch.int16).cpu().numpy().view(np.uint16),
+                w.contiguous().view(torch.int16).cpu().numpy().view(np.uint16),
+            )
+            got = outs[1].contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+            assert np.array_equal(got, want), (case, m, n, k)
+
+
 def test_linear_logp_backward_configurations_rows_and_values():
     from rl_engine import _C, _lib
 
