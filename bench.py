@@ -411,7 +411,7 @@ def main() -> int:
         result["attention_projections"] = proj
         del xa
 
-    # ---- the k-tree contract (leaves on the fp32 matrix pipe, one 32x32x1 MFMA per k) on the same two GEMMs
+    # ---- the k-tree contract (leaves on the fp32 matrix pipe, one reduction-length-one fp32 MFMA per k) on the same two GEMMs
     if not args.no_shapes:
         ms_tree = _time_calls(lambda: gemm.tree_gemm(x, w_gu.t(), out=out_gu), 3, 1)
         ms_tree_down = _time_calls(lambda: gemm.tree_gemm(h, w_d.t(), out=out_d), 3, 1)

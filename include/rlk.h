@@ -119,7 +119,7 @@ int rlk_det_gemm_tree_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stri
 typedef enum rlk_tree_config {
   RLK_TREE_CFG_AUTO = 0,
   RLK_TREE_CFG_VALU = 1,     /* one v_fma_f32 per term */
-  RLK_TREE_CFG_MFMA_F32 = 2, /* one v_mfma_f32_32x32x1_2b_f32 per k (reduction length one: a single fused step) */
+  RLK_TREE_CFG_MFMA_F32 = 2, /* one v_mfma_f32_16x16x1_4b_f32 per k (reduction length one: a single fused step) */
   RLK_TREE_CFG_COUNT = 3
 } rlk_tree_config;
 

@@ -15,17 +15,17 @@
 // a K-sharded rank holds) evaluates to exactly that tree node. The scalar chain of a leaf
 // cannot go through the bf16 matrix instructions (a 16x16x32 step sums its 32 products in its
 // own order). Two leaf loops evaluate it, bit for bit the same:
-//   * vector ALU: a thread owns 4 rows x 8 columns and issues one v_fma_f32 per term;
-//   * fp32 matrix pipe: a wave owns 32 rows x 64 columns and issues one
-//     v_mfma_f32_32x32x1_2b_f32 per k. With a reduction length of one, an instruction adds
-//     exactly one product to every accumulator, and the product of two bf16 values is exact
-//     in fp32, so the step is the same single rounding as the fused multiply-add, at twice
-//     the vector rate.
+//   * vector ALU (det_gemm_tree_kernel): 256 threads per tile, a thread owns 4 rows x 8
+//     columns and issues one v_fma_f32 per term; operands staged in LDS as fp32, [k][row];
+//   * fp32 matrix pipe (det_gemm_tree_wide_kernel, the default): 512 threads per tile, a wave
+//     owns 32 rows x 32 columns and issues one v_mfma_f32_16x16x1_4b_f32 per k. With a
+//     reduction length of one, an instruction adds exactly one product to every accumulator,
+//     and the product of two bf16 values is exact in fp32, so the step is the same single
+//     rounding as the fused multiply-add, at twice the vector rate; operands staged in LDS
+//     as fp32, [row][k].
 //
-// A workgroup of 256 threads owns a 64 x 128 output tile.
-// Leaves are visited left to right. The operands of a leaf are converted to fp32 on their
-// way into LDS ([k][row], so a k step reads consecutive floats of one k row),
-// the next leaf is fetched while the current one is summed. The tree is evaluated on the
+// A workgroup owns a 64 x 128 output tile. Leaves are visited left to right, the next leaf
+// is fetched while the current one is summed. The tree is evaluated on the
 // fly: a finished node waits in the register slot of its depth until its right sibling is
 // finished, so a thread holds at most one bf16 node per tree level. Which slot is read or
 // written is the same for every thread (it depends on K only), so the slot index is a
@@ -44,7 +44,6 @@ constexpr int kTreeBStride = kTreeBN + 4;
 constexpr int kTreeStageFloats = kTreeLeaf * (kTreeAStride + kTreeBStride);
 constexpr int kTreeALoads = kTreeBM * kTreeLeaf / kTreeThreads;  // 8 elements per thread per leaf
 constexpr int kTreeBLoads = kTreeBN * kTreeLeaf / kTreeThreads;  // 16
-constexpr int kTreeRowBytes = 2 * kTreeLeaf + 16;                // bf16 stage of the matrix-pipe leaf
 
 // Depth of the deepest leaf: sizes at depth d are floor or ceil of K / 2^d.
 static int tree_depth(int K) {
@@ -60,18 +59,10 @@ __device__ __forceinline__ uint32_t bf16x2_add(uint32_t x, uint32_t y) {
 }
 
 // MAXD: number of tree levels below the root the kernel has slots for.
-typedef float f32x32_t __attribute__((ext_vector_type(32)));
-
-// MFMA: the leaf loop on the fp32 matrix pipe (else on the vector ALU).
-template <int MAXD, bool MFMA>
+template <int MAXD>
 __global__ __launch_bounds__(kTreeThreads, MAXD <= 10 ? 2 : 1) void det_gemm_tree_kernel(MatView A, MatView B, bf16_bits* __restrict__ C,
-                                                                     int64_t ldc, int M, int N, int K, int tiles_m,
-                                                                     int fast) {
-  // Vector-ALU leaf: fp32 operands, [k][row]. Matrix-pipe leaf: bf16 operands as they lie in
-  // memory, [row][k] with 80-byte rows (16-byte reads of consecutive rows fall on distinct banks).
-  constexpr int kStageBytes = MFMA ? (kTreeBM + kTreeBN) * kTreeRowBytes : kTreeStageFloats * 4;
-  __shared__ __attribute__((aligned(16))) char stage_bytes[2][kStageBytes];
-  auto stage = [&](int buf) { return reinterpret_cast<float*>(stage_bytes[buf]); };
+                                                                     int64_t ldc, int M, int N, int K, int tiles_m) {
+  __shared__ __attribute__((aligned(16))) float stage[2][kTreeStageFloats];
 
   const int tid = threadIdx.x;
   const int tile_m = blockIdx.x % tiles_m;
@@ -91,107 +82,38 @@ __global__ __launch_bounds__(kTreeThreads, MAXD <= 10 ? 2 : 1) void det_gemm_tre
   const int a_last = M - 1 - m0, b_last = N - 1 - n0;
   const bf16_bits* a_tile = A.ptr + (int64_t)m0 * A.row_stride;
   const bf16_bits* b_tile = B.ptr + (int64_t)n0 * B.row_stride;
-  bf16_bits a_reg[MFMA ? 1 : kTreeALoads], b_reg[MFMA ? 1 : kTreeBLoads];
-  // Matrix-pipe kernel: 12 registers per thread. An operand with unit K stride, 16-byte aligned
-  // rows and leaves that begin and end on multiples of 8 (bit 0 of `fast`: A, bit 1: B) is
-  // fetched as 16-byte chunks (row tid / 4 (+ 64), chunk tid % 4 of the leaf); any other layout
-  // element by element, two bf16 per register.
-  uint32_t held[12];
-  const bool a_fast = MFMA && (fast & 1), b_fast = MFMA && (fast & 2);
-  const int chunk_row = tid >> 2, chunk = tid & 3;
+  bf16_bits a_reg[kTreeALoads], b_reg[kTreeBLoads];
   auto fetch = [&](int lo) {
-    if constexpr (MFMA) {
-      const int kc = lo + 8 * chunk < K ? lo + 8 * chunk : 0;  // a chunk past the leaf is not used
-      if (a_fast) {
-        const int row = chunk_row < a_last ? chunk_row : a_last;
-        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(a_tile + (int64_t)row * A.row_stride + kc);
-        held[0] = v[0]; held[1] = v[1]; held[2] = v[2]; held[3] = v[3];
-      }
-      if (b_fast) {
+    const int k = (lo + load_k < K) ? lo + load_k : K - 1;
+    const bf16_bits* a_col = a_tile + (int64_t)k * A.k_stride;
+    const bf16_bits* b_col = b_tile + (int64_t)k * B.k_stride;
+    if (interior) {
+      int64_t off = (int64_t)load_row * A.row_stride;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int row = chunk_row + 64 * j < b_last ? chunk_row + 64 * j : b_last;
-          const u32x4_t v = *reinterpret_cast<const u32x4_t*>(b_tile + (int64_t)row * B.row_stride + kc);
-          held[4 + 4 * j] = v[0]; held[5 + 4 * j] = v[1]; held[6 + 4 * j] = v[2]; held[7 + 4 * j] = v[3];
-        }
-      }
-      const int k = (lo + load_k < K) ? lo + load_k : K - 1;
-      if (!a_fast) {
-        const bf16_bits* a_col = a_tile + (int64_t)k * A.k_stride;
+      for (int j = 0; j < kTreeALoads; ++j, off += 8 * A.row_stride) a_reg[j] = a_col[off];
+      off = (int64_t)load_row * B.row_stride;
 #pragma unroll
-        for (int j = 0; j < kTreeALoads; j += 2) {
-          const int r0 = load_row + 8 * j, r1 = r0 + 8;
-          const uint32_t e0 = a_col[(int64_t)(r0 < a_last ? r0 : a_last) * A.row_stride];
-          const uint32_t e1 = a_col[(int64_t)(r1 < a_last ? r1 : a_last) * A.row_stride];
-          held[j / 2] = e0 | (e1 << 16);
-        }
-      }
-      if (!b_fast) {
-        const bf16_bits* b_col = b_tile + (int64_t)k * B.k_stride;
-#pragma unroll
-        for (int j = 0; j < kTreeBLoads; j += 2) {
-          const int r0 = load_row + 8 * j, r1 = r0 + 8;
-          const uint32_t e0 = b_col[(int64_t)(r0 < b_last ? r0 : b_last) * B.row_stride];
-          const uint32_t e1 = b_col[(int64_t)(r1 < b_last ? r1 : b_last) * B.row_stride];
-          held[4 + j / 2] = e0 | (e1 << 16);
-        }
-      }
+      for (int j = 0; j < kTreeBLoads; ++j, off += 8 * B.row_stride) b_reg[j] = b_col[off];
     } else {
-      const int k = (lo + load_k < K) ? lo + load_k : K - 1;
-      const bf16_bits* a_col = a_tile + (int64_t)k * A.k_stride;
-      const bf16_bits* b_col = b_tile + (int64_t)k * B.k_stride;
-      if (interior) {
-        int64_t off = (int64_t)load_row * A.row_stride;
 #pragma unroll
-        for (int j = 0; j < kTreeALoads; ++j, off += 8 * A.row_stride) a_reg[j] = a_col[off];
-        off = (int64_t)load_row * B.row_stride;
+      for (int j = 0; j < kTreeALoads; ++j) {
+        const int row = load_row + 8 * j;
+        a_reg[j] = a_col[(int64_t)(row < a_last ? row : a_last) * A.row_stride];
+      }
 #pragma unroll
-        for (int j = 0; j < kTreeBLoads; ++j, off += 8 * B.row_stride) b_reg[j] = b_col[off];
-      } else {
-#pragma unroll
-        for (int j = 0; j < kTreeALoads; ++j) {
-          const int row = load_row + 8 * j;
-          a_reg[j] = a_col[(int64_t)(row < a_last ? row : a_last) * A.row_stride];
-        }
-#pragma unroll
-        for (int j = 0; j < kTreeBLoads; ++j) {
-          const int row = load_row + 8 * j;
-          b_reg[j] = b_col[(int64_t)(row < b_last ? row : b_last) * B.row_stride];
-        }
+      for (int j = 0; j < kTreeBLoads; ++j) {
+        const int row = load_row + 8 * j;
+        b_reg[j] = b_col[(int64_t)(row < b_last ? row : b_last) * B.row_stride];
       }
     }
   };
   auto deposit = [&](int buf) {
-    if constexpr (MFMA) {
-      char* as = stage_bytes[buf];
-      char* bs = as + kTreeBM * kTreeRowBytes;
-      if (a_fast) {
-        *reinterpret_cast<u32x4_t*>(as + chunk_row * kTreeRowBytes + 16 * chunk) = u32x4_t{held[0], held[1], held[2], held[3]};
-      } else {
+    float* as = stage[buf];
+    float* bs = as + kTreeLeaf * kTreeAStride;
 #pragma unroll
-        for (int j = 0; j < kTreeALoads; ++j)
-          *reinterpret_cast<bf16_bits*>(as + (load_row + 8 * j) * kTreeRowBytes + 2 * load_k) =
-              (bf16_bits)((held[j / 2] >> (16 * (j & 1))) & 0xffffu);
-      }
-      if (b_fast) {
+    for (int j = 0; j < kTreeALoads; ++j) as[load_k * kTreeAStride + load_row + 8 * j] = bf16_bits_to_float(a_reg[j]);
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-          *reinterpret_cast<u32x4_t*>(bs + (chunk_row + 64 * j) * kTreeRowBytes + 16 * chunk) =
-              u32x4_t{held[4 + 4 * j], held[5 + 4 * j], held[6 + 4 * j], held[7 + 4 * j]};
-      } else {
-#pragma unroll
-        for (int j = 0; j < kTreeBLoads; ++j)
-          *reinterpret_cast<bf16_bits*>(bs + (load_row + 8 * j) * kTreeRowBytes + 2 * load_k) =
-              (bf16_bits)((held[4 + j / 2] >> (16 * (j & 1))) & 0xffffu);
-      }
-    } else {
-      float* as = stage(buf);
-      float* bs = as + kTreeLeaf * kTreeAStride;
-#pragma unroll
-      for (int j = 0; j < kTreeALoads; ++j) as[load_k * kTreeAStride + load_row + 8 * j] = bf16_bits_to_float(a_reg[j]);
-#pragma unroll
-      for (int j = 0; j < kTreeBLoads; ++j) bs[load_k * kTreeBStride + load_row + 8 * j] = bf16_bits_to_float(b_reg[j]);
-    }
+    for (int j = 0; j < kTreeBLoads; ++j) bs[load_k * kTreeBStride + load_row + 8 * j] = bf16_bits_to_float(b_reg[j]);
   };
 
   // [lo, hi) of the node reached from the root by `path` (bit d set: right child at depth d).
@@ -237,47 +159,14 @@ __global__ __launch_bounds__(kTreeThreads, MAXD <= 10 ? 2 : 1) void det_gemm_tre
     }
 
     // The leaf: 32 independent chains per thread, k ascending.
-    const float* as = stage(leaf & 1);
+    const float* as = stage[leaf & 1];
     const float* bs = as + kTreeLeaf * kTreeAStride;
-    const int len = hi - lo;
-    if constexpr (MFMA) {
-      // Wave w: rows 32 (w & 1) ..., columns 64 (w >> 1) .... Block 0 of the instruction takes
-      // columns 0..31, block 1 columns 32..63; the row operand of block 0 serves both (cbsz = 1).
-      const int lane = tid & 63, wave = tid >> 6;
-      const char* arow = stage_bytes[leaf & 1] + (32 * (wave & 1) + (lane & 31)) * kTreeRowBytes;
-      const char* brow = stage_bytes[leaf & 1] + (kTreeBM + 64 * (wave >> 1) + lane) * kTreeRowBytes;
-      f32x32_t acc;
-#pragma unroll
-      for (int r = 0; r < 32; ++r) acc[r] = 0.f;
-      // Element 2 i of a chunk is the low half of word i, element 2 i + 1 the high half; either way
-      // the fp32 operand is the bf16 pattern in the upper 16 bits.
-      auto step = [&](const u32x4_t& av, const u32x4_t& bv, int e) {
-        const float a = __uint_as_float((e & 1) ? (av[e >> 1] & 0xffff0000u) : (av[e >> 1] << 16));
-        const float b = __uint_as_float((e & 1) ? (bv[e >> 1] & 0xffff0000u) : (bv[e >> 1] << 16));
-        acc = __builtin_amdgcn_mfma_f32_32x32x1f32(a, b, acc, 1, 0, 0);
-      };
-      const int whole = len >> 3, rest = len & 7;
-      for (int c = 0; c < whole; ++c) {
-        const u32x4_t av = *reinterpret_cast<const u32x4_t*>(arow + 16 * c);
-        const u32x4_t bv = *reinterpret_cast<const u32x4_t*>(brow + 16 * c);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) step(av, bv, e);
-      }
-      if (rest) {  // the chunk is read whole (it lies inside the row); only its first `rest` elements count
-        const u32x4_t av = *reinterpret_cast<const u32x4_t*>(arow + 16 * whole);
-        const u32x4_t bv = *reinterpret_cast<const u32x4_t*>(brow + 16 * whole);
-#pragma unroll
-        for (int e = 0; e < 7; ++e)
-          if (e < rest) step(av, bv, e);
-      }
-#pragma unroll
-      for (int q = 0; q < 16; ++q) cur[q] = pack_bf16x2(acc[2 * q], acc[2 * q + 1]);
-    } else {
     float acc[4][8];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < 8; ++j) acc[i][j] = 0.f;
+    const int len = hi - lo;
     // Operands of step k + 1 are read while step k is summed (one wave per SIMD: nothing else
     // hides the LDS latency). Row len of the stage is read and not used.
     const float* ap = as + 4 * ty;
@@ -314,8 +203,6 @@ __global__ __launch_bounds__(kTreeThreads, MAXD <= 10 ? 2 : 1) void det_gemm_tre
 #pragma unroll
       for (int j = 0; j < 4; ++j) cur[i * 4 + j] = pack_bf16x2(acc[i][2 * j], acc[i][2 * j + 1]);
 
-    }
-
     // Finished right children meet their waiting siblings.
     int d = depth;
     while (d > 0 && ((path >> d) & 1u)) {
@@ -345,23 +232,6 @@ __global__ __launch_bounds__(kTreeThreads, MAXD <= 10 ? 2 : 1) void det_gemm_tre
     hi = nhi;
   }
 
-  if constexpr (MFMA) {
-    // Accumulator r of the instruction: block r / 16 (32 columns each); within a block
-    // row 8 (q / 4) + 4 (lane / 32) + q % 4 with q = r % 16, column lane % 32. cur packs
-    // accumulators 2 q', 2 q' + 1 (two consecutive rows of one column).
-    const int lane = tid & 63, wave = tid >> 6;
-    const int row_base = m0 + 32 * (wave & 1) + 4 * (lane >> 5);
-    const int col_base = n0 + 64 * (wave >> 1) + (lane & 31);
-#pragma unroll
-    for (int r = 0; r < 32; ++r) {
-      const int q = r & 15;
-      const int row = row_base + 8 * (q >> 2) + (q & 3);
-      const int col = col_base + 32 * (r >> 4);
-      const uint32_t pair = cur[r >> 1];
-      if (row < M && col < N) C[(int64_t)row * ldc + col] = (bf16_bits)((r & 1) ? (pair >> 16) : (pair & 0xffffu));
-    }
-    return;
-  }
   // cur[i * 4 + j]: row 4 ty + i, column pair (j < 2 ? 4 tx + 2 j : 64 + 4 tx + 2 (j - 2)).
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -384,24 +254,305 @@ __global__ __launch_bounds__(kTreeThreads, MAXD <= 10 ? 2 : 1) void det_gemm_tre
   }
 }
 
+// The matrix-pipe leaf with eight waves per tile: a wave owns 32 rows x 32 columns (the four
+// 16 x 16 blocks of v_mfma_f32_16x16x1_4b_f32), 16 accumulators and 8 packed tree registers per
+// level per lane, so four waves fit on a SIMD and one wave's rounding and tree adds run under the
+// matrix instructions of the others. Operands are converted to fp32 once, on their way into LDS
+// ([row][k], 144-byte rows: a lane's 16-byte read of its own row is conflict free), so a k step
+// needs no vector instruction besides the MFMA.
+constexpr int kTreeWideThreads = 512;
+constexpr int kTreeWideRowBytes = 4 * kTreeLeaf + 16;
+constexpr int kTreeWideRowBytesBf16 = 2 * kTreeLeaf + 16;
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+// F32_STAGE = false keeps the operands in LDS as bf16 (80-byte rows) and makes the fp32 pattern
+// with one shift or mask per operand and k instead: fewer live registers, which is what decides
+// between four waves per SIMD and spills when the tree has 8 to 10 levels.
+template <int MAXD, bool F32_STAGE>
+__global__ __launch_bounds__(kTreeWideThreads, MAXD <= 10 ? 4 : 2) void det_gemm_tree_wide_kernel(
+    MatView A, MatView B, bf16_bits* __restrict__ C, int64_t ldc, int M, int N, int K, int tiles_m, int fast) {
+  constexpr int kRowBytes = F32_STAGE ? kTreeWideRowBytes : kTreeWideRowBytesBf16;
+  constexpr int kStageBytes = (kTreeBM + kTreeBN) * kRowBytes;
+  __shared__ __attribute__((aligned(16))) char stage_bytes[2][kStageBytes];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int tile_m = blockIdx.x % tiles_m;
+  const int tile_n = blockIdx.x / tiles_m;
+  const int m0 = tile_m * kTreeBM;
+  const int n0 = tile_n * kTreeBN;
+  const int a_last = M - 1 - m0, b_last = N - 1 - n0;
+  const bf16_bits* a_tile = A.ptr + (int64_t)m0 * A.row_stride;
+  const bf16_bits* b_tile = B.ptr + (int64_t)n0 * B.row_stride;
+
+  // Staging roles. Chunked operand (bit 0 of `fast`: A, bit 1: B): thread t holds chunk t % 4 of
+  // row t / 4 (B: 128 rows, all threads; A: 64 rows, threads 0..255). Element-wise operand:
+  // k = t % 32, rows t / 32 + 16 j, two bf16 per register.
+  const bool a_fast = fast & 1, b_fast = fast & 2;
+  const int chunk_row = tid >> 2, chunk = tid & 3;
+  const int load_k = tid & 31, load_row = tid >> 5;
+  uint32_t held[8];  // [0, 4): A, [4, 8): B
+  auto fetch = [&](int lo) {
+    const int kc = lo + 8 * chunk < K ? lo + 8 * chunk : 0;  // a chunk past the leaf is not used
+    const int k = (lo + load_k < K) ? lo + load_k : K - 1;
+    if (a_fast) {
+      if (tid < 256) {
+        const int row = chunk_row < a_last ? chunk_row : a_last;
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(a_tile + (int64_t)row * A.row_stride + kc);
+        held[0] = v[0]; held[1] = v[1]; held[2] = v[2]; held[3] = v[3];
+      }
+    } else {
+      const bf16_bits* a_col = a_tile + (int64_t)k * A.k_stride;
+#pragma unroll
+      for (int j = 0; j < 4; j += 2) {
+        const int r0 = load_row + 16 * j, r1 = r0 + 16;
+        const uint32_t e0 = a_col[(int64_t)(r0 < a_last ? r0 : a_last) * A.row_stride];
+        const uint32_t e1 = a_col[(int64_t)(r1 < a_last ? r1 : a_last) * A.row_stride];
+        held[j / 2] = e0 | (e1 << 16);
+      }
+    }
+    if (b_fast) {
+      const int row = chunk_row < b_last ? chunk_row : b_last;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(b_tile + (int64_t)row * B.row_stride + kc);
+      held[4] = v[0]; held[5] = v[1]; held[6] = v[2]; held[7] = v[3];
+    } else {
+      const bf16_bits* b_col = b_tile + (int64_t)k * B.k_stride;
+#pragma unroll
+      for (int j = 0; j < 8; j += 2) {
+        const int r0 = load_row + 16 * j, r1 = r0 + 16;
+        const uint32_t e0 = b_col[(int64_t)(r0 < b_last ? r0 : b_last) * B.row_stride];
+        const uint32_t e1 = b_col[(int64_t)(r1 < b_last ? r1 : b_last) * B.row_stride];
+        held[4 + j / 2] = e0 | (e1 << 16);
+      }
+    }
+  };
+  // bf16 pair in one register -> two fp32 patterns
+  auto lo_f32 = [](uint32_t v) { return v << 16; };
+  auto hi_f32 = [](uint32_t v) { return v & 0xffff0000u; };
+  auto deposit_chunk = [&](char* row, const uint32_t* v) {
+    *reinterpret_cast<u32x4_t*>(row + 32 * chunk) = u32x4_t{lo_f32(v[0]), hi_f32(v[0]), lo_f32(v[1]), hi_f32(v[1])};
+    *reinterpret_cast<u32x4_t*>(row + 32 * chunk + 16) = u32x4_t{lo_f32(v[2]), hi_f32(v[2]), lo_f32(v[3]), hi_f32(v[3])};
+  };
+  auto deposit = [&](int buf) {
+    char* as = stage_bytes[buf];
+    char* bs = as + kTreeBM * kRowBytes;
+    if constexpr (F32_STAGE) {
+      if (a_fast) {
+        if (tid < 256) deposit_chunk(as + chunk_row * kRowBytes, held);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          *reinterpret_cast<uint32_t*>(as + (load_row + 16 * j) * kRowBytes + 4 * load_k) =
+              (j & 1) ? hi_f32(held[j / 2]) : lo_f32(held[j / 2]);
+      }
+      if (b_fast) {
+        deposit_chunk(bs + chunk_row * kRowBytes, held + 4);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          *reinterpret_cast<uint32_t*>(bs + (load_row + 16 * j) * kRowBytes + 4 * load_k) =
+              (j & 1) ? hi_f32(held[4 + j / 2]) : lo_f32(held[4 + j / 2]);
+      }
+    } else {
+      if (a_fast) {
+        if (tid < 256)
+          *reinterpret_cast<u32x4_t*>(as + chunk_row * kRowBytes + 16 * chunk) = u32x4_t{held[0], held[1], held[2], held[3]};
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          *reinterpret_cast<bf16_bits*>(as + (load_row + 16 * j) * kRowBytes + 2 * load_k) =
+              (bf16_bits)((held[j / 2] >> (16 * (j & 1))) & 0xffffu);
+      }
+      if (b_fast) {
+        *reinterpret_cast<u32x4_t*>(bs + chunk_row * kRowBytes + 16 * chunk) = u32x4_t{held[4], held[5], held[6], held[7]};
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          *reinterpret_cast<bf16_bits*>(bs + (load_row + 16 * j) * kRowBytes + 2 * load_k) =
+              (bf16_bits)((held[4 + j / 2] >> (16 * (j & 1))) & 0xffffu);
+      }
+    }
+  };
+
+  auto range_at = [&](int depth, uint32_t path, int& lo, int& hi) {
+    lo = 0;
+    hi = K;
+    for (int d = 1; d <= depth; ++d) {
+      const int mid = lo + (hi - lo) / 2;
+      if ((path >> d) & 1u) lo = mid; else hi = mid;
+    }
+  };
+
+  uint32_t slot[MAXD][8];  // slot[d - 1]: finished left child at depth d, waiting for its sibling
+  uint32_t cur[8];
+
+  // Wave w: rows 32 (w & 1) ..., columns 32 (w >> 1) .... Block b of the instruction is rows
+  // 16 (b >> 1) ..., columns 16 (b & 1) ...: lane l feeds row 16 (l >> 5) + l % 16 and column
+  // 16 ((l >> 4) & 1) + l % 16.
+  const int a_row = 32 * (wave & 1) + 16 * (lane >> 5) + (lane & 15);
+  const int b_row = kTreeBM + 32 * (wave >> 1) + 16 * ((lane >> 4) & 1) + (lane & 15);
+
+  int depth = 0, lo = 0, hi = K;
+  uint32_t path = 0;
+  while (hi - lo > kTreeLeaf) {
+    hi = lo + (hi - lo) / 2;
+    ++depth;
+  }
+  fetch(lo);
+  deposit(0);
+  __syncthreads();
+
+  for (int leaf = 0;; ++leaf) {
+    bool has_next;
+    uint32_t npath = path;
+    int nlo = 0, nhi = 0, ndepth = 0;
+    if (fast & 4) {
+      // All leaves equally long (2^depth divides K): leaf i is [i * len, (i + 1) * len) at the
+      // deepest level, and bit d of its path is bit depth - d of i.
+      const int next = leaf + 1;
+      has_next = next < (1 << depth);
+      if (has_next) {
+        nlo = next * (hi - lo);
+        nhi = nlo + (hi - lo);
+        ndepth = depth;
+        npath = (__brev((uint32_t)next) >> (32 - depth)) << 1;
+      }
+    } else {
+      int nd = depth;
+      while (nd > 0 && ((path >> nd) & 1u)) --nd;
+      has_next = nd > 0;
+      if (has_next) {
+        npath = (path & ((1u << nd) - 1u)) | (1u << nd);
+        range_at(nd, npath, nlo, nhi);
+        ndepth = nd;
+        while (nhi - nlo > kTreeLeaf) {
+          nhi = nlo + (nhi - nlo) / 2;
+          ++ndepth;
+        }
+      }
+    }
+    if (has_next) fetch(nlo);
+
+    const int len = hi - lo;
+    const char* arow = stage_bytes[leaf & 1] + a_row * kRowBytes;
+    const char* brow = stage_bytes[leaf & 1] + b_row * kRowBytes;
+    f32x16_t acc;
+    if constexpr (F32_STAGE) {
+      // Four k per 16-byte read. The first step of a leaf adds to a literal zero (no registers to
+      // clear); a group past the leaf's length is read whole (it lies inside the row) and only its
+      // first len % 4 elements count.
+      auto read4 = [&](int g, f32x4_t& av, f32x4_t& bv) {
+        av = *reinterpret_cast<const f32x4_t*>(arow + 16 * g);
+        bv = *reinterpret_cast<const f32x4_t*>(brow + 16 * g);
+      };
+      f32x4_t av, bv;
+      read4(0, av, bv);
+      acc = __builtin_amdgcn_mfma_f32_16x16x1f32(av[0], bv[0], f32x16_t{}, 0, 0, 0);
+      const int groups = len >> 2, rest = len & 3;
+      if (groups > 0) {
+#pragma unroll
+        for (int e = 1; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x1f32(av[e], bv[e], acc, 0, 0, 0);
+        for (int g = 1; g < groups; ++g) {
+          read4(g, av, bv);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x1f32(av[e], bv[e], acc, 0, 0, 0);
+        }
+        if (rest) {
+          read4(groups, av, bv);
+#pragma unroll
+          for (int e = 0; e < 3; ++e)
+            if (e < rest) acc = __builtin_amdgcn_mfma_f32_16x16x1f32(av[e], bv[e], acc, 0, 0, 0);
+        }
+      } else {
+#pragma unroll
+        for (int e = 1; e < 3; ++e)
+          if (e < rest) acc = __builtin_amdgcn_mfma_f32_16x16x1f32(av[e], bv[e], acc, 0, 0, 0);
+      }
+    } else {
+      // Eight k per 16-byte read; element 2 i of a chunk is the low half of word i, element 2 i + 1
+      // the high half, and the fp32 operand is that bf16 pattern in the upper 16 bits.
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+      auto step = [&](const u32x4_t& av, const u32x4_t& bv, int e) {
+        const float a = __uint_as_float((e & 1) ? (av[e >> 1] & 0xffff0000u) : (av[e >> 1] << 16));
+        const float b = __uint_as_float((e & 1) ? (bv[e >> 1] & 0xffff0000u) : (bv[e >> 1] << 16));
+        acc = __builtin_amdgcn_mfma_f32_16x16x1f32(a, b, acc, 0, 0, 0);
+      };
+      const int whole = len >> 3, rest = len & 7;
+      for (int c = 0; c < whole; ++c) {
+        const u32x4_t av = *reinterpret_cast<const u32x4_t*>(arow + 16 * c);
+        const u32x4_t bv = *reinterpret_cast<const u32x4_t*>(brow + 16 * c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) step(av, bv, e);
+      }
+      if (rest) {  // the chunk is read whole (it lies inside the row); only its first `rest` elements count
+        const u32x4_t av = *reinterpret_cast<const u32x4_t*>(arow + 16 * whole);
+        const u32x4_t bv = *reinterpret_cast<const u32x4_t*>(brow + 16 * whole);
+#pragma unroll
+        for (int e = 0; e < 7; ++e)
+          if (e < rest) step(av, bv, e);
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 8; ++q) cur[q] = pack_bf16x2(acc[2 * q], acc[2 * q + 1]);
+
+    int d = depth;
+    while (d > 0 && ((path >> d) & 1u)) {
+#pragma unroll
+      for (int s = 1; s <= MAXD; ++s) {
+        if (s == d) {
+#pragma unroll
+          for (int r = 0; r < 8; ++r) cur[r] = bf16x2_add(slot[s - 1][r], cur[r]);
+        }
+      }
+      --d;
+    }
+    if (d == 0) break;  // cur is the root
+#pragma unroll
+    for (int s = 1; s <= MAXD; ++s) {
+      if (s == d) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) slot[s - 1][r] = cur[r];
+      }
+    }
+
+    deposit((leaf + 1) & 1);
+    __syncthreads();
+    depth = ndepth;
+    path = npath;
+    lo = nlo;
+    hi = nhi;
+  }
+
+  // Accumulator r: block r / 4; row 16 (block >> 1) + 4 (lane / 16) + r % 4, column 16 (block & 1) + lane % 16.
+  // cur[q] packs accumulators 2 q, 2 q + 1 (two consecutive rows of one column).
+  const int row_base = m0 + 32 * (wave & 1) + 4 * (lane >> 4);
+  const int col_base = n0 + 32 * (wave >> 1) + (lane & 15);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int block = r >> 2;
+    const int row = row_base + 16 * (block >> 1) + (r & 3);
+    const int col = col_base + 16 * (block & 1);
+    const uint32_t pair = cur[r >> 1];
+    if (row < M && col < N) C[(int64_t)row * ldc + col] = (bf16_bits)((r & 1) ? (pair >> 16) : (pair & 0xffffu));
+  }
+}
+
 int det_gemm_tree_max_k() { return kTreeLeaf << 20; }
 
-template <bool MFMA>
-static hipError_t launch_tree(const MatView& A, const MatView& B, bf16_bits* out, int64_t ldc, int M, int N, int K,
-                              int depth, unsigned tiles, int tiles_m, int fast, hipStream_t stream) {
-  if (depth <= 7) {  // K <= 4096: few enough slots for two workgroups per CU
-    hipLaunchKernelGGL((det_gemm_tree_kernel<7, MFMA>), dim3(tiles), dim3(kTreeThreads), 0, stream, A, B, out, ldc, M, N,
-                       K, tiles_m, fast);
-  } else if (depth <= 10) {
-    hipLaunchKernelGGL((det_gemm_tree_kernel<10, MFMA>), dim3(tiles), dim3(kTreeThreads), 0, stream, A, B, out, ldc, M,
-                       N, K, tiles_m, fast);
-  } else if (depth <= 20) {
-    hipLaunchKernelGGL((det_gemm_tree_kernel<20, MFMA>), dim3(tiles), dim3(kTreeThreads), 0, stream, A, B, out, ldc, M,
-                       N, K, tiles_m, fast);
-  } else {
-    return hipErrorInvalidValue;
-  }
-  return hipGetLastError();
+template <int MAXD>
+static void launch_valu(const MatView& A, const MatView& B, bf16_bits* out, int64_t ldc, int M, int N, int K,
+                        unsigned tiles, int tiles_m, hipStream_t stream) {
+  hipLaunchKernelGGL(det_gemm_tree_kernel<MAXD>, dim3(tiles), dim3(kTreeThreads), 0, stream, A, B, out, ldc, M, N, K,
+                     tiles_m);
+}
+
+template <int MAXD>
+static void launch_wide(const MatView& A, const MatView& B, bf16_bits* out, int64_t ldc, int M, int N, int K,
+                        unsigned tiles, int tiles_m, int fast, hipStream_t stream) {
+  // fp32 staging except for 8 to 10 tree levels, where its extra live registers would spill
+  hipLaunchKernelGGL((det_gemm_tree_wide_kernel<MAXD, MAXD != 10>), dim3(tiles), dim3(kTreeWideThreads), 0, stream, A, B,
+                     out, ldc, M, N, K, tiles_m, fast);
 }
 
 // A[M, K] and B as rows of output columns (B.rows = N), any strides; C[m * ldc + n].
@@ -410,23 +561,32 @@ hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int
                                 int config, hipStream_t stream) {
   const int tiles_m = (M + kTreeBM - 1) / kTreeBM;
   const int tiles_n = (N + kTreeBN - 1) / kTreeBN;
-  const int64_t tiles = (int64_t)tiles_m * tiles_n;
-  if (tiles > 0x7fffffff) return hipErrorInvalidValue;
+  const int64_t tiles64 = (int64_t)tiles_m * tiles_n;
+  if (tiles64 > 0x7fffffff) return hipErrorInvalidValue;
+  const unsigned tiles = (unsigned)tiles64;
   const int depth = tree_depth(K);
+  if (depth > 20) return hipErrorInvalidValue;
   bf16_bits* out = reinterpret_cast<bf16_bits*>(C);
-  if (config == RLK_TREE_CFG_VALU)
-    return launch_tree<false>(A, B, out, ldc, M, N, K, depth, (unsigned)tiles, tiles_m, 0, stream);
-  if (config == RLK_TREE_CFG_AUTO || config == RLK_TREE_CFG_MFMA_F32) {
-    // 16-byte chunks: every leaf begins and ends on a multiple of 8 (all leaves are K >> depth
-    // long when that divides), rows contiguous in K and 16-byte aligned.
-    const bool leaves_whole = depth <= 20 && K % (8 << depth) == 0;
-    auto chunked = [&](const MatView& v) {
-      return leaves_whole && v.k_stride == 1 && v.row_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0;
-    };
-    const int fast = (chunked(A) ? 1 : 0) | (chunked(B) ? 2 : 0);
-    return launch_tree<true>(A, B, out, ldc, M, N, K, depth, (unsigned)tiles, tiles_m, fast, stream);
+  // Register slots for 7 levels (K <= 4096), 10 (K <= 32768) or 20: the fewer, the more waves per SIMD.
+  if (config == RLK_TREE_CFG_VALU) {
+    if (depth <= 7) launch_valu<7>(A, B, out, ldc, M, N, K, tiles, tiles_m, stream);
+    else if (depth <= 10) launch_valu<10>(A, B, out, ldc, M, N, K, tiles, tiles_m, stream);
+    else launch_valu<20>(A, B, out, ldc, M, N, K, tiles, tiles_m, stream);
+    return hipGetLastError();
   }
-  return hipErrorInvalidValue;
+  if (config != RLK_TREE_CFG_AUTO && config != RLK_TREE_CFG_MFMA_F32) return hipErrorInvalidValue;
+  // 16-byte chunks: every leaf begins and ends on a multiple of 8 (all leaves are K >> depth long
+  // when that divides), rows contiguous in K and 16-byte aligned. Uniform tree: 2^depth divides K.
+  const bool leaves_whole = K % (8 << depth) == 0;
+  auto chunked = [&](const MatView& v) {
+    return leaves_whole && v.k_stride == 1 && v.row_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0;
+  };
+  const bool uniform = depth >= 1 && K % (1 << depth) == 0;
+  const int fast = (chunked(A) ? 1 : 0) | (chunked(B) ? 2 : 0) | (uniform ? 4 : 0);
+  if (depth <= 7) launch_wide<7>(A, B, out, ldc, M, N, K, tiles, tiles_m, fast, stream);
+  else if (depth <= 10) launch_wide<10>(A, B, out, ldc, M, N, K, tiles, tiles_m, fast, stream);
+  else launch_wide<20>(A, B, out, ldc, M, N, K, tiles, tiles_m, fast, stream);
+  return hipGetLastError();
 }
 
 }  // namespace rlk

@@ -147,7 +147,7 @@ def test_tree_special_values(gemm, oracle):
 
 
 def test_both_leaf_loops_compute_the_same_bits(oracle):
-    # The fp32 matrix-pipe leaf (one v_mfma_f32_32x32x1 per k) against the vector-ALU leaf (one
+    # The fp32 matrix-pipe leaf (one v_mfma_f32_16x16x1 per k) against the vector-ALU leaf (one
     # v_fma_f32 per term): every shape of the oracle test, special values (signed zeros, bf16
     # denormals whose products are fp32 denormals, the largest finite values), strided operands.
     from rl_engine import _C
