@@ -288,7 +288,11 @@ __global__ __launch_bounds__(kTreeWideThreads, MAXD <= 10 ? 4 : 2) void det_gemm
   // Staging roles. Chunked operand (bit 0 of `fast`: A, bit 1: B): thread t holds chunk t % 4 of
   // row t / 4 (B: 128 rows, all threads; A: 64 rows, threads 0..255). Element-wise operand:
   // k = t % 32, rows t / 32 + 16 j, two bf16 per register.
+  // Row-contiguous operand (K-major; bit 3: A, bit 4: B; rows a multiple of 8): thread t holds the
+  // 16-byte chunk of eight rows at one k: A rows 8 (t % 8) ..., k = t / 8 (threads 0..255); B rows
+  // 8 (t % 16) ..., k = t / 16.
   const bool a_fast = fast & 1, b_fast = fast & 2;
+  const bool a_rows8 = fast & 8, b_rows8 = fast & 16;
   const int chunk_row = tid >> 2, chunk = tid & 3;
   const int load_k = tid & 31, load_row = tid >> 5;
   uint32_t held[8];  // [0, 4): A, [4, 8): B
@@ -299,6 +303,13 @@ __global__ __launch_bounds__(kTreeWideThreads, MAXD <= 10 ? 4 : 2) void det_gemm
       if (tid < 256) {
         const int row = chunk_row < a_last ? chunk_row : a_last;
         const u32x4_t v = *reinterpret_cast<const u32x4_t*>(a_tile + (int64_t)row * A.row_stride + kc);
+        held[0] = v[0]; held[1] = v[1]; held[2] = v[2]; held[3] = v[3];
+      }
+    } else if (a_rows8) {
+      if (tid < 256) {
+        const int kk = lo + (tid >> 3) < K ? lo + (tid >> 3) : K - 1;
+        const int row = 8 * (tid & 7) <= a_last ? 8 * (tid & 7) : 0;  // a group past the edge is not stored
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(a_tile + (int64_t)kk * A.k_stride + row);
         held[0] = v[0]; held[1] = v[1]; held[2] = v[2]; held[3] = v[3];
       }
     } else {
@@ -314,6 +325,11 @@ __global__ __launch_bounds__(kTreeWideThreads, MAXD <= 10 ? 4 : 2) void det_gemm
     if (b_fast) {
       const int row = chunk_row < b_last ? chunk_row : b_last;
       const u32x4_t v = *reinterpret_cast<const u32x4_t*>(b_tile + (int64_t)row * B.row_stride + kc);
+      held[4] = v[0]; held[5] = v[1]; held[6] = v[2]; held[7] = v[3];
+    } else if (b_rows8) {
+      const int kk = lo + (tid >> 4) < K ? lo + (tid >> 4) : K - 1;
+      const int row = 8 * (tid & 15) <= b_last ? 8 * (tid & 15) : 0;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(b_tile + (int64_t)kk * B.k_stride + row);
       held[4] = v[0]; held[5] = v[1]; held[6] = v[2]; held[7] = v[3];
     } else {
       const bf16_bits* b_col = b_tile + (int64_t)k * B.k_stride;
@@ -333,13 +349,27 @@ __global__ __launch_bounds__(kTreeWideThreads, MAXD <= 10 ? 4 : 2) void det_gemm
     *reinterpret_cast<u32x4_t*>(row + 32 * chunk) = u32x4_t{lo_f32(v[0]), hi_f32(v[0]), lo_f32(v[1]), hi_f32(v[1])};
     *reinterpret_cast<u32x4_t*>(row + 32 * chunk + 16) = u32x4_t{lo_f32(v[2]), hi_f32(v[2]), lo_f32(v[3]), hi_f32(v[3])};
   };
+  // eight rows of one k: element i of the chunk goes to row first + i, column k
+  auto deposit_rows8 = [&](char* stage_rows, int first, int k, const uint32_t* v) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      char* at = stage_rows + (first + i) * kRowBytes;
+      if constexpr (F32_STAGE) {
+        *reinterpret_cast<uint32_t*>(at + 4 * k) = (i & 1) ? hi_f32(v[i / 2]) : lo_f32(v[i / 2]);
+      } else {
+        *reinterpret_cast<bf16_bits*>(at + 2 * k) = (bf16_bits)((v[i / 2] >> (16 * (i & 1))) & 0xffffu);
+      }
+    }
+  };
   auto deposit = [&](int buf) {
     char* as = stage_bytes[buf];
     char* bs = as + kTreeBM * kRowBytes;
+    if (a_rows8 && tid < 256) deposit_rows8(as, 8 * (tid & 7), tid >> 3, held);
+    if (b_rows8) deposit_rows8(bs, 8 * (tid & 15), tid >> 4, held + 4);
     if constexpr (F32_STAGE) {
       if (a_fast) {
         if (tid < 256) deposit_chunk(as + chunk_row * kRowBytes, held);
-      } else {
+      } else if (!a_rows8) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           *reinterpret_cast<uint32_t*>(as + (load_row + 16 * j) * kRowBytes + 4 * load_k) =
@@ -347,7 +377,7 @@ __global__ __launch_bounds__(kTreeWideThreads, MAXD <= 10 ? 4 : 2) void det_gemm
       }
       if (b_fast) {
         deposit_chunk(bs + chunk_row * kRowBytes, held + 4);
-      } else {
+      } else if (!b_rows8) {
 #pragma unroll
         for (int j = 0; j < 8; ++j)
           *reinterpret_cast<uint32_t*>(bs + (load_row + 16 * j) * kRowBytes + 4 * load_k) =
@@ -357,7 +387,7 @@ __global__ __launch_bounds__(kTreeWideThreads, MAXD <= 10 ? 4 : 2) void det_gemm
       if (a_fast) {
         if (tid < 256)
           *reinterpret_cast<u32x4_t*>(as + chunk_row * kRowBytes + 16 * chunk) = u32x4_t{held[0], held[1], held[2], held[3]};
-      } else {
+      } else if (!a_rows8) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           *reinterpret_cast<bf16_bits*>(as + (load_row + 16 * j) * kRowBytes + 2 * load_k) =
@@ -365,7 +395,7 @@ __global__ __launch_bounds__(kTreeWideThreads, MAXD <= 10 ? 4 : 2) void det_gemm
       }
       if (b_fast) {
         *reinterpret_cast<u32x4_t*>(bs + chunk_row * kRowBytes + 16 * chunk) = u32x4_t{held[4], held[5], held[6], held[7]};
-      } else {
+      } else if (!b_rows8) {
 #pragma unroll
         for (int j = 0; j < 8; ++j)
           *reinterpret_cast<bf16_bits*>(bs + (load_row + 16 * j) * kRowBytes + 2 * load_k) =
@@ -582,7 +612,14 @@ hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int
     return leaves_whole && v.k_stride == 1 && v.row_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0;
   };
   const bool uniform = depth >= 1 && K % (1 << depth) == 0;
-  const int fast = (chunked(A) ? 1 : 0) | (chunked(B) ? 2 : 0) | (uniform ? 4 : 0);
+  // Row-contiguous (K-major) operand: 16-byte chunks of eight rows at one k.
+  auto rows8 = [&](const MatView& v, int rows) {
+    return v.row_stride == 1 && rows % 8 == 0 && v.k_stride >= rows && v.k_stride % 8 == 0 &&
+           (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0;
+  };
+  const bool a_chunked = chunked(A), b_chunked = chunked(B);
+  const int fast = (a_chunked ? 1 : 0) | (b_chunked ? 2 : 0) | (uniform ? 4 : 0) |
+                   (!a_chunked && rows8(A, M) ? 8 : 0) | (!b_chunked && rows8(B, N) ? 16 : 0);
   if (depth <= 7) launch_wide<7>(A, B, out, ldc, M, N, K, tiles, tiles_m, fast, stream);
   else if (depth <= 10) launch_wide<10>(A, B, out, ldc, M, N, K, tiles, tiles_m, fast, stream);
   else launch_wide<20>(A, B, out, ldc, M, N, K, tiles, tiles_m, fast, stream);
