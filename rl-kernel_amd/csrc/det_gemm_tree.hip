@@ -256,10 +256,11 @@ __global__ __launch_bounds__(kTreeThreads, MAXD <= 10 ? 2 : 1) void det_gemm_tre
 
 // The matrix-pipe leaf with eight waves per tile: a wave owns 32 rows x 32 columns (the four
 // 16 x 16 blocks of v_mfma_f32_16x16x1_4b_f32), 16 accumulators and 8 packed tree registers per
-// level per lane, so four waves fit on a SIMD and one wave's rounding and tree adds run under the
-// matrix instructions of the others. Operands are converted to fp32 once, on their way into LDS
-// ([row][k], 144-byte rows: a lane's 16-byte read of its own row is conflict free), so a k step
-// needs no vector instruction besides the MFMA.
+// level per lane, so four waves fit on a SIMD. Measured, vector instructions do not run under this
+// matrix instruction (matrix-pipe busy cycles and vector issue cycles add up to the kernel's time),
+// so what the kernel saves is vector instructions: operands are converted to fp32 once, on their
+// way into LDS ([row][k], 144-byte rows: a lane's 16-byte read of its own row is conflict free),
+// and a k step needs none besides the MFMA.
 constexpr int kTreeWideThreads = 512;
 constexpr int kTreeWideRowBytes = 4 * kTreeLeaf + 16;
 constexpr int kTreeWideRowBytesBf16 = 2 * kTreeLeaf + 16;
