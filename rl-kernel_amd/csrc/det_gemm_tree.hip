@@ -569,6 +569,114 @@ __global__ __launch_bounds__(kTreeWideThreads, MAXD <= 10 ? 4 : 2) void det_gemm
   }
 }
 
+// Up to 16 rows of A (decode): the weight must stream at memory rate, and one chain per output
+// is too little parallelism (N lanes in all). The contract's own tree supplies more: the 16 nodes
+// at depth 4 are independent, so a workgroup of 16 waves takes 64 columns, wave w evaluates node w
+// (a sixteenth of K) for them, one column per lane and MR fp32 chains per lane (plain v_fma_f32,
+// A values uniform across the wave), and wave 0 folds the 16 bf16 nodes in tree order. Needs
+// a uniform tree (every leaf K >> depth long, a multiple of 8), K-contiguous 16-byte aligned rows.
+constexpr int kTreeSkinnySplit = 4;                       // depth of the nodes the waves take
+constexpr int kTreeSkinnyWaves = 1 << kTreeSkinnySplit;   // 16
+constexpr int kTreeSkinnyLevels = 8;                      // tree levels below a wave's node
+
+template <int MR>
+__global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_skinny_kernel(
+    MatView A, MatView B, bf16_bits* __restrict__ C, int64_t ldc, int M, int N, int K, int depth) {
+  static_assert(MR % 2 == 0 && MR <= 16, "rows are packed in pairs");
+  constexpr int PR = MR / 2;
+  __shared__ uint32_t nodes[kTreeSkinnyWaves][PR][64];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int col = blockIdx.x * 64 + lane;
+  const bf16_bits* wrow = B.ptr + (int64_t)(col < N ? col : N - 1) * B.row_stride;
+  const int len = K >> depth;                              // leaf length, 8 ... 32, a multiple of 8
+  const int leaves = 1 << (depth - kTreeSkinnySplit);      // leaves under this wave's node
+  const int first = wave * leaves * len;                   // node w covers leaves [w * leaves, (w + 1) * leaves)
+  const bf16_bits* arow[MR];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) arow[m] = A.ptr + (int64_t)(m < M ? m : M - 1) * A.row_stride;
+
+  uint32_t slot[kTreeSkinnyLevels][PR];  // slot[l]: finished left child l levels above the leaves
+  uint32_t cur[PR];
+  u32x4_t w_now[4], w_next[4];
+  auto fetch = [&](int lo, u32x4_t (&w)[4]) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      if (8 * c < len) w[c] = *reinterpret_cast<const u32x4_t*>(wrow + lo + 8 * c);
+  };
+  fetch(first, w_now);
+  for (int i = 0; i < leaves; ++i) {
+    const int lo = first + i * len;
+    if (i + 1 < leaves) fetch(lo + len, w_next);
+    float acc[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[m] = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      if (8 * c < len) {
+        u32x4_t a8[MR];  // eight k of every row of A: the same address in every lane
+#pragma unroll
+        for (int m = 0; m < MR; ++m) a8[m] = *reinterpret_cast<const u32x4_t*>(arow[m] + lo + 8 * c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const uint32_t wb = w_now[c][e >> 1];
+          const float b = __uint_as_float((e & 1) ? (wb & 0xffff0000u) : (wb << 16));
+#pragma unroll
+          for (int m = 0; m < MR; ++m) {
+            const uint32_t ab = a8[m][e >> 1];
+            const float a = __uint_as_float((e & 1) ? (ab & 0xffff0000u) : (ab << 16));
+            acc[m] = __builtin_fmaf(a, b, acc[m]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < PR; ++r) cur[r] = pack_bf16x2(acc[2 * r], acc[2 * r + 1]);
+    // Leaf i closes one node per trailing one bit of i; then it waits at the level of its lowest zero bit.
+    int level = 0;
+    for (int j = i; j & 1; j >>= 1, ++level) {
+#pragma unroll
+      for (int l = 0; l < kTreeSkinnyLevels; ++l) {
+        if (l == level) {
+#pragma unroll
+          for (int r = 0; r < PR; ++r) cur[r] = bf16x2_add(slot[l][r], cur[r]);
+        }
+      }
+    }
+    if (i + 1 < leaves) {
+#pragma unroll
+      for (int l = 0; l < kTreeSkinnyLevels; ++l) {
+        if (l == level) {
+#pragma unroll
+          for (int r = 0; r < PR; ++r) slot[l][r] = cur[r];
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c) w_now[c] = w_next[c];
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < PR; ++r) nodes[wave][r][lane] = cur[r];
+  __syncthreads();
+  if (wave != 0) return;
+  // nodes 0..15 left to right at depth 4: pairs, then pairs of pairs, ... up to the root
+#pragma unroll
+  for (int r = 0; r < PR; ++r) {
+    uint32_t v[kTreeSkinnyWaves];
+#pragma unroll
+    for (int w = 0; w < kTreeSkinnyWaves; ++w) v[w] = nodes[w][r][lane];
+#pragma unroll
+    for (int width = kTreeSkinnyWaves / 2; width >= 1; width /= 2)
+#pragma unroll
+      for (int w = 0; w < width; ++w) v[w] = bf16x2_add(v[2 * w], v[2 * w + 1]);
+    if (col < N) {
+      if (2 * r < M) C[(int64_t)(2 * r) * ldc + col] = (bf16_bits)(v[0] & 0xffffu);
+      if (2 * r + 1 < M) C[(int64_t)(2 * r + 1) * ldc + col] = (bf16_bits)(v[0] >> 16);
+    }
+  }
+}
+
 int det_gemm_tree_max_k() { return kTreeLeaf << 20; }
 
 template <int MAXD>
@@ -605,7 +713,8 @@ hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int
     else launch_valu<20>(A, B, out, ldc, M, N, K, tiles, tiles_m, stream);
     return hipGetLastError();
   }
-  if (config != RLK_TREE_CFG_AUTO && config != RLK_TREE_CFG_MFMA_F32) return hipErrorInvalidValue;
+  if (config != RLK_TREE_CFG_AUTO && config != RLK_TREE_CFG_MFMA_F32 && config != RLK_TREE_CFG_SKINNY)
+    return hipErrorInvalidValue;
   // 16-byte chunks: every leaf begins and ends on a multiple of 8 (all leaves are K >> depth long
   // when that divides), rows contiguous in K and 16-byte aligned. Uniform tree: 2^depth divides K.
   const bool leaves_whole = K % (8 << depth) == 0;
@@ -619,6 +728,20 @@ hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int
            (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0;
   };
   const bool a_chunked = chunked(A), b_chunked = chunked(B);
+  // Up to 16 rows: the kernel that gives each of the 16 depth-4 nodes to a wave of its own.
+  const bool skinny_ok = M <= 16 && a_chunked && b_chunked && depth >= kTreeSkinnySplit &&
+                         depth - kTreeSkinnySplit <= kTreeSkinnyLevels;
+  if (config == RLK_TREE_CFG_SKINNY && !skinny_ok) return hipErrorInvalidValue;
+  if (skinny_ok && config != RLK_TREE_CFG_MFMA_F32) {
+    const dim3 grid((unsigned)((N + 63) / 64)), block(64 * kTreeSkinnyWaves);
+    if (M <= 4)
+      hipLaunchKernelGGL(det_gemm_tree_skinny_kernel<4>, grid, block, 0, stream, A, B, out, ldc, M, N, K, depth);
+    else if (M <= 8)
+      hipLaunchKernelGGL(det_gemm_tree_skinny_kernel<8>, grid, block, 0, stream, A, B, out, ldc, M, N, K, depth);
+    else
+      hipLaunchKernelGGL(det_gemm_tree_skinny_kernel<16>, grid, block, 0, stream, A, B, out, ldc, M, N, K, depth);
+    return hipGetLastError();
+  }
   const int fast = (a_chunked ? 1 : 0) | (b_chunked ? 2 : 0) | (uniform ? 4 : 0) |
                    (!a_chunked && rows8(A, M) ? 8 : 0) | (!b_chunked && rows8(B, N) ? 16 : 0);
   if (depth <= 7) launch_wide<7>(A, B, out, ldc, M, N, K, tiles, tiles_m, fast, stream);

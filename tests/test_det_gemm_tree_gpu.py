@@ -178,7 +178,35 @@ def test_both_leaf_loops_compute_the_same_bits(oracle):
         want_nan = (want & 0x7FFF) > 0x7F80
         assert np.array_equal(inputs.bits(mfma)[~want_nan], want[~want_nan]), k
     with pytest.raises(ValueError, match="unknown configuration"):
-        run(a_d, w_d.t(), 7)
+        run(a_d, w_d.t(), 9)
+
+
+def test_skinny_kernel_folds_the_depth_4_nodes_to_the_same_bits(oracle):
+    # Up to 16 rows the 16 tree nodes at depth 4 run on 16 waves and are folded in tree order:
+    # the same bits as the one-chain-per-output kernels, for every row count and ragged N.
+    from rl_engine import _C
+
+    def run(a_d, b_kn, config):
+        out = torch.empty((a_d.size(0), b_kn.size(1)), dtype=torch.bfloat16, device=DEV)
+        return _C.gemm_tree_strided(a_d, b_kn, out, config)
+
+    for k in (512, 384, 4096, 6144, 12288, 65536):
+        for m, n in ((1, 64), (3, 100), (4, 257), (7, 64), (8, 130), (13, 96), (16, 320)):
+            a = inputs.randn_bf16(9800 + k + m, m, k).to(DEV)
+            w = inputs.randn_bf16(9801 + k + m, n, k, 0.02).to(DEV)
+            skinny = run(a, w.t(), 3)
+            assert _same_bits(skinny, run(a, w.t(), 1)), (m, k, n)
+            assert _same_bits(skinny, run(a, w.t(), 2)) and _same_bits(skinny, run(a, w.t(), 0)), (m, k, n)
+    a = inputs.randn_bf16(9810, 5, 4096)
+    w = inputs.randn_bf16(9811, 70, 4096, 0.02)
+    assert np.array_equal(inputs.bits(run(a.to(DEV), w.to(DEV).t(), 3)), _oracle_tree(oracle, a, w))
+    # not eligible: more than 16 rows, a tree of fewer than 4 levels, ragged leaves, K-major operand
+    a17 = inputs.randn_bf16(9812, 17, 4096).to(DEV)
+    w_d = w.to(DEV)
+    for bad_a, bad_b in ((a17, w_d.t()), (a17[:4, :256], w_d[:, :256].t()), (a17[:4, :4000], w_d[:, :4000].t()),
+                         (a17[:4], w_d.t().contiguous())):
+        with pytest.raises(ValueError, match="RLK_TREE_CFG_SKINNY needs"):
+            run(bad_a, bad_b, 3)
 
 
 def test_tree_out_argument_empty_shapes_and_errors(gemm):
