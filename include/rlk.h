@@ -122,7 +122,10 @@ typedef enum rlk_tree_config {
   RLK_TREE_CFG_MFMA_F32 = 2, /* one v_mfma_f32_16x16x1_4b_f32 per k (reduction length one: a single fused step) */
   RLK_TREE_CFG_SKINNY = 3,   /* up to 16 rows: the 16 tree nodes at depth 4 on 16 waves, folded in tree order;
                                 needs K-contiguous aligned operands and equal leaves, else invalid argument */
-  RLK_TREE_CFG_COUNT = 4
+  RLK_TREE_CFG_NODES = 4,    /* any row count: 16 rows x 64 columns per workgroup, the 16 depth-4 nodes on 16 waves
+                                (fp32 MFMA, operands from memory to registers); same eligibility as SKINNY but
+                                trees of 4 to 10 levels */
+  RLK_TREE_CFG_COUNT = 5
 } rlk_tree_config;
 
 /* rlk_det_gemm_tree_bf16 with an explicit leaf loop (rlk_tree_config). */

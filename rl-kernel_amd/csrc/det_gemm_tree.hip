@@ -677,6 +677,113 @@ __global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_skinny_ke
   }
 }
 
+// The same split for more rows, on the matrix pipe: a workgroup of 16 waves takes 16 rows x 64
+// columns, wave w evaluates node w at depth 4 with one v_mfma_f32_16x16x1_4b_f32 per k (the row
+// operand of block 0 broadcast to the four 16-column blocks), operands straight from global
+// memory into registers (a lane streams the weight row of its own column and the A row
+// lane % 16), no LDS stage and no barrier until the 16 nodes are folded. 16 x the workgroups of
+// the tiled kernel: for row counts whose tiles do not fill the chip.
+constexpr int kTreeNodeLevels = 6;  // tree levels below a wave's node (K <= 32768)
+
+__global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_nodes_kernel(
+    MatView A, MatView B, bf16_bits* __restrict__ C, int64_t ldc, int M, int N, int K, int depth) {
+  __shared__ uint32_t nodes[kTreeSkinnyWaves][8][64];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n0 = blockIdx.x * 64, m0 = blockIdx.y * 16;
+  const int col = n0 + lane;
+  const int a_index = m0 + (lane & 15);
+  const bf16_bits* wrow = B.ptr + (int64_t)(col < N ? col : N - 1) * B.row_stride;
+  const bf16_bits* arow = A.ptr + (int64_t)(a_index < M ? a_index : M - 1) * A.row_stride;
+  const int len = K >> depth;                          // leaf length, 8 ... 32, a multiple of 8
+  const int leaves = 1 << (depth - kTreeSkinnySplit);  // leaves under this wave's node
+  const int first = wave * leaves * len;
+
+  uint32_t slot[kTreeNodeLevels][8];
+  uint32_t cur[8];
+  u32x4_t w_now[4], w_next[4], a_now[4], a_next[4];
+  auto fetch = [&](int lo, u32x4_t (&w)[4], u32x4_t (&a)[4]) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      if (8 * c < len) {
+        w[c] = *reinterpret_cast<const u32x4_t*>(wrow + lo + 8 * c);
+        a[c] = *reinterpret_cast<const u32x4_t*>(arow + lo + 8 * c);
+      }
+    }
+  };
+  fetch(first, w_now, a_now);
+  for (int i = 0; i < leaves; ++i) {
+    const int lo = first + i * len;
+    if (i + 1 < leaves) fetch(lo + len, w_next, a_next);
+    f32x16_t acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      if (8 * c < len) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const uint32_t wb = w_now[c][e >> 1], ab = a_now[c][e >> 1];
+          const float b = __uint_as_float((e & 1) ? (wb & 0xffff0000u) : (wb << 16));
+          const float a = __uint_as_float((e & 1) ? (ab & 0xffff0000u) : (ab << 16));
+          acc = __builtin_amdgcn_mfma_f32_16x16x1f32(a, b, acc, 2, 0, 0);
+        }
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 8; ++q) cur[q] = pack_bf16x2(acc[2 * q], acc[2 * q + 1]);
+    int level = 0;
+    for (int j = i; j & 1; j >>= 1, ++level) {
+#pragma unroll
+      for (int l = 0; l < kTreeNodeLevels; ++l) {
+        if (l == level) {
+#pragma unroll
+          for (int r = 0; r < 8; ++r) cur[r] = bf16x2_add(slot[l][r], cur[r]);
+        }
+      }
+    }
+    if (i + 1 < leaves) {
+#pragma unroll
+      for (int l = 0; l < kTreeNodeLevels; ++l) {
+        if (l == level) {
+#pragma unroll
+          for (int r = 0; r < 8; ++r) slot[l][r] = cur[r];
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        w_now[c] = w_next[c];
+        a_now[c] = a_next[c];
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 8; ++r) nodes[wave][r][lane] = cur[r];
+  __syncthreads();
+  if (wave != 0) return;
+  // Accumulator r: block r / 4 (16 columns each); row 4 (lane / 16) + r % 4, column lane % 16.
+  // cur[q] packs accumulators 2 q, 2 q + 1 (two consecutive rows of one column).
+  const int out_col = n0 + (lane & 15);
+  const int out_row = m0 + 4 * (lane >> 4);
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    uint32_t v[kTreeSkinnyWaves];
+#pragma unroll
+    for (int w = 0; w < kTreeSkinnyWaves; ++w) v[w] = nodes[w][q][lane];
+#pragma unroll
+    for (int width = kTreeSkinnyWaves / 2; width >= 1; width /= 2)
+#pragma unroll
+      for (int w = 0; w < width; ++w) v[w] = bf16x2_add(v[2 * w], v[2 * w + 1]);
+    const int c = out_col + 16 * (q >> 1);
+    const int r = out_row + 2 * (q & 1);
+    if (c < N) {
+      if (r < M) C[(int64_t)r * ldc + c] = (bf16_bits)(v[0] & 0xffffu);
+      if (r + 1 < M) C[(int64_t)(r + 1) * ldc + c] = (bf16_bits)(v[0] >> 16);
+    }
+  }
+}
+
 int det_gemm_tree_max_k() { return kTreeLeaf << 20; }
 
 template <int MAXD>
@@ -713,7 +820,8 @@ hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int
     else launch_valu<20>(A, B, out, ldc, M, N, K, tiles, tiles_m, stream);
     return hipGetLastError();
   }
-  if (config != RLK_TREE_CFG_AUTO && config != RLK_TREE_CFG_MFMA_F32 && config != RLK_TREE_CFG_SKINNY)
+  if (config != RLK_TREE_CFG_AUTO && config != RLK_TREE_CFG_MFMA_F32 && config != RLK_TREE_CFG_SKINNY &&
+      config != RLK_TREE_CFG_NODES)
     return hipErrorInvalidValue;
   // 16-byte chunks: every leaf begins and ends on a multiple of 8 (all leaves are K >> depth long
   // when that divides), rows contiguous in K and 16-byte aligned. Uniform tree: 2^depth divides K.
@@ -732,7 +840,26 @@ hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int
   const bool skinny_ok = M <= 16 && a_chunked && b_chunked && depth >= kTreeSkinnySplit &&
                          depth - kTreeSkinnySplit <= kTreeSkinnyLevels;
   if (config == RLK_TREE_CFG_SKINNY && !skinny_ok) return hipErrorInvalidValue;
-  if (skinny_ok && config != RLK_TREE_CFG_MFMA_F32) {
+  const bool nodes_ok = a_chunked && b_chunked && depth >= kTreeSkinnySplit &&
+                        depth - kTreeSkinnySplit <= kTreeNodeLevels && (M + 15) / 16 <= 65535;
+  if (config == RLK_TREE_CFG_NODES && !nodes_ok) return hipErrorInvalidValue;
+  if (config == RLK_TREE_CFG_AUTO && nodes_ok && M > 8) {
+    // Node-per-wave kernel against the tiled one (fitted to the Qwen3-8B projections at 8 ... 4096 rows):
+    // the first runs at about 40 TFLOP/s on rows padded to 16 whatever the grid; the second needs about
+    // 2.25 us per leaf per round of 512 tiles and reaches about 80 TFLOP/s once the chip is full.
+    const double work = 2.0 * N * (double)K;
+    const double t_nodes = work * (16.0 * ((M + 15) / 16)) / 40e12;
+    const double rounds = (double)((tiles64 + 511) / 512);
+    const double t_tiled_latency = rounds * (double)(1 << depth) * 2.25e-6;
+    const double t_tiled_rate = work * M / 80e12;
+    if (t_nodes < (t_tiled_latency > t_tiled_rate ? t_tiled_latency : t_tiled_rate)) config = RLK_TREE_CFG_NODES;
+  }
+  if (config == RLK_TREE_CFG_NODES) {
+    hipLaunchKernelGGL(det_gemm_tree_nodes_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((M + 15) / 16)),
+                       dim3(64 * kTreeSkinnyWaves), 0, stream, A, B, out, ldc, M, N, K, depth);
+    return hipGetLastError();
+  }
+  if (skinny_ok && (config == RLK_TREE_CFG_SKINNY || (config == RLK_TREE_CFG_AUTO && (M <= 8 || !nodes_ok)))) {
     const dim3 grid((unsigned)((N + 63) / 64)), block(64 * kTreeSkinnyWaves);
     if (M <= 4)
       hipLaunchKernelGGL(det_gemm_tree_skinny_kernel<4>, grid, block, 0, stream, A, B, out, ldc, M, N, K, depth);

@@ -135,10 +135,11 @@ int rlk_det_gemm_tree_bf16_config(const void* a, int64_t a_row_stride, int64_t a
   MatView A{reinterpret_cast<const bf16_bits*>(a), a_row_stride, a_k_stride, M};
   MatView B{reinterpret_cast<const bf16_bits*>(b), b_n_stride, b_k_stride, N};
   hipError_t err = det_gemm_tree_launch(A, B, c, ldc, M, N, K, config, s);
-  if (err == hipErrorInvalidValue && config == RLK_TREE_CFG_SKINNY) {
+  if (err == hipErrorInvalidValue && (config == RLK_TREE_CFG_SKINNY || config == RLK_TREE_CFG_NODES)) {
     set_last_error(
         "rlk_det_gemm_tree_bf16: RLK_TREE_CFG_SKINNY needs M <= 16, K-contiguous 16-byte aligned operands and a tree "
-        "of 4 to 12 levels whose leaves are equally long and a multiple of 8 (M=%d K=%d)", M, K);
+        "of 4 to 12 levels whose leaves are equally long and a multiple of 8; RLK_TREE_CFG_NODES the same with any M "
+        "and 4 to 10 levels (M=%d K=%d)", M, K);
     return RLK_ERR_INVALID_ARGUMENT;
   }
   return err == hipSuccess ? RLK_OK : device_error("rlk_det_gemm_tree_bf16", err);

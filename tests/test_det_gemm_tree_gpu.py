@@ -209,6 +209,35 @@ def test_skinny_kernel_folds_the_depth_4_nodes_to_the_same_bits(oracle):
             run(bad_a, bad_b, 3)
 
 
+def test_node_per_wave_kernel_computes_the_same_bits(oracle):
+    # 16 rows x 64 columns per workgroup, one depth-4 node per wave on the fp32 matrix pipe: any row
+    # count, ragged M and N, against the vector-ALU kernel; one case against the oracle.
+    from rl_engine import _C
+
+    def run(a_d, b_kn, config):
+        out = torch.empty((a_d.size(0), b_kn.size(1)), dtype=torch.bfloat16, device=DEV)
+        return _C.gemm_tree_strided(a_d, b_kn, out, config)
+
+    for k in (512, 384, 4096, 6144, 12288, 32768):
+        for m, n in ((1, 64), (16, 100), (17, 257), (50, 64), (64, 130), (200, 96), (333, 320)):
+            a = inputs.randn_bf16(9900 + k + m, m, k).to(DEV)
+            w = inputs.randn_bf16(9901 + k + m, n, k, 0.02).to(DEV)
+            assert _same_bits(run(a, w.t(), 4), run(a, w.t(), 1)), (m, k, n)
+    a = inputs.randn_bf16(9910, 37, 4096)
+    w = inputs.randn_bf16(9911, 70, 4096, 0.02)
+    assert np.array_equal(inputs.bits(run(a.to(DEV), w.to(DEV).t(), 4)), _oracle_tree(oracle, a, w))
+    finite = np.array([0x0000, 0x8000, 0x3F80, 0xBF80, 0x0080, 0x8080, 0x0001, 0x8001, 0x7F7F, 0xFF7F, 0x4000, 0x3F00], dtype=np.uint16)
+    rng = np.random.default_rng(9912)
+    a_bits, w_bits = rng.choice(finite, size=(40, 1024)), rng.choice(finite[:7], size=(70, 1024))
+    a_d, w_d = inputs.from_bits(a_bits, DEV), inputs.from_bits(w_bits, DEV)
+    got, want = run(a_d, w_d.t(), 4), run(a_d, w_d.t(), 1)
+    nan = torch.isnan(want.float())
+    assert torch.equal(nan, torch.isnan(got.float()))
+    assert torch.equal(got.view(torch.int16)[~nan], want.view(torch.int16)[~nan])
+    with pytest.raises(ValueError, match="RLK_TREE_CFG_NODES"):
+        run(a_d[:, :256], w_d[:, :256].t(), 4)  # a tree of three levels
+
+
 def test_tree_out_argument_empty_shapes_and_errors(gemm):
     a = inputs.randn_bf16(9600, 20, 256).to(DEV)
     w = inputs.randn_bf16(9601, 48, 256, 0.02).to(DEV)
