@@ -84,8 +84,9 @@ def gemm_strided(
 def gemm_tree_strided(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor, config: int = 0) -> torch.Tensor:
     """``out[M,N] = a[M,K] @ b[K,N]`` under the k-tree contract, arbitrary non-negative strides.
 
-    ``config``: 0 picks the leaf loop, 1 forces the vector-ALU loop, 2 the fp32 matrix-pipe loop
-    (``rlk_tree_config``; the same bits either way)."""
+    ``config`` (``rlk_tree_config``; the same bits whichever runs): 0 picks the kernel, 1 forces the
+    vector-ALU tiled kernel, 2 the fp32 matrix-pipe tiled kernel, 3 / 4 the node-per-wave kernels for up
+    to 16 rows / any row count (``ValueError`` when the operands are not eligible)."""
     m, k = a.shape
     n = b.shape[1]
     if m == 0 or n == 0:
