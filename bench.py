@@ -58,7 +58,7 @@ def _parse():
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-T table")
     ap.add_argument("--rotate-weights", action="store_true",
                     help="gate_up_tN / down_tN legs: launch over copies of the weight (~1.3 GB in rotation) so that it is read from HBM")
-    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|gate_up_tN|down_tN|logp|logp_decode|logp_mid|logp_bwd|from_logits|ffn|tree|tree_down|copy|power (used for profiling)")
+    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|gate_up_tN|down_tN|logp|logp_decode|logp_mid|logp_bwd|from_logits|ffn|tree|tree_down|tree_decode|copy|power (used for profiling)")
     return ap.parse_args()
 
 
@@ -243,6 +243,16 @@ def main() -> int:
                "random_operands": looped(x, w_gu), "zero_operands": looped(torch.zeros_like(x), torch.zeros_like(w_gu))}
         print(json.dumps(res))
         return 0
+    if args.only == "tree_decode":
+        # the k-tree contract at 1, 16 and 64 tokens: the node-per-wave kernels
+        legs = []
+        for ts in (1, 16, 64):
+            for name, act, w, out in (("gate_up", x, w_gu, out_gu), ("down", h, w_d, out_d)):
+                ms = _time_calls(lambda: gemm.tree_gemm(act[:ts], w.t(), out=out[:ts]), args.steps, args.warmup)
+                legs.append({"op": name, "T": ts, "us": round(ms * 1e3, 1),
+                             "weight_gbps": round(w.numel() * 2 / ms * 1e-6, 1)})
+        print(json.dumps({"leg": "tree_decode", "legs": legs, "launches": 6 * (args.steps + args.warmup)}))
+        return 0
     if args.only in ("tree", "tree_down"):
         if args.only == "tree":
             ms = _time_calls(lambda: gemm.tree_gemm(x, w_gu.t(), out=out_gu), args.steps, args.warmup)
@@ -426,6 +436,13 @@ def main() -> int:
                      "frac_of_fp32_mfma_peak": round(flops_d / ms_tree_down * 1e-9 / 157.3, 4)},
             "contract": _lib.load().rlk_det_gemm_tree_contract_id().decode(),
         }
+        decode = []
+        for ts in (1, 16, 64):
+            for name, act, w, out in (("gate_up", x, w_gu, out_gu), ("down", h, w_d, out_d)):
+                ms_t = _time_calls(lambda: gemm.tree_gemm(act[:ts], w.t(), out=out[:ts]), 20, 5)
+                decode.append({"op": name, "T": ts, "us": round(ms_t * 1e3, 1),
+                               "weight_gbps": round(w.numel() * 2 / ms_t * 1e-6, 1)})
+        result["det_gemm_tree"]["decode"] = decode
 
     # ---- fused linear-LogP at T=8192, V=151936
     if not args.no_logp:

@@ -24,7 +24,11 @@
 //     rounding as the fused multiply-add, at twice the vector rate; operands staged in LDS
 //     as fp32, [row][k].
 //
-// A workgroup owns a 64 x 128 output tile. Leaves are visited left to right, the next leaf
+// For few rows (decode) two more kernels split K along the contract's own tree: the 16 nodes at
+// depth 4 are independent, a wave evaluates one of them for a block of outputs, and the 16 bf16
+// nodes are folded in tree order (det_gemm_tree_skinny_kernel, det_gemm_tree_nodes_kernel below).
+//
+// Tiled kernels: a workgroup owns a 64 x 128 output tile. Leaves are visited left to right, the next leaf
 // is fetched while the current one is summed. The tree is evaluated on the
 // fly: a finished node waits in the register slot of its depth until its right sibling is
 // finished, so a thread holds at most one bf16 node per tree level. Which slot is read or
