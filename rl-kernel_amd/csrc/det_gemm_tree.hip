@@ -582,8 +582,11 @@ __global__ __launch_bounds__(kTreeWideThreads, MAXD <= 10 ? 4 : 2) void det_gemm
 constexpr int kTreeSkinnySplit = 4;                       // depth of the nodes the waves take
 constexpr int kTreeSkinnyWaves = 1 << kTreeSkinnySplit;   // 16
 constexpr int kTreeSkinnyLevels = 8;                      // tree levels below a wave's node
+constexpr int kTreeHalvesMaxN = 8192;                     // up to this many columns (and 8 rows) the wave halves split a node
 
-template <int MR>
+// HALVES: the two halves of a wave take the two children of the wave's node (32 nodes at depth 5, 32
+// columns per workgroup) and exchange them through a lane shuffle: twice the workgroups for narrow N.
+template <int MR, bool HALVES>
 __global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_skinny_kernel(
     MatView A, MatView B, bf16_bits* __restrict__ C, int64_t ldc, int M, int N, int K, int depth) {
   static_assert(MR % 2 == 0 && MR <= 16, "rows are packed in pairs");
@@ -592,11 +595,14 @@ __global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_skinny_ke
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int col = blockIdx.x * 64 + lane;
+  constexpr int kCols = HALVES ? 32 : 64;
+  const int col = blockIdx.x * kCols + (lane & (kCols - 1));
+  const int node = HALVES ? 2 * wave + (lane >> 5) : wave;
+  const int node_depth = HALVES ? kTreeSkinnySplit + 1 : kTreeSkinnySplit;
   const bf16_bits* wrow = B.ptr + (int64_t)(col < N ? col : N - 1) * B.row_stride;
   const int len = K >> depth;                              // leaf length, 8 ... 32, a multiple of 8
-  const int leaves = 1 << (depth - kTreeSkinnySplit);      // leaves under this wave's node
-  const int first = wave * leaves * len;                   // node w covers leaves [w * leaves, (w + 1) * leaves)
+  const int leaves = 1 << (depth - node_depth);            // leaves under this lane's node
+  const int first = node * leaves * len;                   // node j covers leaves [j * leaves, (j + 1) * leaves)
   const bf16_bits* arow[MR];
 #pragma unroll
   for (int m = 0; m < MR; ++m) arow[m] = A.ptr + (int64_t)(m < M ? m : M - 1) * A.row_stride;
@@ -660,6 +666,14 @@ __global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_skinny_ke
       for (int c = 0; c < 4; ++c) w_now[c] = w_next[c];
     }
   }
+  if constexpr (HALVES) {
+    // left child in lanes 0..31, right child in lanes 32..63 of the same column
+#pragma unroll
+    for (int r = 0; r < PR; ++r) {
+      const uint32_t other = (uint32_t)__shfl_xor((int)cur[r], 32, 64);
+      cur[r] = lane < 32 ? bf16x2_add(cur[r], other) : bf16x2_add(other, cur[r]);
+    }
+  }
 #pragma unroll
   for (int r = 0; r < PR; ++r) nodes[wave][r][lane] = cur[r];
   __syncthreads();
@@ -674,7 +688,7 @@ __global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_skinny_ke
     for (int width = kTreeSkinnyWaves / 2; width >= 1; width /= 2)
 #pragma unroll
       for (int w = 0; w < width; ++w) v[w] = bf16x2_add(v[2 * w], v[2 * w + 1]);
-    if (col < N) {
+    if (col < N && lane < kCols) {
       if (2 * r < M) C[(int64_t)(2 * r) * ldc + col] = (bf16_bits)(v[0] & 0xffffu);
       if (2 * r + 1 < M) C[(int64_t)(2 * r + 1) * ldc + col] = (bf16_bits)(v[0] >> 16);
     }
@@ -864,13 +878,19 @@ hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int
     return hipGetLastError();
   }
   if (skinny_ok && (config == RLK_TREE_CFG_SKINNY || (config == RLK_TREE_CFG_AUTO && (M <= 8 || !nodes_ok)))) {
-    const dim3 grid((unsigned)((N + 63) / 64)), block(64 * kTreeSkinnyWaves);
-    if (M <= 4)
-      hipLaunchKernelGGL(det_gemm_tree_skinny_kernel<4>, grid, block, 0, stream, A, B, out, ldc, M, N, K, depth);
-    else if (M <= 8)
-      hipLaunchKernelGGL(det_gemm_tree_skinny_kernel<8>, grid, block, 0, stream, A, B, out, ldc, M, N, K, depth);
-    else
-      hipLaunchKernelGGL(det_gemm_tree_skinny_kernel<16>, grid, block, 0, stream, A, B, out, ldc, M, N, K, depth);
+    // Narrow N: 32 columns per workgroup and the wave halves on the two children of a node (down at one
+    // token 78 -> 61 us, o_proj 24 -> 20 us; gate_up 66 -> 73 us, and 16 rows twice as slow: not there).
+    const bool halves = depth > kTreeSkinnySplit && depth - kTreeSkinnySplit - 1 <= kTreeSkinnyLevels && M <= 8 &&
+                        N <= kTreeHalvesMaxN;
+    const dim3 grid((unsigned)(halves ? (N + 31) / 32 : (N + 63) / 64)), block(64 * kTreeSkinnyWaves);
+    auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, block, 0, stream, A, B, out, ldc, M, N, K, depth); };
+    if (M <= 4) {
+      if (halves) launch(det_gemm_tree_skinny_kernel<4, true>); else launch(det_gemm_tree_skinny_kernel<4, false>);
+    } else if (M <= 8) {
+      if (halves) launch(det_gemm_tree_skinny_kernel<8, true>); else launch(det_gemm_tree_skinny_kernel<8, false>);
+    } else {
+      launch(det_gemm_tree_skinny_kernel<16, false>);
+    }
     return hipGetLastError();
   }
   const int fast = (a_chunked ? 1 : 0) | (b_chunked ? 2 : 0) | (uniform ? 4 : 0) |

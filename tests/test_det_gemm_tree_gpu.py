@@ -191,7 +191,7 @@ def test_skinny_kernel_folds_the_depth_4_nodes_to_the_same_bits(oracle):
         return _C.gemm_tree_strided(a_d, b_kn, out, config)
 
     for k in (512, 384, 4096, 6144, 12288, 65536):
-        for m, n in ((1, 64), (3, 100), (4, 257), (7, 64), (8, 130), (13, 96), (16, 320)):
+        for m, n in ((1, 64), (3, 100), (4, 257), (7, 64), (8, 130), (13, 96), (16, 320), (2, 9000), (8, 8200)):  # beyond 8192 columns: whole waves per node
             a = inputs.randn_bf16(9800 + k + m, m, k).to(DEV)
             w = inputs.randn_bf16(9801 + k + m, n, k, 0.02).to(DEV)
             skinny = run(a, w.t(), 3)
