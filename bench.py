@@ -42,10 +42,29 @@ PEAK_HBM_GBPS = 8000.0  # HBM3E
 
 HIDDEN, INTER, VOCAB = 4096, 12288, 151936
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs of this script (profiles/det_gemm_gate_up_T4096_pmc.md), scaled
-# by the same counters read on a plain device copy of known size. None = not measured.
-MEASURED_TRAFFIC_BYTES = {"det_gemm_gate_up_T4096": 1.417e9}  # 1.212 GB fetched + 0.205 GB written
+# Steps launched before the caller's --warmup, always: after idle the part boosts, over-throttles around
+# the sixth launch and settles after about thirty, so a short warm-up would time that transient.
+CONDITIONING_STEPS = 40  # 80 kernel launches
+
+# HBM bytes per launch of the dominant kernel come from a tracked record of two rocprofv3 --pmc runs
+# (FETCH_SIZE, then WRITE_SIZE) of `bench.py --only gate_up`, each scaled by what the same counter reads on
+# the plain copy kernel of `bench.py --only copy`; the record names the commit it was measured on.
+TRAFFIC_RECORD = ROOT / "profiles" / "det_gemm_gate_up_T4096_traffic.txt"
+
+
+def _measured_traffic() -> dict:
+    """`key: value` lines of the traffic record -> {"bytes": float | None, "commit": str | None}."""
+    out = {"bytes": None, "commit": None}
+    try:
+        for line in TRAFFIC_RECORD.read_text().splitlines():
+            key, _, value = line.partition(":")
+            if key.strip() == "traffic_bytes_per_launch":
+                out["bytes"] = float(value)
+            elif key.strip() == "measured_on_commit":
+                out["commit"] = value.strip()
+    except (OSError, ValueError):
+        pass
+    return out
 
 
 def _parse():
@@ -295,6 +314,8 @@ def main() -> int:
     flops_d = 2.0 * T * HIDDEN * INTER
 
     # ---- timed region: exactly `steps` steps, synchronised on both sides
+    for _ in range(CONDITIONING_STEPS):  # fixed conditioning phase, then the caller's warm-up
+        step()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -309,6 +330,7 @@ def main() -> int:
     ms_gu = _time_calls(gate_up, args.steps, 5)
     ms_d = _time_calls(down, args.steps, 5)
     achieved = flops_gu / ms_gu * 1e-9
+    traffic = _measured_traffic()
     roofline = {
         "kernel": "det_gemm_kernel<256x256 tile, 8 waves> on gate_up [4096x4096]x[24576x4096]^T",
         "bound": "mfma",
@@ -318,7 +340,8 @@ def main() -> int:
         "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
         "ms_per_launch": round(ms_gu, 4),
         "flops_per_launch": flops_gu,
-        "traffic": MEASURED_TRAFFIC_BYTES["det_gemm_gate_up_T4096"],
+        "traffic": traffic["bytes"],
+        "traffic_measured_on_commit": traffic["commit"],
     }
     roofline.update(_launch_percentiles(gate_up, args.steps, 5))
 
@@ -329,6 +352,7 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "conditioning_launches": 2 * CONDITIONING_STEPS,
         "ms_per_step": round(wall_ms, 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -404,6 +428,28 @@ def main() -> int:
                 shapes.append(row)
             del copies
         result["shapes"] = shapes
+
+    # ---- the eager host path at one token (no HIP graph): wall clock per call of det_gemm_linear from
+    # Python against the kernel's own time, i.e. what a decode loop that does not capture graphs pays
+    if not args.no_shapes:
+        host = []
+        for name, act, w in (("gate_up", x, w_gu), ("down", h, w_d)):
+            a1 = act[:1]
+            kernel_ms = _time_calls(lambda: gemm.det_gemm_linear(a1, w), 200, 50)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(200):
+                gemm.det_gemm_linear(a1, w)
+            issue_us = (time.perf_counter() - t0) / 200 * 1e6  # host time to issue a call (the queue absorbs the kernels)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(50):
+                gemm.det_gemm_linear(a1, w)
+                torch.cuda.synchronize()
+            sync_us = (time.perf_counter() - t0) / 50 * 1e6  # one call and a wait for its result
+            host.append({"op": name, "T": 1, "kernel_us_back_to_back": round(kernel_ms * 1e3, 1),
+                         "host_issue_us_per_call": round(issue_us, 1), "call_and_wait_us": round(sync_us, 1)})
+        result["eager_host_path"] = host
 
     # ---- attention projections at the packed token count (ragged packing does not change the launch)
     if not args.no_shapes:

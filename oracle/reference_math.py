@@ -662,7 +662,9 @@ def group_advantages(rewards, *, samples_per_prompt=None, group_boundaries=None,
     if samples_per_prompt is not None:
         bounds = list(range(0, r.size + 1, int(samples_per_prompt)))
     else:
-        bounds = [int(b) for b in group_boundaries]
+        # only the differences count (repeat_interleave over the sizes, grpo_loss.py:189-206)
+        raw = [int(b) for b in group_boundaries]
+        bounds = [b - raw[0] for b in raw]
     out = np.empty_like(r)
     for lo, hi in zip(bounds[:-1], bounds[1:]):
         g = r[lo:hi]

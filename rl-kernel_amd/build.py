@@ -14,6 +14,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "librlk_gfx950.so"
+OBJ_DIR = PKG_DIR / "build"  # object files (git-ignored)
 SOURCES = ["det_gemm.hip", "det_gemm_stream.hip", "det_gemm_tree.hip", "linear_logp.hip",
     "linear_logp_bwd.hip", "logits_logp.hip", "swiglu.hip", "grpo.hip", "rlk_api.hip"]
 
@@ -42,22 +43,47 @@ def find_hipcc() -> str:
     raise RuntimeError("hipcc not found; set HIPCC or install ROCm")
 
 
-def build(verbose: bool = True) -> Path:
-    """Compile every HIP source for gfx950 into one shared library."""
-    cmd = [find_hipcc(), *HIPCC_FLAGS, "-o", str(LIB_PATH), *[str(CSRC / s) for s in SOURCES]]
-    if verbose:
-        print("[rlk build]", " ".join(cmd), flush=True)
+def _run(cmd: list[str]) -> str:
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(
-        line for line in proc.stdout.splitlines() if "packed-fp32-ops" not in line and line.strip()
-    )
+    out = "\n".join(line for line in proc.stdout.splitlines() if "packed-fp32-ops" not in line and line.strip())
     if proc.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{out}")
-    if verbose and out:
-        print(out, flush=True)
+        raise RuntimeError(f"hipcc failed ({proc.returncode}): {' '.join(cmd)}\n{out}")
+    return out
+
+
+def build(verbose: bool = True, only: list[str] | None = None) -> Path:
+    """Compile every HIP source for gfx950 (one hipcc per source, side by side) and link them into
+    one shared library. `only` names the sources to recompile; the objects of the others are reused
+    when they exist (a developer's shortcut, the default recompiles everything)."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    hipcc = find_hipcc()
+    OBJ_DIR.mkdir(exist_ok=True)
+    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    jobs = []
+    for src in SOURCES:
+        obj = OBJ_DIR / (src + ".o")
+        if only is not None and src not in only and obj.exists():
+            continue
+        jobs.append([hipcc, *compile_flags, "-c", "-o", str(obj), str(CSRC / src)])
+    if verbose:
+        for cmd in jobs:
+            print("[rlk build]", " ".join(cmd), flush=True)
+    workers = max(1, min(len(jobs), int(os.environ.get("MAX_JOBS", "0")) or os.cpu_count() or 1))
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        outs = list(pool.map(_run, jobs))
+    link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH),
+            *[str(OBJ_DIR / (s + ".o")) for s in SOURCES]]
+    if verbose:
+        print("[rlk build]", " ".join(link), flush=True)
+    outs.append(_run(link))
+    if verbose:
+        for out in outs:
+            if out:
+                print(out, flush=True)
     return LIB_PATH
 
 
 if __name__ == "__main__":
-    build()
+    build(only=sys.argv[1:] or None)
     sys.exit(0)

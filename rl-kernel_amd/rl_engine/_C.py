@@ -856,7 +856,8 @@ def grpo_ratio_kl_loss(
     if mask is not None:
         if tuple(mask.shape) != (rollouts, tokens):
             raise RuntimeError("grpo_ratio_kl_loss: mask shape must match logp")
-        mask_u8 = mask.to(device=logp.device, dtype=torch.uint8).contiguous()
+        # any non-zero mask value keeps the token (mask.bool(), rl_engine/reference/definitions.py:50-70)
+        mask_u8 = mask.to(device=logp.device).bool().to(torch.uint8).contiguous()
     lib = _lib.load()
     ratio = torch.empty_like(logp_c)
     k3 = torch.empty_like(logp_c)

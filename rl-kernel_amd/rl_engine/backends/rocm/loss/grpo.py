@@ -31,6 +31,12 @@ def _as_2d(t: torch.Tensor) -> torch.Tensor:
     return t.reshape(1, -1) if t.dim() == 1 else t
 
 
+def _bool_mask(mask: torch.Tensor, device: torch.device) -> torch.Tensor:
+    """The mask as the reference reads it (``mask.bool()``, rl_engine/reference/definitions.py:50-70):
+    any non-zero value, fractional or above 255 included, keeps the token, and keeps it with weight one."""
+    return _as_2d(mask).to(device=device).bool()
+
+
 class _GrpoLossAutograd(torch.autograd.Function):
     """Forward on the HIP kernel; backward elementwise on the saved per-token outputs.
 
@@ -42,6 +48,7 @@ class _GrpoLossAutograd(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, cur, old, ref, adv, mask, clip_eps, beta):
+        # `mask` is already the boolean mask (see _bool_mask): the kernel and the backward weigh with the same tensor
         out3, ratio, k3 = _C.grpo_ratio_kl_loss(cur, old, ref, adv, mask, clip_eps, beta)
         ctx.save_for_backward(cur, old, ref, adv, mask if mask is not None else torch.empty(0, device=cur.device))
         ctx.has_mask = mask is not None
@@ -97,7 +104,7 @@ def grpo_ratio_kl_loss(
         raise ValueError(f"expected {cur.size(0)} per-rollout advantages, got {adv.numel()}")
     mask = None
     if completion_mask is not None:
-        mask = _as_2d(completion_mask)
+        mask = _bool_mask(completion_mask, cur.device)
         if mask.shape != cur.shape:
             raise ValueError("completion_mask must match the log-prob shape")
     if torch.is_grad_enabled() and cur.requires_grad:
@@ -132,32 +139,33 @@ def group_advantages(
             raise ValueError("samples_per_prompt must be at least 2 for group normalization.")
         if n % samples_per_prompt != 0:
             raise ValueError(f"num_sequences ({n}) must be divisible by samples_per_prompt ({samples_per_prompt}).")
-        bounds = list(range(0, n + 1, int(samples_per_prompt)))
+        sizes = [int(samples_per_prompt)] * (n // int(samples_per_prompt))
     else:
         b = torch.as_tensor(group_boundaries, dtype=torch.long).cpu()
         if b.ndim != 1 or b.numel() < 2:
             raise ValueError("group_boundaries must be a 1D tensor of length num_groups + 1.")
-        bounds = [int(v) for v in b.tolist()]
-        sizes = [hi - lo for lo, hi in zip(bounds[:-1], bounds[1:])]
+        # Only the differences count, as in the reference (repeat_interleave over the sizes): group g is the
+        # run of sizes[g] sequences after the groups before it, wherever the boundaries themselves start.
+        sizes = [int(v) for v in (b[1:] - b[:-1]).tolist()]
         if sum(sizes) != n:
             raise ValueError(f"group sizes sum to {sum(sizes)} but there are {n} sequences.")
         if any(size < 1 for size in sizes):
             raise ValueError("each group must contain at least one sequence.")
-    out = torch.empty_like(flat)
-    uniform = len(bounds) > 1 and len({hi - lo for lo, hi in zip(bounds[:-1], bounds[1:])}) == 1 and bounds[0] == 0
-    groups = list(zip(bounds[:-1], bounds[1:]))
-    if uniform and n:
-        size = bounds[1] - bounds[0]
-        g = flat.view(-1, size)
+    if n == 0:
+        return flat.clone()
+
+    def _normalise(g: torch.Tensor, size: int) -> torch.Tensor:  # g: [groups, size]
         mean = g.sum(dim=1, keepdim=True) / size
         var = (g * g).sum(dim=1, keepdim=True) / size - mean * mean
-        return ((g - mean) / var.clamp_min(eps**2).sqrt()).reshape(-1)
-    for lo, hi in groups:
-        g = flat[lo:hi]
-        mean = g.sum() / (hi - lo)
-        var = (g * g).sum() / (hi - lo) - mean * mean
-        out[lo:hi] = (g - mean) / var.clamp_min(eps**2).sqrt()
-    return out
+        return (g - mean) / var.clamp_min(eps**2).sqrt()
+
+    if len(set(sizes)) == 1:
+        return _normalise(flat.view(-1, sizes[0]), sizes[0]).reshape(-1)
+    pieces, start = [], 0
+    for size in sizes:
+        pieces.append(_normalise(flat[start : start + size].view(1, size), size).reshape(-1))
+        start += size
+    return torch.cat(pieces)
 
 
 def compute_policy_ratio(current_logps, old_logps, mask=None) -> torch.Tensor:

@@ -71,8 +71,14 @@ def test_config1_parity_and_batch_invariance(gemm, oracle):
     assert c.shape == (128, 1024) and c.dtype == torch.bfloat16
     _assert_parity(oracle, c, a, b.t().contiguous(), "config1")
     # sequential-k restatement (the reference's native twin of the contract)
-    seq = oracle.det_gemm_seq(inputs.bits(a[:16]), inputs.bits(b.t().contiguous()))
-    assert oracle.bf16_ulp_distance(inputs.bits(c[:16]), seq).max() <= 1 or True  # cancellation handled above
+    # (a different fp32 summation order: within 1 bf16 ulp away from near-total cancellation)
+    a16, bt = inputs.bits(a[:16]), inputs.bits(b.t().contiguous())
+    seq = oracle.det_gemm_seq(a16, bt)
+    af, wf = oracle.bf16_to_f32(a16).astype(np.float64), oracle.bf16_to_f32(bt).astype(np.float64)
+    clean = np.abs(af @ wf.T) > 2.0**-6 * (np.abs(af) @ np.abs(wf).T)
+    seq_ulp = oracle.bf16_ulp_distance(inputs.bits(c[:16]), seq)
+    assert clean.mean() > 0.5 and seq_ulp[clean].max() <= 1, "more than 1 bf16 ulp from the sequential-k restatement"
+    assert (seq_ulp > 1).mean() < 1e-3
     # rows 0..6 recomputed at M=1 and M=7 must be bit-identical
     c7 = gemm.deterministic_gemm(a_d[:7], b_d)
     assert _same_bits(c7, c[:7])
@@ -238,15 +244,36 @@ def test_config2_rows_are_bit_invariant_across_token_counts(gemm, ffn):
     assert _same_bits(gemm.det_gemm_linear(ffn["h"][4095:4096], ffn["w_d"]), dn_full[4095:4096])
 
 
-def test_config2_parity_on_sampled_rows_and_columns(gemm, oracle, ffn):
+def _edge_rows(m: int, seed: int, extra: int = 64) -> torch.Tensor:
+    """Rows on both sides of every tile height in use (16 ... 256), the last rows, and `extra` random ones."""
+    fixed = [0, 1, 15, 16, 63, 64, 127, 128, 191, 192, 255, 256, 257, 511, 512, m // 2 - 1, m // 2, m - 257, m - 256, m - 2, m - 1]
+    rnd = torch.randperm(m, generator=torch.Generator().manual_seed(seed))[:extra].tolist()
+    return torch.tensor(sorted({r for r in fixed + rnd if 0 <= r < m}))
+
+
+def _edge_cols(n: int) -> torch.Tensor:
+    """Columns on both sides of the 64 / 192 / 256-wide tile seams, of the last tile and of the gate | up seam."""
+    fixed = [0, 15, 16, 63, 64, 191, 192, 255, 256, 383, 384, 511, 512, n // 2 - 1, n // 2, n - 257, n - 256, n - 193, n - 192, n - 65, n - 64, n - 1]
+    return torch.tensor(sorted({c for c in fixed if 0 <= c < n}))
+
+
+def _assert_whole_rows_and_columns(oracle, got, a, w, seed, tag):
+    """Every column of the rows at tile edges (plus 64 random rows) and every row of the columns at tile
+    edges, against the fp64 oracle on the host: a refill or edge-clamp mistake at a tile seam shows here,
+    where bit-equality of the kernel with itself would not."""
+    m, n = got.shape
+    rows, cols = _edge_rows(m, seed), _edge_cols(n)
+    _assert_parity(oracle, got[rows.to(DEV)], a[rows], w, f"{tag} whole rows")
+    _assert_parity(oracle, got[:, cols.to(DEV)], a, w[cols], f"{tag} whole columns")
+
+
+@pytest.mark.parametrize("tokens", [4096, 256])
+def test_config2_parity_on_whole_rows_and_columns_at_tile_edges(gemm, oracle, ffn, tokens):
     w_gu, w_d, x, h = ffn["cpu"]
-    gu = gemm.det_gemm_linear(ffn["x"], ffn["w_gu"])
-    dn = gemm.det_gemm_linear(ffn["h"], ffn["w_d"])
-    rows = torch.tensor([0, 1, 15, 255, 1023, 2048, 4095])
-    cols_gu = torch.arange(0, 24576, 97)
-    cols_dn = torch.arange(0, 4096, 17)
-    _assert_parity(oracle, gu[rows.to(DEV)][:, cols_gu.to(DEV)], x[rows], w_gu[cols_gu], "gate_up sample")
-    _assert_parity(oracle, dn[rows.to(DEV)][:, cols_dn.to(DEV)], h[rows], w_d[cols_dn], "down sample")
+    gu = gemm.det_gemm_linear(ffn["x"][:tokens], ffn["w_gu"])
+    dn = gemm.det_gemm_linear(ffn["h"][:tokens], ffn["w_d"])
+    _assert_whole_rows_and_columns(oracle, gu, x[:tokens], w_gu, 2101 + tokens, f"gate_up T={tokens}")
+    _assert_whole_rows_and_columns(oracle, dn, h[:tokens], w_d, 2102 + tokens, f"down T={tokens}")
 
 
 def test_config2_small_t_full_parity(gemm, oracle, ffn):
@@ -281,9 +308,8 @@ def test_config3_same_token_same_bits_across_packings(gemm, oracle):
         canon_a[map_a.to(DEV)] = out_a
         canon_b[map_b.to(DEV)] = out_b
         assert _same_bits(canon_a, canon_b), name
-        rows = torch.tensor([0, 777, 8191, 16383])
-        cols = torch.arange(0, w.size(0), 61)
-        _assert_parity(oracle, canon_a[rows.to(DEV)][:, cols.to(DEV)], tokens[rows], w[cols], f"{name} sample")
+        # packing A against the oracle in packed order, so the rows at tile edges are the kernel's own
+        _assert_whole_rows_and_columns(oracle, out_a, tokens[map_a], w, 3100, f"{name} packing A")
 
 
 # ---------------------------------------------------------------------------

@@ -10,6 +10,7 @@ import subprocess
 import sys
 from pathlib import Path
 
+import numpy as np
 import pytest
 import torch
 
@@ -264,6 +265,15 @@ def test_group_advantages_known_answers_and_errors():
     assert torch.allclose(uniform, torch.from_numpy(oracle.group_advantages(rewards.numpy(), samples_per_prompt=4)), atol=1e-6)
     ragged = group_advantages(rewards, group_boundaries=torch.tensor([0, 1, 5, 12]))
     assert torch.allclose(ragged, torch.from_numpy(oracle.group_advantages(rewards.numpy(), group_boundaries=[0, 1, 5, 12])), atol=1e-5)
+    # boundaries that do not start at zero: only the group sizes count (the reference builds its group ids with
+    # repeat_interleave over the differences), and every sequence gets a value
+    six = rewards[:6]
+    shifted = group_advantages(six, group_boundaries=[2, 5, 8])
+    assert torch.equal(shifted, group_advantages(six, group_boundaries=[0, 3, 6]))
+    g0 = six[:3]
+    want0 = (g0 - g0.mean()) / ((g0 * g0).mean() - g0.mean() ** 2).clamp_min(1e-12).sqrt()
+    assert torch.allclose(shifted[:3], want0, atol=1e-5) and bool(torch.isfinite(shifted).all())
+    assert np.allclose(oracle.group_advantages(six.numpy(), group_boundaries=[2, 5, 8]), shifted.numpy(), atol=1e-5)
     assert float(ragged[0]) == 0.0  # a group of one: zero variance is floored at eps, the numerator is zero
     assert torch.equal(group_advantages(torch.full((4,), 2.5), samples_per_prompt=2), torch.zeros(4))
     for kwargs in ({}, {"samples_per_prompt": 4, "group_boundaries": [0, 4, 8, 12]}, {"samples_per_prompt": 1},

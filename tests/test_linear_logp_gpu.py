@@ -307,7 +307,10 @@ def test_config4_full_size(logp_mod, oracle, config4):
     packed, _ = logp_mod.deterministic_linear_logp(c["h_d"][perm], c["w_d"], c["t_d"][perm])
     assert _same_bits(packed, logp[perm])
     # parity with the oracle's chunked online LSE on a random 256-row sample
-    sample = torch.randperm(8192, generator=torch.Generator().manual_seed(4003))[:256].sort().values
+    # plus the rows on both sides of every token-tile seam and the last rows
+    sample = torch.randperm(8192, generator=torch.Generator().manual_seed(4003))[:256]
+    edges = torch.tensor([0, 15, 16, 63, 64, 127, 128, 255, 256, 257, 511, 512, 4095, 4096, 7935, 7936, 8190, 8191])
+    sample = torch.unique(torch.cat([sample, edges]))
     ref_logp, ref_lse = oracle.linear_logp_chunked(
         inputs.bits(c["h"][sample]), inputs.bits(c["w"]), c["t"][sample].numpy(), chunk_elems=256 * 2048
     )[:2]
@@ -424,6 +427,36 @@ def test_grpo_loss_gradients_match_torch_autograd(loss_mod):
     a = loss_mod.grpo_ratio_kl_loss(cur, old, ref, adv, mask, beta=0.01)
     b = loss_mod.grpo_ratio_kl_loss(cur.detach(), old, ref, adv, mask, beta=0.01)
     assert _same_bits(a.loss.detach().reshape(1), b.loss.reshape(1)) and _same_bits(a.k3, b.k3)
+
+
+def test_grpo_mask_is_read_as_a_boolean_in_forward_and_backward(loss_mod):
+    """A mask with values other than 0 / 1 (2, 0.5, 256) keeps those tokens with weight one, forward and
+    backward alike: the reference reads every mask through ``mask.bool()`` (reference/definitions.py:50-70)."""
+    g = torch.Generator().manual_seed(5310)
+    rollouts, tokens = 5, 40
+    base = -torch.randn((rollouts, tokens), generator=g).abs()
+    old = (base + 0.2 * torch.randn((rollouts, tokens), generator=g)).to(DEV)
+    ref = (base + 0.2 * torch.randn((rollouts, tokens), generator=g)).to(DEV)
+    adv = torch.randn(rollouts, generator=g).to(DEV)
+    keep = (torch.rand((rollouts, tokens), generator=g) < 0.7).to(DEV)
+    values = torch.tensor([2.0, 0.5, 256.0, 1.0], device=DEV)
+    odd = keep.float() * values[torch.arange(rollouts * tokens, device=DEV).view(rollouts, tokens) % 4]
+    assert bool(((odd != 0) == keep).all())
+    results = []
+    for mask in (keep, odd, odd.to(torch.int32)):
+        cur = base.to(DEV).clone().requires_grad_(True)
+        out = loss_mod.grpo_ratio_kl_loss(cur, old, ref, adv, mask, beta=0.05)
+        out.loss.backward()
+        results.append((out.loss.detach().reshape(1), out.ratio, out.k3, cur.grad))
+    # int32 truncates 0.5 to 0 before the library sees it, exactly as `.to(int32).bool()` does in the reference
+    as_int = odd.to(torch.int32).bool()
+    for got, want in zip(results[1], results[0]):
+        assert _same_bits(got, want)
+    cur = base.to(DEV).clone().requires_grad_(True)
+    out = loss_mod.grpo_ratio_kl_loss(cur, old, ref, adv, as_int, beta=0.05)
+    out.loss.backward()
+    for got, want in zip(results[2], (out.loss.detach().reshape(1), out.ratio, out.k3, cur.grad)):
+        assert _same_bits(got, want)
 
 
 def test_rl_loss_step_end_to_end(logp_mod, loss_mod):
