@@ -218,6 +218,30 @@ int rlk_linear_logp_fwd_shard(const void* hidden, int64_t h_row_stride, const vo
                               float* target_logit, float* lse, void* workspace, size_t workspace_bytes, int T,
                               int D, int V, int64_t vocab_start, int real_vocab_end, int config, void* stream);
 
+/* Size of the scratch array built into the library for rlk_linear_logp_fwd_noalloc (32 MiB per GPU). */
+#define RLK_NOALLOC_SCRATCH_BYTES (32u << 20)
+
+/*
+ * rlk_linear_logp_fwd for callers that cannot allocate device memory or pass a workspace: code
+ * under HIP-graph capture, tight serving loops, harnesses that forbid hipMalloc. Same inputs,
+ * outputs, checks, kernels and result bits as rlk_linear_logp_fwd; the fp32 partials go into a
+ * scratch array that is part of the loaded library (RLK_NOALLOC_SCRATCH_BYTES of device memory per
+ * GPU, held until the process ends) instead of a caller workspace. The call allocates and frees
+ * nothing and calls no allocating routine. It serves every (T, V) with
+ * rlk_linear_logp_workspace_bytes(T, V) <= RLK_NOALLOC_SCRATCH_BYTES (V = 151936: up to 1024
+ * tokens, and 1025 ... 18765 tokens, whose partials are 17 times smaller per token) and returns
+ * RLK_ERR_INVALID_ARGUMENT beyond that. All calls on one GPU share that GPU's array: calls that
+ * may overlap on one GPU (different streams, different host threads) race on it and must be
+ * ordered by the caller. The first call on a device looks the array's address up once
+ * (hipGetSymbolAddress), so make that call outside graph capture.
+ *
+ * No counterpart in the reference: it exists for the callers named above.
+ */
+int rlk_linear_logp_fwd_noalloc(const void* hidden, int64_t h_row_stride, const void* weight, int64_t w_row_stride,
+                                const int64_t* target, const float* bias, const float* temperature, float* logp,
+                                float* lse, int T, int D, int V, int64_t vocab_start, int real_vocab_end, int config,
+                                void* stream);
+
 /* Bytes of workspace rlk_linear_logp_bwd needs: the bf16 d(logits) [T, V rounded up to 64]
  * plus, when a bias gradient is wanted, fp32 block sums [ceil(T / 256), V]. */
 size_t rlk_linear_logp_bwd_workspace_bytes(int T, int V, int with_bias);

@@ -39,6 +39,30 @@ static int device_error(const char* what, hipError_t err) {
   return RLK_ERR_DEVICE;
 }
 
+// Scratch of rlk_linear_logp_fwd_noalloc: device memory that belongs to the loaded code object, one copy
+// per GPU, held until the process ends. In host code the array's name is only a handle for
+// hipGetSymbolAddress; kernels and fills get the per-device address looked up below.
+static __device__ __align__(256) unsigned char scratch[RLK_NOALLOC_SCRATCH_BYTES];
+
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// The current device's copy of `scratch` (looked up once per device; no allocation).
+static hipError_t scratch_for_current_device(void** out) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return err;
+    if (ptr == nullptr) return hipErrorInvalidSymbol;
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // several threads may store the same address
+  }
+  *out = ptr;
+  return hipSuccess;
+}
+
 }  // namespace rlk
 
 using namespace rlk;
@@ -209,6 +233,28 @@ int rlk_linear_logp_fwd_shard(const void* hidden, int64_t h_row_stride, const vo
   return linear_logp_fwd_checked("rlk_linear_logp_fwd_shard", hidden, h_row_stride, weight, w_row_stride, target,
                                  bias, temperature, nullptr, lse, target_logit, workspace, workspace_bytes, T, D, V,
                                  vocab_start, real_vocab_end, config, stream);
+}
+
+int rlk_linear_logp_fwd_noalloc(const void* hidden, int64_t h_row_stride, const void* weight, int64_t w_row_stride,
+                                const int64_t* target, const float* bias, const float* temperature, float* logp,
+                                float* lse, int T, int D, int V, int64_t vocab_start, int real_vocab_end, int config,
+                                void* stream) {
+  const size_t need = (T > 0 && V > 0) ? linear_logp_workspace_bytes(T, V) : 0;
+  if (need > (size_t)RLK_NOALLOC_SCRATCH_BYTES) {
+    set_last_error(
+        "rlk_linear_logp_fwd_noalloc: T=%d tokens x V=%d vocabulary rows need %zu bytes of partials, the built-in "
+        "scratch holds %zu; use rlk_linear_logp_fwd with a workspace",
+        T, V, need, (size_t)RLK_NOALLOC_SCRATCH_BYTES);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  void* ptr = nullptr;
+  hipError_t err = scratch_for_current_device(&ptr);
+  if (err != hipSuccess) return device_error("rlk_linear_logp_fwd_noalloc(scratch lookup)", err);
+  // Every partial a call reads was written by that call's own kernels first, so nothing left in the
+  // scratch by an earlier (larger) call needs clearing.
+  return linear_logp_fwd_checked("rlk_linear_logp_fwd_noalloc", hidden, h_row_stride, weight, w_row_stride, target,
+                                 bias, temperature, logp, lse, nullptr, ptr, (size_t)RLK_NOALLOC_SCRATCH_BYTES, T, D,
+                                 V, vocab_start, real_vocab_end, config, stream);
 }
 
 size_t rlk_linear_logp_bwd_workspace_bytes(int T, int V, int with_bias) {

@@ -42,6 +42,7 @@ GEMM_CONFIGS = {
 }
 # OR-ed into a GEMM or LogP configuration: register-staged main loop (bit-neutral).
 FORCE_STAGED = 0x100
+NOALLOC_SCRATCH_BYTES = 32 << 20  # RLK_NOALLOC_SCRATCH_BYTES
 # rlk_dtype (element types of materialised logits)
 DTYPE_BF16, DTYPE_FP16, DTYPE_FP32 = 0, 1, 2
 # rlk_logp_config
@@ -61,6 +62,7 @@ EXPORTED_SYMBOLS = (
     "rlk_linear_logp_workspace_bytes",
     "rlk_linear_logp_fwd",
     "rlk_linear_logp_fwd_shard",
+    "rlk_linear_logp_fwd_noalloc",
     "rlk_linear_logp_bwd_workspace_bytes",
     "rlk_linear_logp_bwd",
     "rlk_logits_tile_stats",
@@ -131,6 +133,8 @@ def load() -> ctypes.CDLL:
     lib.rlk_linear_logp_fwd.argtypes = [vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, sz, i32, i32, i32, i64, i32, i32, vp]
     lib.rlk_linear_logp_fwd_shard.restype = i32
     lib.rlk_linear_logp_fwd_shard.argtypes = lib.rlk_linear_logp_fwd.argtypes
+    lib.rlk_linear_logp_fwd_noalloc.restype = i32
+    lib.rlk_linear_logp_fwd_noalloc.argtypes = [vp, i64, vp, i64, vp, vp, vp, vp, vp, i32, i32, i32, i64, i32, i32, vp]
 
     lib.rlk_linear_logp_bwd_workspace_bytes.restype = sz
     lib.rlk_linear_logp_bwd_workspace_bytes.argtypes = [i32, i32, i32]
