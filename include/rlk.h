@@ -198,6 +198,24 @@ int rlk_linear_logp_fwd(const void* hidden, int64_t h_row_stride, const void* we
                         int64_t vocab_start, int real_vocab_end, int config, void* stream);
 
 /*
+ * rlk_linear_logp_fwd that also stores the logits, from the same pass (no second GEMM):
+ *   logits [T, logits_row_stride >= V] fp32 out: the fp32 accumulators of the lm_head GEMM with the
+ *          bias added and padded lanes (columns >= real_vocab_end) set to -inf, NOT scaled by the
+ *          temperature. Bit for bit what rlk_det_gemm_bf16 with out_fp32 writes for hidden @ weight^T,
+ *          plus the bias. logp and lse have the bits rlk_linear_logp_fwd gives.
+ * Everything else as in rlk_linear_logp_fwd. HBM-bound on the T * V * 4 bytes it writes.
+ *
+ * Stands in for return_logits=True of rl_engine._C.fused_linear_logp_sm90 (csrc/bindings/ops.cpp:514-520;
+ * csrc/cuda/logprob/fused_linear_logp_sm90.cu:2040-2176) and of triton_deterministic_linear_logp
+ * (store_logits, rl_engine/backends/shared/triton/logprob/linear_logp.py:366-380, 693).
+ */
+int rlk_linear_logp_fwd_logits(const void* hidden, int64_t h_row_stride, const void* weight, int64_t w_row_stride,
+                               const int64_t* target, const float* bias, const float* temperature, float* logp,
+                               float* lse, float* logits, int64_t logits_row_stride, void* workspace,
+                               size_t workspace_bytes, int T, int D, int V, int64_t vocab_start, int real_vocab_end,
+                               int config, void* stream);
+
+/*
  * The same pass for one shard of a vocabulary split over ranks: `weight` holds rows
  * [vocab_start, vocab_start + V) of the lm_head, `target` stays in global ids, and the
  * outputs are the two terms a caller merges across shards,
@@ -243,7 +261,8 @@ int rlk_linear_logp_fwd_noalloc(const void* hidden, int64_t h_row_stride, const 
                                 void* stream);
 
 /* Bytes of workspace rlk_linear_logp_bwd needs: the bf16 d(logits) [T, V rounded up to 64]
- * plus, when a bias gradient is wanted, fp32 block sums [ceil(T / 256), V]. */
+ * plus, when a bias gradient is wanted, fp32 column sums per token tile
+ * ([ceil(T / 16), V] up to 1024 tokens, [ceil(T / 64), V] above). */
 size_t rlk_linear_logp_bwd_workspace_bytes(int T, int V, int with_bias);
 
 /*
@@ -258,7 +277,9 @@ size_t rlk_linear_logp_bwd_workspace_bytes(int T, int V, int with_bias);
  *   d(logits) = (p * (grad_lse - grad_logp) + [column == target] * grad_logp) / temperature,
  * rounded once to bf16; grad_hidden = d(logits) @ weight over the vocabulary ascending,
  * grad_weight = d(logits)^T @ hidden over tokens ascending (both under the det_gemm
- * contract), grad_bias = column sums of d(logits) in fixed 256-token blocks. The clamp
+ * contract), grad_bias = column sums of the fp32 d(logits) BEFORE that rounding (as the
+ * reference's chunked backward sums them), in a fixed tree over the token index inside
+ * 256-token blocks, blocks added ascending. The clamp
  * logp = min(., 0) of the forward is not differentiated (gradient 1), as in the reference.
  * workspace must be 256-byte aligned.
  *
@@ -275,6 +296,27 @@ int rlk_linear_logp_bwd(const void* hidden, int64_t h_row_stride, const void* we
 
 /* Element types of materialised logits. */
 typedef enum rlk_dtype { RLK_DTYPE_BF16 = 0, RLK_DTYPE_FP16 = 1, RLK_DTYPE_FP32 = 2 } rlk_dtype;
+
+/*
+ * C[M,N] = A[M,K] @ B[K,N] with a strictly sequential fp32 chain (rlk_det_gemm_seq_contract_id):
+ *   C[i,j] = fma(a[i,K-1], b[K-1,j], ... fma(a[i,1], b[1,j], fma(a[i,0], b[0,j], +0)) ...),
+ * one fp32 fused multiply-add per k, k ascending, one accumulator per element, nothing rounded below fp32.
+ * a_dtype / b_dtype / c_dtype are RLK_DTYPE_BF16 or RLK_DTYPE_FP32 (bf16 operands are widened exactly; a
+ * bf16 output is the fp32 result rounded once). Strides in elements as in rlk_det_gemm_bf16, any
+ * non-negative values. Rows are batch invariant. Vector-ALU kernel (about 45 TFLOP/s): the fp32-result
+ * path of the strict GEMM, not a replacement for rlk_det_gemm_bf16.
+ *
+ * Stands in for _triton_gemm_fp32 / _det_gemm_fp32_kernel
+ * (rl_engine/backends/shared/triton/gemm/det_gemm.py:680-749), i.e. DetGemmOp.forward_fp32 and
+ * forward_accum_fp32 with bf16 or fp32 operands (rl_engine/backends/rocm/gemm/det_gemm.py:545-555), and for
+ * rl_engine._C.det_gemm_fwd_fp32 / det_gemm_accum_fwd_fp32 (rl_engine/_C.pyi:244-248; csrc/musa/det_gemm.mu:25-48).
+ */
+int rlk_det_gemm_seq(const void* a, int a_dtype, int64_t a_row_stride, int64_t a_k_stride, const void* b, int b_dtype,
+                     int64_t b_k_stride, int64_t b_n_stride, void* c, int c_dtype, int64_t ldc, int M, int N, int K,
+                     void* stream);
+
+/* Contract id of rlk_det_gemm_seq. */
+const char* rlk_det_gemm_seq_contract_id(void);
 
 /*
  * Per-row, per-tile statistics of materialised logits [T, V] (row stride in elements):

@@ -156,6 +156,23 @@ def det_gemm_seq(a_bits: np.ndarray, bt_bits: np.ndarray) -> np.ndarray:
     return out
 
 
+def det_gemm_seq_f32(a: np.ndarray, bt: np.ndarray) -> np.ndarray:
+    """fp32 ``a[M,K] @ bt[N,K].T`` by one fused multiply-add per k, k ascending from +0, unrounded fp32 result
+    (the float instantiation of csrc/musa/det_gemm.mu:25-48; the role of _det_gemm_fp32_kernel,
+    rl_engine/backends/shared/triton/gemm/det_gemm.py:680-749). Operands are float32 arrays (widen bf16
+    bit patterns with bf16_to_f32 first)."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    bt = np.ascontiguousarray(bt, dtype=np.float32)
+    assert a.ndim == 2 and bt.ndim == 2 and a.shape[1] == bt.shape[1]
+    out = np.empty((a.shape[0], bt.shape[0]), dtype=np.float32)
+    f32p = ctypes.POINTER(ctypes.c_float)
+    lib = _c()
+    lib.oracle_gemm_seq_fma_f32in.argtypes = [f32p, f32p, f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+    lib.oracle_gemm_seq_fma_f32in.restype = None
+    lib.oracle_gemm_seq_fma_f32in(a.ctypes.data_as(f32p), bt.ctypes.data_as(f32p), out.ctypes.data_as(f32p), a.shape[0], bt.shape[0], a.shape[1])
+    return out
+
+
 def det_gemm_f64(a_bits: np.ndarray, bt_bits: np.ndarray) -> np.ndarray:
     """The exact products accumulated in fp64, unrounded (brute-force anchor)."""
     a, bt = _prep(a_bits, bt_bits)

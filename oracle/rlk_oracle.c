@@ -56,6 +56,23 @@ void oracle_gemm_seq_f32(const uint16_t* a, const uint16_t* bt, uint16_t* c, int
     }
 }
 
+/*
+ * The sequential chain on fp32 operands with an fp32 result: acc = fmaf(a_ik, b_kj, acc), k ascending
+ * from +0, nothing rounded below fp32. Follows the same kernel with float inputs and a float output
+ * (csrc/musa/det_gemm.mu:25-48 instantiated for float, its det_gemm_fwd_fp32) and the role of the
+ * reference's fp32-output strict GEMM, rl_engine/backends/shared/triton/gemm/det_gemm.py:680-749. The
+ * step is written as one fused multiply-add (for bf16-valued operands the product is exact, so the fused
+ * step equals multiply-then-add; for general fp32 operands this is the stated choice).
+ */
+void oracle_gemm_seq_fma_f32in(const float* a, const float* bt, float* c, int M, int N, int K) {
+  for (int i = 0; i < M; ++i)
+    for (int j = 0; j < N; ++j) {
+      float acc = 0.0f;
+      for (int k = 0; k < K; ++k) acc = fmaf(a[(size_t)i * K + k], bt[(size_t)j * K + k], acc);
+      c[(size_t)i * N + j] = acc;
+    }
+}
+
 /* The same sum accumulated in fp64 (every product is exact; the fp64 sum of
  * K <= 2^20 such products is exact to far below one fp32 ulp). Output is the
  * unrounded double, for tests that bound the distance to the true value. */

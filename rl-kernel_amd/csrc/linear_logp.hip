@@ -38,6 +38,8 @@ struct LogpArgs {
   const float* bias;         // [V] or null
   const float* temperature;  // [T] or null
   float* part;               // [3][n_split][T]: max, sum, target logit
+  float* logits;             // [T, logits_ld] fp32 biased logits (no temperature), or null: not wanted
+  int64_t logits_ld;
   int T, V, D;
   int vocab_limit;  // local column bound of the real vocabulary (<= V)
   int64_t vocab_start;
@@ -109,9 +111,15 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_partial_kernel(LogpAr
     for (int jm = 0; jm < S::TM; ++jm) {
       float y[16];
 #pragma unroll
-      for (int c = 0; c < 16; ++c)
-        y[c] = scaled_logit(acc[c >> 2][jm][c & 3], a.bias != nullptr, bias_run[c], col0 + c, a.vocab_limit,
-                            a.temperature != nullptr, inv_t[jm]);
+      for (int c = 0; c < 16; ++c) y[c] = biased_logit(acc[c >> 2][jm][c & 3], a.bias != nullptr, bias_run[c], col0 + c, a.vocab_limit);
+      if (a.logits) {  // the same accumulators the reduction sees, stored before the temperature
+        const int m = m0 + tok_local + jm * 16;
+        if (m < a.T) store_logit_run(a.logits + (int64_t)m * a.logits_ld, col0, a.V, y);
+      }
+      if (a.temperature) {
+#pragma unroll
+        for (int c = 0; c < 16; ++c) y[c] = y[c] * inv_t[jm];
+      }
       logp_fold_run(y, tgt[jm] - col0, run_m[jm], run_s[jm], run_zt[jm]);
     }
   }
@@ -210,9 +218,12 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_streamgroup_kernel(Lo
         }
         float y[16];
 #pragma unroll
-        for (int c = 0; c < 16; ++c)
-          y[c] = scaled_logit(acc[c >> 2][jm][c & 3], a.bias != nullptr, bias_run[c], col0 + c, a.vocab_limit,
-                              a.temperature != nullptr, inv_t);
+        for (int c = 0; c < 16; ++c) y[c] = biased_logit(acc[c >> 2][jm][c & 3], a.bias != nullptr, bias_run[c], col0 + c, a.vocab_limit);
+        if (a.logits && m < a.T) store_logit_run(a.logits + (int64_t)m * a.logits_ld, col0, a.V, y);
+        if (a.temperature) {
+#pragma unroll
+          for (int c = 0; c < 16; ++c) y[c] = y[c] * inv_t;
+        }
         logp_fold_run(y, tgt - col0, run_m, run_s, run_zt);
         sm[slot] = run_m;
         ss[slot] = run_s;
@@ -425,9 +436,11 @@ int pick_linear_logp_config(int T, int V) {
 
 hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t* target, const float* bias,
                               const float* temperature, float* logp, float* lse, float* target_logit,
-                              float* workspace, int T, int D, int V, int64_t vocab_start, int vocab_limit, int config,
-                              hipStream_t stream) {
+                              float* logits, int64_t logits_ld, float* workspace, int T, int D, int V,
+                              int64_t vocab_start, int vocab_limit, int config, hipStream_t stream) {
   LogpArgs a;
+  a.logits = logits;
+  a.logits_ld = logits_ld;
   a.W = W;
   a.H = H;
   a.target = target;

@@ -19,8 +19,13 @@
 //      it is batch invariant like the forward.
 //   3. grad_weight[V, D] = dz^T[V, T] @ H[T, D]: det_gemm over tokens, ascending, both
 //      operands read K-major (no transposed copies).
-//      grad_bias[V] = column sums of the bf16 dz in fp32: 256-token blocks summed
-//      ascending inside a block, block sums added ascending.
+//      grad_bias[V] = column sums of the UNROUNDED fp32 dz (the reference sums dz before it is cast,
+//      rl_engine/reference/logprob/linear_logp.py:704-705), accumulated by the dlogits kernel itself in a
+//      fixed tree over the token index that no tile configuration changes: inside a block of 256 tokens,
+//      token t = 16 g + l; first the 16 tokens of a group g are added in an xor butterfly over l (steps
+//      1, 2, 4, 8), then the 16 groups in a balanced binary tree over g (adjacent pairs first); tokens past T
+//      and groups past the last tile enter as +0, so every configuration performs the same additions; the
+//      256-token block sums are added ascending.
 #include "linear_logp_common.h"
 #include "rlk_host.h"
 
@@ -37,14 +42,25 @@ struct LogpBwdArgs {
   const float* grad_lse;     // [T] or null (= 0)
   bf16_bits* dz;             // [T, ld_dz]
   int64_t ld_dz;
+  float* bias_part;          // [tiles_m, V] per-token-tile column sums of the fp32 dz (BIAS_GRAD kernels)
   int T, V, D;
   int vocab_limit;
   int64_t vocab_start;
   int tiles_m, tiles_v, group_m;
 };
 
+// Sum over the 16 lanes of a lane group (lanes that share lane >> 4), identical in all of them: xor butterfly.
+__device__ __forceinline__ float group16_sum(float v) {
+  v = v + __shfl_xor(v, 1);
+  v = v + __shfl_xor(v, 2);
+  v = v + __shfl_xor(v, 4);
+  v = v + __shfl_xor(v, 8);
+  return v;
+}
+
 // LOOP: 0 generic element loader, 1 register-staged 16-byte loads, 2 direct-to-LDS ping-pong.
-template <class S, int LOOP>
+// BIAS_GRAD: also write the tile's column sums of the fp32 dz to a.bias_part (see the header for the order).
+template <class S, int LOOP, bool BIAS_GRAD>
 __global__ __launch_bounds__(S::kThreads) void linear_logp_dlogits_kernel(LogpBwdArgs a) {
   static_assert(S::BN == kLogpTileCols && S::kRun == 16 && S::WN == 4, "a lane owns 16 consecutive columns");
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -85,18 +101,26 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_dlogits_kernel(LogpBw
     for (int c = 0; c < 16; ++c) bias_run[c] = (col0 + c < a.V) ? a.bias[col0 + c] : 0.f;
   }
 
+  // Tree slots of the bias gradient: level[L] holds the finished sum of 2^L consecutive 16-token groups.
+  constexpr int kLevels = S::TM >= 8 ? 4 : S::TM >= 4 ? 3 : S::TM >= 2 ? 2 : 1;
+  static_assert((S::TM & (S::TM - 1)) == 0 && S::TM <= 8, "token groups per lane: a power of two");
+  float level[BIAS_GRAD ? kLevels : 1][16];
+
 #pragma unroll
   for (int jm = 0; jm < S::TM; ++jm) {
     const int m = m0 + tok_local + jm * 16;
-    if (m >= a.T) continue;
-    const int64_t local = a.target[m] - a.vocab_start;
+    const bool live = m < a.T;
+    if (!BIAS_GRAD && !live) continue;
+    const int mr = live ? m : a.T - 1;  // a dead row reads a valid row's scalars and contributes +0
+    const int64_t local = a.target[mr] - a.vocab_start;
     const int tl = (local >= 0 && local < a.vocab_limit) ? (int)local - col0 : -1;
-    const float inv_t = a.temperature ? 1.0f / a.temperature[m] : 1.0f;
-    const float row_lse = a.lse[m];
-    const float g_logp = a.grad_logp ? a.grad_logp[m] : 0.f;
-    const float g_lse = a.grad_lse ? a.grad_lse[m] : 0.f;
+    const float inv_t = a.temperature ? 1.0f / a.temperature[mr] : 1.0f;
+    const float row_lse = a.lse[mr];
+    const float g_logp = a.grad_logp ? a.grad_logp[mr] : 0.f;
+    const float g_lse = a.grad_lse ? a.grad_lse[mr] : 0.f;
     const float coeff = g_lse - g_logp;
     uint32_t packed[8];
+    float cur[16];
 #pragma unroll
     for (int c = 0; c < 16; c += 2) {
       float d[2];
@@ -109,9 +133,24 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_dlogits_kernel(LogpBw
         if (tl == cc) v = v + g_logp;
         if (a.temperature) v = v * inv_t;
         d[e] = v;
+        if constexpr (BIAS_GRAD) cur[cc] = group16_sum(live ? v : 0.f);
       }
       packed[c >> 1] = pack_bf16x2(d[0], d[1]);
     }
+    if constexpr (BIAS_GRAD) {
+      // binary-counter merge: group jm closes every tree node whose last group it is
+#pragma unroll
+      for (int L = 0; L < kLevels; ++L) {
+        if (((jm >> L) & 1) == 0) {
+#pragma unroll
+          for (int c = 0; c < 16; ++c) level[L][c] = cur[c];
+          break;
+        }
+#pragma unroll
+        for (int c = 0; c < 16; ++c) cur[c] = level[L][c] + cur[c];
+      }
+    }
+    if (!live) continue;
     bf16_bits* dst = a.dz + (int64_t)m * a.ld_dz + col0;
     if (col0 + 16 <= a.V) {
       *reinterpret_cast<u32x4_t*>(dst) = u32x4_t{packed[0], packed[1], packed[2], packed[3]};
@@ -122,37 +161,50 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_dlogits_kernel(LogpBw
         if (col0 + c < a.V) dst[c] = (bf16_bits)((packed[c >> 1] >> ((c & 1) * 16)) & 0xffffu);
     }
   }
+
+  if constexpr (BIAS_GRAD) {
+    // A lane's node covers its wave's S::TM groups and sits in the slot of that size; the waves along the
+    // token axis hold consecutive nodes and are added in pairs through LDS (the main loop ended on a
+    // barrier, so the staging memory is free).
+    constexpr int kTop = S::TM >= 8 ? 3 : S::TM >= 4 ? 2 : S::TM >= 2 ? 1 : 0;
+    static_assert(S::WM == 1 || S::WM == 2, "one or two waves along the token axis");
+    float* sums = reinterpret_cast<float*>(lds);  // [WM][256 columns]
+    if (l16 == 0) {
+#pragma unroll
+      for (int c = 0; c < 16; ++c) sums[wave_m * kLogpTileCols + (wave_n * 4 + grp) * 16 + c] = level[kTop][c];
+    }
+    __syncthreads();
+    for (int col = threadIdx.x; col < kLogpTileCols; col += S::kThreads) {
+      float total = sums[col];
+      if constexpr (S::WM == 2) total = total + sums[kLogpTileCols + col];
+      if (v0 + col < a.V) a.bias_part[(int64_t)tile_m * a.V + v0 + col] = total;
+    }
+  }
 }
 
-// grad_bias, step 1: fp32 sums of 256-token blocks, tokens ascending. One thread per column pair.
+// grad_bias from the per-tile column sums: the `per_block` tiles of a 256-token block are added in the
+// balanced tree that continues the in-kernel one (adjacent pairs first, a tile past the last one is +0),
+// then the block sums ascending.
 constexpr int kBiasBlockTokens = 256;
 
-__global__ void logp_bias_block_sums_kernel(const bf16_bits* __restrict__ dz, int64_t ld, float* __restrict__ part,
-                                            int T, int V) {
-  const int pair = blockIdx.x * blockDim.x + threadIdx.x;
-  const int col = pair * 2;
-  if (col >= V) return;
-  const int t0 = blockIdx.y * kBiasBlockTokens;
-  const int t1 = (t0 + kBiasBlockTokens < T) ? t0 + kBiasBlockTokens : T;
-  const bool two = col + 1 < V;
-  float s0 = 0.f, s1 = 0.f;
-  for (int t = t0; t < t1; ++t) {
-    const bf16_bits* row = dz + (int64_t)t * ld + col;
-    s0 = s0 + __uint_as_float((uint32_t)row[0] << 16);
-    if (two) s1 = s1 + __uint_as_float((uint32_t)row[1] << 16);
-  }
-  float* out = part + (int64_t)blockIdx.y * V + col;
-  out[0] = s0;
-  if (two) out[1] = s1;
-}
-
-// grad_bias, step 2: block sums added ascending.
-__global__ void logp_bias_merge_kernel(const float* __restrict__ part, float* __restrict__ grad_bias, int blocks,
-                                       int V) {
+__global__ void logp_bias_merge_kernel(const float* __restrict__ part, float* __restrict__ grad_bias, int tiles,
+                                       int per_block, int V) {
   const int col = blockIdx.x * blockDim.x + threadIdx.x;
   if (col >= V) return;
   float s = 0.f;
-  for (int b = 0; b < blocks; ++b) s = s + part[(int64_t)b * V + col];
+  for (int t0 = 0; t0 < tiles; t0 += per_block) {
+    float node[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) node[i] = (i < per_block && t0 + i < tiles) ? part[(int64_t)(t0 + i) * V + col] : 0.f;
+#pragma unroll
+    for (int w = 1; w < 16; w *= 2) {
+      if (w < per_block) {
+#pragma unroll
+        for (int i = 0; i < 16; i += 2 * w) node[i] = node[i] + node[i + w];
+      }
+    }
+    s = s + node[0];
+  }
   grad_bias[col] = s;
 }
 
@@ -173,15 +225,22 @@ static size_t dz_bytes(int T, int V) {
   return (raw + 255) / 256 * 256;
 }
 
+// Token tiles the bias gradient may be collected over: 16-token tiles up to 1024 tokens, else 64-token ones.
+constexpr int kBiasSmallTileMaxTokens = 1024;
+
+static int bias_part_rows(int T) { return T <= kBiasSmallTileMaxTokens ? (T + 15) / 16 : (T + 63) / 64; }
+
 size_t linear_logp_bwd_workspace_bytes(int T, int V, bool with_bias) {
   size_t bytes = dz_bytes(T, V);
-  if (with_bias && T > 0) bytes += (size_t)((T + kBiasBlockTokens - 1) / kBiasBlockTokens) * (size_t)V * sizeof(float);
+  if (with_bias && T > 0) bytes += (size_t)bias_part_rows(T) * (size_t)V * sizeof(float);
   return bytes;
 }
 
-template <class S, int LOOP>
-static hipError_t launch_dlogits(LogpBwdArgs a, hipStream_t stream) {
-  auto kernel = linear_logp_dlogits_kernel<S, LOOP>;
+template <class S, int LOOP, bool BIAS_GRAD>
+static hipError_t launch_dlogits_as(LogpBwdArgs a, hipStream_t stream) {
+  auto kernel = linear_logp_dlogits_kernel<S, LOOP, BIAS_GRAD>;
+  constexpr int kSumBytes = 2 * kLogpTileCols * (int)sizeof(float);
+  static_assert(S::kLdsBytes >= kSumBytes, "the column sums reuse the staging memory");
   static PerDeviceOnce once;
   hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), S::kLdsBytes, once);
   if (err != hipSuccess) return err;
@@ -190,6 +249,11 @@ static hipError_t launch_dlogits(LogpBwdArgs a, hipStream_t stream) {
   a.group_m = a.tiles_m < 8 ? a.tiles_m : 8;
   hipLaunchKernelGGL(kernel, dim3(a.tiles_m * a.tiles_v), dim3(S::kThreads), S::kLdsBytes, stream, a);
   return hipGetLastError();
+}
+
+template <class S, int LOOP>
+static hipError_t launch_dlogits(LogpBwdArgs a, hipStream_t stream) {
+  return a.bias_part ? launch_dlogits_as<S, LOOP, true>(a, stream) : launch_dlogits_as<S, LOOP, false>(a, stream);
 }
 
 hipError_t linear_logp_bwd_launch(const MatView& H, const MatView& W, const int64_t* target, const float* bias,
@@ -215,6 +279,7 @@ hipError_t linear_logp_bwd_launch(const MatView& H, const MatView& W, const int6
   a.vocab_start = vocab_start;
   a.tiles_m = a.tiles_v = 0;
   a.group_m = 1;
+  a.bias_part = grad_bias ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + dz_bytes(T, V)) : nullptr;
 
   const bool vec = W.k_stride == 1 && H.k_stride == 1 && (W.row_stride % kChunkElems) == 0 &&
                    (H.row_stride % kChunkElems) == 0 && (reinterpret_cast<uintptr_t>(W.ptr) & 15) == 0 &&
@@ -227,6 +292,9 @@ hipError_t linear_logp_bwd_launch(const MatView& H, const MatView& W, const int6
   if (config == RLK_LOGP_CFG_128_STREAMS) config = RLK_LOGP_CFG_128;
   if (config == RLK_LOGP_CFG_256_STREAMS) config = RLK_LOGP_CFG_256;
   if (!vec && config == RLK_LOGP_CFG_256) config = RLK_LOGP_CFG_128;
+  // the bias-gradient partials of 16-token tiles only fit the workspace up to kBiasSmallTileMaxTokens
+  if (grad_bias && config == RLK_LOGP_CFG_16 && T > kBiasSmallTileMaxTokens) config = RLK_LOGP_CFG_64;
+  const int tile_tokens = config == RLK_LOGP_CFG_256 ? 256 : config == RLK_LOGP_CFG_128 ? 128 : config == RLK_LOGP_CFG_64 ? 64 : 16;
   const int loop = !vec ? 0 : (D % kTileK == 0 && !force_staged) ? 2 : 1;
   hipError_t err;
   switch (config) {
@@ -267,14 +335,9 @@ hipError_t linear_logp_bwd_launch(const MatView& H, const MatView& W, const int6
     if (err != hipSuccess) return err;
   }
   if (grad_bias) {
-    float* part = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + dz_bytes(T, V));
-    const int blocks = (T + kBiasBlockTokens - 1) / kBiasBlockTokens;
-    const int pairs = (V + 1) / 2;
-    hipLaunchKernelGGL(logp_bias_block_sums_kernel, dim3((pairs + 255) / 256, blocks), dim3(256), 0, stream, a.dz,
-                       a.ld_dz, part, T, V);
-    err = hipGetLastError();
-    if (err != hipSuccess) return err;
-    hipLaunchKernelGGL(logp_bias_merge_kernel, dim3((V + 255) / 256), dim3(256), 0, stream, part, grad_bias, blocks, V);
+    const int tiles = (T + tile_tokens - 1) / tile_tokens;
+    hipLaunchKernelGGL(logp_bias_merge_kernel, dim3((V + 255) / 256), dim3(256), 0, stream, a.bias_part, grad_bias,
+                       tiles, kBiasBlockTokens / tile_tokens, V);
     err = hipGetLastError();
   }
   return err;

@@ -25,14 +25,34 @@ __device__ __forceinline__ float round_through_bf16(float v) { return bf16_to_f3
 __device__ __forceinline__ float sigmoid_f32(float x) { return __builtin_amdgcn_rcpf(1.0f + pinned_exp(-x)); }
 __device__ __forceinline__ float swiglu_f32(float g, float u) { return (g * sigmoid_f32(g)) * u; }
 
-// The scaled logit y of the contract for accumulator value z at column `col`:
-// bias added, padded lanes -inf, then the temperature scaling.
+// The logit of the contract before the temperature: accumulator value z at column `col` with the bias
+// added and padded lanes set to -inf. This is the value a caller who asks for the logits receives.
+__device__ __forceinline__ float biased_logit(float z, bool has_bias, float bias, int col, int vocab_limit) {
+  if (has_bias) z = z + bias;
+  return (col < vocab_limit) ? z : kNegInf;
+}
+
+// The scaled logit y of the contract: the biased logit, then the temperature scaling.
 __device__ __forceinline__ float scaled_logit(float z, bool has_bias, float bias, int col, int vocab_limit,
                                               bool has_temp, float inv_t) {
-  if (has_bias) z = z + bias;
-  z = (col < vocab_limit) ? z : kNegInf;
+  z = biased_logit(z, has_bias, bias, col, vocab_limit);
   if (has_temp) z = z * inv_t;
   return z;
+}
+
+// A lane's run of 16 consecutive biased logits of one token -> row[col0 .. col0 + 16) of the fp32 logits,
+// cut at V: four 16-byte stores when the run is whole and aligned, element stores otherwise.
+__device__ __forceinline__ void store_logit_run(float* __restrict__ row, int col0, int V, const float (&u)[16]) {
+  float* dst = row + col0;
+  if (col0 + 16 <= V && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      *reinterpret_cast<f32x4_t*>(dst + 4 * q) = f32x4_t{u[4 * q], u[4 * q + 1], u[4 * q + 2], u[4 * q + 3]};
+  } else {
+#pragma unroll
+    for (int c = 0; c < 16; ++c)
+      if (col0 + c < V) dst[c] = u[c];
+  }
 }
 
 // One step of a stream's online chain: the 16 scaled logits y of the stream's run in one

@@ -169,6 +169,47 @@ int rlk_det_gemm_tree_bf16_config(const void* a, int64_t a_row_stride, int64_t a
   return err == hipSuccess ? RLK_OK : device_error("rlk_det_gemm_tree_bf16", err);
 }
 
+const char* rlk_det_gemm_seq_contract_id(void) { return "rlkernel.det_gemm.hip_seqfma32_gfx950.v1"; }
+
+int rlk_det_gemm_seq(const void* a, int a_dtype, int64_t a_row_stride, int64_t a_k_stride, const void* b, int b_dtype,
+                     int64_t b_k_stride, int64_t b_n_stride, void* c, int c_dtype, int64_t ldc, int M, int N, int K,
+                     void* stream) {
+  if (M < 0 || N < 0 || K < 0) {
+    set_last_error("rlk_det_gemm_seq: negative size M=%d N=%d K=%d", M, N, K);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  auto operand_ok = [](int dtype) { return dtype == RLK_DTYPE_BF16 || dtype == RLK_DTYPE_FP32; };
+  if (!operand_ok(a_dtype) || !operand_ok(b_dtype) || !operand_ok(c_dtype)) {
+    set_last_error("rlk_det_gemm_seq: operands and output must be bf16 or fp32 (a=%d b=%d c=%d)", a_dtype, b_dtype,
+                   c_dtype);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (a_row_stride < 0 || a_k_stride < 0 || b_k_stride < 0 || b_n_stride < 0) {
+    set_last_error("rlk_det_gemm_seq: operands must not use negative strides");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (M == 0 || N == 0) return RLK_OK;
+  if (c == nullptr || ldc < N) {
+    set_last_error("rlk_det_gemm_seq: output needs a non-null pointer and ldc >= N (ldc=%lld N=%d)", (long long)ldc, N);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const bool out_bf16 = c_dtype == RLK_DTYPE_BF16;
+  if (K == 0) {
+    hipError_t err = fill_zero_launch(c, M, N, ldc, out_bf16 ? 2 : 4, s);
+    return err == hipSuccess ? RLK_OK : device_error("rlk_det_gemm_seq(fill)", err);
+  }
+  if (a == nullptr || b == nullptr) {
+    set_last_error("rlk_det_gemm_seq: null operand");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  SeqOperand A{a, a_row_stride, a_k_stride};
+  SeqOperand B{b, b_n_stride, b_k_stride};
+  hipError_t err = det_gemm_seq_launch(A, a_dtype == RLK_DTYPE_FP32, B, b_dtype == RLK_DTYPE_FP32, c, ldc, M, N, K,
+                                       out_bf16, s);
+  return err == hipSuccess ? RLK_OK : device_error("rlk_det_gemm_seq", err);
+}
+
 const char* rlk_linear_logp_contract_id(void) { return "rlkernel.linear_logp.hip_streams16x256_split1024_gfx950.v1"; }
 
 int rlk_linear_logp_split_count(int V) { return V > 0 ? linear_logp_split_count(V) : 0; }
@@ -182,7 +223,8 @@ static int linear_logp_fwd_checked(const char* who, const void* hidden, int64_t 
                                    int64_t w_row_stride, const int64_t* target, const float* bias,
                                    const float* temperature, float* logp, float* lse, float* target_logit,
                                    void* workspace, size_t workspace_bytes, int T, int D, int V, int64_t vocab_start,
-                                   int real_vocab_end, int config, void* stream) {
+                                   int real_vocab_end, int config, void* stream, float* logits = nullptr,
+                                   int64_t logits_row_stride = 0) {
   if (T < 0 || D <= 0 || V <= 0) {
     set_last_error("%s: bad sizes T=%d D=%d V=%d", who, T, D, V);
     return RLK_ERR_INVALID_ARGUMENT;
@@ -204,6 +246,10 @@ static int linear_logp_fwd_checked(const char* who, const void* hidden, int64_t 
     set_last_error("%s: row strides must be >= D", who);
     return RLK_ERR_INVALID_ARGUMENT;
   }
+  if (logits != nullptr && logits_row_stride < V) {
+    set_last_error("%s: logits row stride must be >= V", who);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
   const size_t need = linear_logp_workspace_bytes(T, V);
   if (workspace == nullptr || workspace_bytes < need) {
     set_last_error("%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
@@ -211,9 +257,9 @@ static int linear_logp_fwd_checked(const char* who, const void* hidden, int64_t 
   }
   MatView H{reinterpret_cast<const bf16_bits*>(hidden), h_row_stride, 1, T};
   MatView W{reinterpret_cast<const bf16_bits*>(weight), w_row_stride, 1, V};
-  hipError_t err = linear_logp_launch(H, W, target, bias, temperature, logp, lse, target_logit,
-                                      reinterpret_cast<float*>(workspace), T, D, V, vocab_start, real_vocab_end,
-                                      config, reinterpret_cast<hipStream_t>(stream));
+  hipError_t err = linear_logp_launch(H, W, target, bias, temperature, logp, lse, target_logit, logits,
+                                      logits_row_stride, reinterpret_cast<float*>(workspace), T, D, V, vocab_start,
+                                      real_vocab_end, config, reinterpret_cast<hipStream_t>(stream));
   return err == hipSuccess ? RLK_OK : device_error(who, err);
 }
 
@@ -224,6 +270,20 @@ int rlk_linear_logp_fwd(const void* hidden, int64_t h_row_stride, const void* we
   return linear_logp_fwd_checked("rlk_linear_logp_fwd", hidden, h_row_stride, weight, w_row_stride, target, bias,
                                  temperature, logp, lse, nullptr, workspace, workspace_bytes, T, D, V, vocab_start,
                                  real_vocab_end, config, stream);
+}
+
+int rlk_linear_logp_fwd_logits(const void* hidden, int64_t h_row_stride, const void* weight, int64_t w_row_stride,
+                               const int64_t* target, const float* bias, const float* temperature, float* logp,
+                               float* lse, float* logits, int64_t logits_row_stride, void* workspace,
+                               size_t workspace_bytes, int T, int D, int V, int64_t vocab_start, int real_vocab_end,
+                               int config, void* stream) {
+  if (logits == nullptr && T > 0) {
+    set_last_error("rlk_linear_logp_fwd_logits: null logits (use rlk_linear_logp_fwd when they are not wanted)");
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  return linear_logp_fwd_checked("rlk_linear_logp_fwd_logits", hidden, h_row_stride, weight, w_row_stride, target,
+                                 bias, temperature, logp, lse, nullptr, workspace, workspace_bytes, T, D, V,
+                                 vocab_start, real_vocab_end, config, stream, logits, logits_row_stride);
 }
 
 int rlk_linear_logp_fwd_shard(const void* hidden, int64_t h_row_stride, const void* weight, int64_t w_row_stride,

@@ -44,6 +44,17 @@ int det_gemm_tree_max_k();
 hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int64_t ldc, int M, int N, int K,
                                 int config, hipStream_t stream);
 
+// The strictly sequential fp32 chain (one fused multiply-add per k, ascending, no rounding below fp32).
+// An operand is bf16 or fp32, addressed as ptr[row * row_stride + k * k_stride] in elements; B holds one
+// row per output column. C is fp32 [M, ldc], or bf16 when out_bf16. K >= 1.
+struct SeqOperand {
+  const void* ptr;
+  int64_t row_stride;
+  int64_t k_stride;
+};
+hipError_t det_gemm_seq_launch(const SeqOperand& A, bool a_f32, const SeqOperand& B, bool b_f32, void* C, int64_t ldc,
+                               int M, int N, int K, bool out_bf16, hipStream_t stream);
+
 // Up to 64 tokens, unit K stride, 16-byte aligned rows, K % 64 == 0. `shallow`: M <= 16 with
 // two workgroups per CU.
 hipError_t det_gemm_stream_launch(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
@@ -61,11 +72,13 @@ size_t linear_logp_workspace_bytes(int T, int V);
 
 // H[T,D] hidden states, W[V,D] lm_head weight; workspace holds
 // linear_logp_workspace_bytes(T, V) bytes of fp32 partials. logp, lse and target_logit
-// (the unclamped scaled logit of a target this weight owns, else 0) may each be null.
+// (the unclamped scaled logit of a target this weight owns, else 0) may each be null, and so may
+// logits ([T, logits_ld] fp32: the accumulators with the bias added and padded lanes -inf, before
+// the temperature, stored by the same pass).
 hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t* target, const float* bias,
                               const float* temperature, float* logp, float* lse, float* target_logit,
-                              float* workspace, int T, int D, int V, int64_t vocab_start, int vocab_limit, int config,
-                              hipStream_t stream);
+                              float* logits, int64_t logits_ld, float* workspace, int T, int D, int V,
+                              int64_t vocab_start, int vocab_limit, int config, hipStream_t stream);
 
 // Ascending merge of (max, sum, target logit) partials laid out [3][n_split][T] into
 // lse = M + log(S), logp = target - lse (clamped at 0 when `clamp`) and the merged target

@@ -156,6 +156,52 @@ def det_gemm_fwd_out_fp32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     return gemm_strided(a, b, out)
 
 
+_SEQ_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float32: _lib.DTYPE_FP32}
+
+
+def det_gemm_seq(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """``a[M,K] @ b[K,N]`` with one fp32 fused multiply-add per k, k ascending, nothing rounded below fp32;
+    bf16 or fp32 operands (any strides), fp32 result or one rounding to bf16 (rlk_det_gemm_seq)."""
+    for name, t in (("A", a), ("B", b)):
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} must be CUDA")
+        if t.dtype not in _SEQ_DTYPES:
+            raise RuntimeError(f"{name} must be bf16 or fp32")
+    if a.dim() != 2 or b.dim() != 2:
+        raise RuntimeError("det_gemm_fwd_fp32: expect 2D [M,K]@[K,N]")
+    if b.size(0) != a.size(1):
+        raise RuntimeError("det_gemm_fwd_fp32: K mismatch")
+    if out_dtype not in _SEQ_DTYPES:
+        raise RuntimeError("det_gemm_fwd_fp32: output must be bf16 or fp32")
+    m, k = a.shape
+    n = b.size(1)
+    out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+    if m == 0 or n == 0:
+        return out
+    with torch.cuda.device(a.device):
+        status = _lib.load().rlk_det_gemm_seq(
+            a.data_ptr(), _SEQ_DTYPES[a.dtype], a.stride(0), a.stride(1), b.data_ptr(), _SEQ_DTYPES[b.dtype],
+            b.stride(0), b.stride(1), out.data_ptr(), _SEQ_DTYPES[out_dtype], n, m, n, k, _stream_handle(a.device),
+        )  # fmt: skip
+    _lib.check(status, "rlk_det_gemm_seq failed")
+    return out
+
+
+def det_gemm_fwd_fp32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """fp32 ``a @ b`` from bf16 or fp32 operands, sequential fp32 chain (rl_engine/_C.pyi:244;
+    csrc/musa/det_gemm.mu:25-48)."""
+    return det_gemm_seq(a, b, torch.float32)
+
+
+def det_gemm_accum_fwd_fp32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """The same chain, result rounded once to the dtype of ``a`` (rl_engine/_C.pyi:245-248)."""
+    return det_gemm_seq(a, b, a.dtype if a.dtype in _SEQ_DTYPES else torch.float32)
+
+
+# the name the facade uses for the fp32-result path
+det_gemm_seq_fp32 = det_gemm_fwd_fp32
+
+
 def _reduction_major(t: torch.Tensor) -> torch.Tensor:
     """``t.t()`` ready for a GEMM whose reduction runs over ``t``'s rows.
 
@@ -239,11 +285,12 @@ def _linear_logp_forward(
     real_vocab_size: int,
     vocab_start_index: int,
     config: int,
+    want_logits: bool = False,
 ):
     """Checks shared by the fused linear-LogP entries, then one call of ``entry`` in the C ABI.
 
-    Returns ``(first, lse, bias_f32, real_vocab)``; ``first`` is logp or the target
-    logit, whichever ``entry`` writes."""
+    Returns ``(first, lse, logits)``; ``first`` is logp or the target logit, whichever ``entry``
+    writes; ``logits`` is the fp32 ``[N, V]`` tensor the same pass stored when ``want_logits``, else None."""
     if not hidden.is_cuda or not weight.is_cuda or not target.is_cuda:
         raise RuntimeError(f"{who}: hidden, weight and target must be CUDA tensors")
     if hidden.dtype != _BF16 or weight.dtype != _BF16:
@@ -276,32 +323,25 @@ def _linear_logp_forward(
     lib = _lib.load()
     first = torch.empty((n,), dtype=torch.float32, device=hidden.device)
     lse = torch.empty((n,), dtype=torch.float32, device=hidden.device)
+    logits = torch.empty((n, v), dtype=torch.float32, device=hidden.device) if want_logits else None
     ws_bytes = int(lib.rlk_linear_logp_workspace_bytes(n, v))
     workspace = torch.empty((max(ws_bytes, 4) // 4,), dtype=torch.float32, device=hidden.device)
     if n > 0:
+        head = (
+            hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), target_i64.data_ptr(),
+            bias_f32.data_ptr() if bias_f32 is not None else None,
+            temp_f32.data_ptr() if temp_f32 is not None else None,
+            first.data_ptr(), lse.data_ptr(),
+        )  # fmt: skip
+        tail = (workspace.data_ptr(), ws_bytes, n, d, v, int(vocab_start_index), real_vocab, config, _stream_handle(hidden.device))
         with torch.cuda.device(hidden.device):
-            status = getattr(lib, entry)(
-                hidden.data_ptr(),
-                hidden.stride(0),
-                weight.data_ptr(),
-                weight.stride(0),
-                target_i64.data_ptr(),
-                bias_f32.data_ptr() if bias_f32 is not None else None,
-                temp_f32.data_ptr() if temp_f32 is not None else None,
-                first.data_ptr(),
-                lse.data_ptr(),
-                workspace.data_ptr(),
-                ws_bytes,
-                n,
-                d,
-                v,
-                int(vocab_start_index),
-                real_vocab,
-                config,
-                _stream_handle(hidden.device),
-            )
+            if want_logits:  # the logits come out of the same pass: entry + "_logits"
+                entry = entry + "_logits"
+                status = getattr(lib, entry)(*head, logits.data_ptr(), logits.stride(0), *tail)
+            else:
+                status = getattr(lib, entry)(*head, *tail)
         _lib.check(status, f"{entry} failed")
-    return first, lse, bias_f32, real_vocab
+    return first, lse, logits
 
 
 def fused_linear_logp(
@@ -320,25 +360,15 @@ def fused_linear_logp(
 
     Same arguments, checks and return convention as ``_C.fused_linear_logp_sm90``
     (csrc/bindings/ops.cpp:514-520; csrc/cuda/logprob/fused_linear_logp_sm90.cu:2040-2176).
-    ``return_logits=True`` appends the unscaled fp32 logits ``[N, V]`` (bias
-    applied, padded lanes -inf) computed by the same MFMA chain through
-    rlk_det_gemm_bf16 with fp32 output; it does not change logp / lse.
+    ``return_logits=True`` appends the unscaled fp32 logits ``[N, V]`` (bias applied, padded
+    lanes -inf), stored by the same kernel pass from the accumulators the reduction sees
+    (rlk_linear_logp_fwd_logits; no second GEMM); it does not change logp / lse.
     """
-    logp, lse, bias_f32, real_vocab = _linear_logp_forward(
+    logp, lse, logits = _linear_logp_forward(
         "fused_linear_logp", "rlk_linear_logp_fwd", hidden, weight, target, bias, temperature,
-        real_vocab_size, vocab_start_index, config,
+        real_vocab_size, vocab_start_index, config, want_logits=bool(return_logits),
     )  # fmt: skip
-    outputs = [logp, lse]
-    if return_logits:
-        n, v = hidden.size(0), weight.size(0)
-        logits = torch.empty((n, v), dtype=torch.float32, device=hidden.device)
-        gemm_strided(hidden, weight.t(), logits)
-        if bias_f32 is not None:
-            logits += bias_f32
-        if real_vocab < v:
-            logits[:, real_vocab:] = float("-inf")
-        outputs.append(logits)
-    return outputs
+    return [logp, lse, logits] if return_logits else [logp, lse]
 
 
 # The name the reference's CUDA build binds the same function under (csrc/bindings/ops.cpp:514).
@@ -365,7 +395,7 @@ def fused_linear_logp_sm90_global_target(
     Argument order and return convention of ``_C.fused_linear_logp_sm90_global_target``
     (csrc/bindings/ops.cpp:522-526; csrc/cuda/logprob/fused_linear_logp_sm90.cu:2169-2176).
     """
-    target_logit, lse, _, _ = _linear_logp_forward(
+    target_logit, lse, _ = _linear_logp_forward(
         "fused_linear_logp_sm90_global_target", "rlk_linear_logp_fwd_shard", hidden, weight, target, bias,
         temperature, real_vocab_size, vocab_start_index, config,
     )  # fmt: skip

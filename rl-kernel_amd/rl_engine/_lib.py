@@ -57,10 +57,13 @@ EXPORTED_SYMBOLS = (
     "rlk_det_gemm_tree_bf16",
     "rlk_det_gemm_tree_bf16_config",
     "rlk_det_gemm_tree_contract_id",
+    "rlk_det_gemm_seq",
+    "rlk_det_gemm_seq_contract_id",
     "rlk_linear_logp_contract_id",
     "rlk_linear_logp_split_count",
     "rlk_linear_logp_workspace_bytes",
     "rlk_linear_logp_fwd",
+    "rlk_linear_logp_fwd_logits",
     "rlk_linear_logp_fwd_shard",
     "rlk_linear_logp_fwd_noalloc",
     "rlk_linear_logp_bwd_workspace_bytes",
@@ -120,6 +123,10 @@ def load() -> ctypes.CDLL:
     lib.rlk_det_gemm_tree_bf16_config.argtypes = [vp, i64, i64, vp, i64, i64, vp, i64, i32, i32, i32, i32, vp]
     lib.rlk_det_gemm_tree_contract_id.restype = c.c_char_p
     lib.rlk_det_gemm_tree_contract_id.argtypes = []
+    lib.rlk_det_gemm_seq.restype = i32
+    lib.rlk_det_gemm_seq.argtypes = [vp, i32, i64, i64, vp, i32, i64, i64, vp, i32, i64, i32, i32, i32, vp]
+    lib.rlk_det_gemm_seq_contract_id.restype = c.c_char_p
+    lib.rlk_det_gemm_seq_contract_id.argtypes = []
     lib.rlk_det_gemm_pick_config.restype = i32
     lib.rlk_det_gemm_pick_config.argtypes = [i32, i32, i32]
 
@@ -133,6 +140,10 @@ def load() -> ctypes.CDLL:
     lib.rlk_linear_logp_fwd.argtypes = [vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, sz, i32, i32, i32, i64, i32, i32, vp]
     lib.rlk_linear_logp_fwd_shard.restype = i32
     lib.rlk_linear_logp_fwd_shard.argtypes = lib.rlk_linear_logp_fwd.argtypes
+    lib.rlk_linear_logp_fwd_logits.restype = i32
+    lib.rlk_linear_logp_fwd_logits.argtypes = [
+        vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, i64, vp, sz, i32, i32, i32, i64, i32, i32, vp,
+    ]  # fmt: skip
     lib.rlk_linear_logp_fwd_noalloc.restype = i32
     lib.rlk_linear_logp_fwd_noalloc.argtypes = [vp, i64, vp, i64, vp, vp, vp, vp, vp, i32, i32, i32, i64, i32, i32, vp]
 

@@ -20,6 +20,7 @@ import torch
 from torch import Tensor
 
 from rl_engine import _C, _lib
+from rl_engine._checks import enforce
 from rl_engine.backends.rocm.gemm import swiglu_gemm
 from rl_engine.backends.rocm.gemm.det_gemm import (
     det_gemm_linear,
@@ -41,44 +42,32 @@ def _single_rank(group: Any, name: str) -> None:
 
 
 def _validate_ffn_inputs(rmsnorm_output, gate_weight, up_weight, down_weight, fused_gate_up_weight) -> None:
-    """Same checks and messages as _validate_ffn_inputs (ffn.py:585-640 of the reference)."""
-    tensors = {
-        "rmsnorm_output": rmsnorm_output,
-        "gate_weight": gate_weight,
-        "up_weight": up_weight,
-        "down_weight": down_weight,
-    }
+    """The checks, exception types and messages of the reference's _validate_ffn_inputs (ffn.py:585-640),
+    written as one table per stage: argument types, ranks, shapes, then dtype and placement of every tensor."""
+    named = [("rmsnorm_output", rmsnorm_output), ("gate_weight", gate_weight), ("up_weight", up_weight),
+             ("down_weight", down_weight)]  # fmt: skip
     if fused_gate_up_weight is not None:
-        tensors["fused_gate_up_weight"] = fused_gate_up_weight
-    for name, tensor in tensors.items():
-        if not isinstance(tensor, Tensor):
-            raise TypeError(f"{name} must be a torch.Tensor, got {type(tensor)!r}.")
-    if rmsnorm_output.dim() < 1:
-        raise ValueError("rmsnorm_output must have at least one dimension.")
-    if rmsnorm_output.numel() == 0:
-        raise ValueError("rmsnorm_output must contain at least one token.")
-    for name in ("gate_weight", "up_weight", "down_weight"):
-        if tensors[name].dim() != 2:
-            raise ValueError(f"{name} must be 2-D, got shape {tuple(tensors[name].shape)}.")
-    hidden_size = rmsnorm_output.size(-1)
-    intermediate_size = gate_weight.size(0)
-    expected = {
-        "gate_weight": (intermediate_size, hidden_size),
-        "up_weight": (intermediate_size, hidden_size),
-        "down_weight": (hidden_size, intermediate_size),
-    }
-    if fused_gate_up_weight is not None:
-        expected["fused_gate_up_weight"] = (2 * intermediate_size, hidden_size)
-    for name, shape in expected.items():
-        if tuple(tensors[name].shape) != shape:
-            raise ValueError(f"{name} must have shape {shape}, got {tuple(tensors[name].shape)}.")
-    for name, tensor in tensors.items():
-        if tensor.dtype != torch.bfloat16:
-            raise TypeError(f"{name} must have dtype bfloat16, got {tensor.dtype}.")
-        if not tensor.is_cuda:
-            raise RuntimeError(f"{name} must be on a CUDA/ROCm GPU device, got '{tensor.device}'.")
-        if tensor.device != rmsnorm_output.device:
-            raise RuntimeError(f"all FFN inputs must be on {rmsnorm_output.device}, got {name} on {tensor.device}.")
+        named.append(("fused_gate_up_weight", fused_gate_up_weight))
+    enforce((isinstance(t, Tensor), TypeError, f"{name} must be a torch.Tensor, got {type(t)!r}.") for name, t in named)
+    enforce([
+        (rmsnorm_output.dim() >= 1, ValueError, "rmsnorm_output must have at least one dimension."),
+        (rmsnorm_output.numel() > 0, ValueError, "rmsnorm_output must contain at least one token."),
+    ])  # fmt: skip
+    enforce((t.dim() == 2, ValueError, f"{name} must be 2-D, got shape {tuple(t.shape)}.") for name, t in named[1:4])
+    hidden, inter = rmsnorm_output.size(-1), gate_weight.size(0)
+    wanted = {"gate_weight": (inter, hidden), "up_weight": (inter, hidden), "down_weight": (hidden, inter),
+              "fused_gate_up_weight": (2 * inter, hidden)}  # fmt: skip
+    enforce(
+        (tuple(t.shape) == wanted[name], ValueError, f"{name} must have shape {wanted[name]}, got {tuple(t.shape)}.")
+        for name, t in named[1:]
+    )
+    home = rmsnorm_output.device
+    for name, t in named:
+        enforce([
+            (t.dtype == torch.bfloat16, TypeError, f"{name} must have dtype bfloat16, got {t.dtype}."),
+            (t.is_cuda, RuntimeError, f"{name} must be on a CUDA/ROCm GPU device, got '{t.device}'."),
+            (t.device == home, RuntimeError, f"all FFN inputs must be on {home}, got {name} on {t.device}."),
+        ])  # fmt: skip
 
 
 # ---------------------------------------------------------------------------
@@ -108,7 +97,7 @@ def _(rmsnorm_output, fused_gate_up_weight, down_weight):
 
 @torch.library.custom_op("rl_kernel::qwen3_ffn_packed_inference_to_staging", mutates_args={"output"})
 def _qwen3_ffn_packed_inference_to_staging(
-    rmsnorm_output: Tensor, fused_gate_up_weight: Tensor, down_weight: Tensor, output: Tensor
+    rmsnorm_output: Tensor, fused_gate_up_weight: Tensor, down_weight: Tensor, output: Tensor,
 ) -> None:
     """Same with the down projection written into a caller-owned staging buffer."""
     hidden_2d = rmsnorm_output.reshape(-1, rmsnorm_output.shape[-1]).contiguous()
@@ -121,25 +110,18 @@ def _(rmsnorm_output, fused_gate_up_weight, down_weight, output):
 
 
 def qwen3_ffn_packed_inference(
-    rmsnorm_output: Tensor,
-    fused_gate_up_weight: Tensor,
-    down_weight: Tensor,
-    *,
-    collective_handle: int = 0,
-    tp_world_size: int = 1,
-    collective: Any | None = None,
+    rmsnorm_output: Tensor, fused_gate_up_weight: Tensor, down_weight: Tensor, *, collective_handle: int = 0,
+    tp_world_size: int = 1, collective: Any | None = None,
 ) -> Tensor:
     """Inference-only packed FFN entry (ffn.py:303-330 of the reference), one rank."""
     del collective_handle, collective
     if tp_world_size != 1:
         raise RuntimeError("packed rollout FFN with tensor parallelism needs a collective; this build runs on one GPU")
-    for name, tensor in (
-        ("rmsnorm_output", rmsnorm_output),
-        ("fused_gate_up_weight", fused_gate_up_weight),
-        ("down_weight", down_weight),
-    ):
-        if tensor.dtype != torch.bfloat16:
-            raise TypeError(f"{name} must have dtype bfloat16, got {tensor.dtype}.")
+    operands = {"rmsnorm_output": rmsnorm_output, "fused_gate_up_weight": fused_gate_up_weight, "down_weight": down_weight}
+    enforce(
+        (t.dtype == torch.bfloat16, TypeError, f"{name} must have dtype bfloat16, got {t.dtype}.")
+        for name, t in operands.items()
+    )
     return torch.ops.rl_kernel.qwen3_ffn_packed_inference(rmsnorm_output, fused_gate_up_weight, down_weight)
 
 
@@ -193,17 +175,9 @@ class _DeterministicFFNFunction(torch.autograd.Function):
 
 
 def qwen3_ffn(
-    rmsnorm_output: Tensor,
-    gate_weight: Tensor,
-    up_weight: Tensor,
-    down_weight: Tensor,
-    *,
-    fused_gate_up_weight: Tensor | None = None,
-    tp_group: Any = None,
-    cp_group: Any = None,
-    sequence_parallel: bool = False,
-    deterministic: bool | None = None,
-    disable_split_k: bool | None = None,
+    rmsnorm_output: Tensor, gate_weight: Tensor, up_weight: Tensor, down_weight: Tensor, *,
+    fused_gate_up_weight: Tensor | None = None, tp_group: Any = None, cp_group: Any = None,
+    sequence_parallel: bool = False, deterministic: bool | None = None, disable_split_k: bool | None = None,
 ) -> Tensor:
     """SiLU-gated FFN ``down(swiglu(gate(x), up(x)))`` with deterministic forward and backward.
 

@@ -19,12 +19,14 @@ and invariant to the tensor-parallel degree of a K-sharded layer; about 20 times
 from __future__ import annotations
 
 import os
+import weakref
 from collections.abc import Callable, Iterable
 from threading import Lock
 
 import torch
 
 from rl_engine import _C, _lib
+from rl_engine._checks import enforce, output_buffer_rules
 
 _BACKEND_ENV = "RL_KERNEL_DET_GEMM_BACKEND"
 _AUTO_BACKEND = "auto"
@@ -42,8 +44,12 @@ _BACKEND_ALIASES = {
 }
 _ROUTE_REPORTED = False
 _ROUTE_REPORT_LOCK = Lock()
-_WEIGHT_TRANSPOSE_CACHE: dict[tuple[int, str, tuple[int, ...], torch.dtype], tuple[int | None, torch.Tensor]] = {}
-_WEIGHT_TRANSPOSE_CACHE_LIMIT = 256
+# Prepared [K,N] copies by source weight: what refresh_cached_weight_transposes re-copies. The kernels read
+# the native [N,K] layout directly, so no transpose is ever made behind the caller's back; the only
+# transposed buffers alive are the ones prepare_det_gemm_linear_weight handed out. They are held weakly:
+# a buffer the caller dropped is forgotten.
+_PREPARED_TRANSPOSES: dict[tuple[int, str, tuple[int, ...], torch.dtype], list[weakref.ReferenceType]] = {}
+_PREPARED_LOCK = Lock()
 
 
 def _resolve_backend_request(value: str) -> str:
@@ -103,28 +109,41 @@ def _report_strict_route_once() -> None:
 # ---------------------------------------------------------------------------
 
 
+def _operand_rules(a: torch.Tensor, b: torch.Tensor) -> list:
+    def strides_ok(t: torch.Tensor):
+        return lambda: min(t.stride()) >= 0
+
+    def one_unit_stride(t: torch.Tensor):
+        return lambda: t.numel() <= 1 or 1 in t.stride()
+
+    return [
+        (a.dim() == 2 and b.dim() == 2, ValueError, "MFMA GEMM expects two 2-D tensors"),
+        (lambda: a.size(1) == b.size(0), ValueError, lambda: f"MFMA GEMM K mismatch: {a.size(1)} and {b.size(0)}"),
+        (a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16, TypeError, "MFMA GEMM requires BF16 inputs"),
+        (a.is_cuda and b.is_cuda and a.device == b.device, RuntimeError, "MFMA GEMM inputs must share one ROCm device"),
+        (strides_ok(a), ValueError, "MFMA GEMM operand a must not use negative strides"),
+        (one_unit_stride(a), ValueError, "MFMA GEMM operand a needs one unit-stride dimension"),
+        (strides_ok(b), ValueError, "MFMA GEMM operand b must not use negative strides"),
+        (one_unit_stride(b), ValueError, "MFMA GEMM operand b needs one unit-stride dimension"),
+    ]
+
+
 def _validate_operands(a: torch.Tensor, b: torch.Tensor) -> None:
-    if a.dim() != 2 or b.dim() != 2:
-        raise ValueError("MFMA GEMM expects two 2-D tensors")
-    if a.size(1) != b.size(0):
-        raise ValueError(f"MFMA GEMM K mismatch: {a.size(1)} and {b.size(0)}")
-    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
-        raise TypeError("MFMA GEMM requires BF16 inputs")
-    if not a.is_cuda or not b.is_cuda or a.device != b.device:
-        raise RuntimeError("MFMA GEMM inputs must share one ROCm device")
-    for name, tensor in (("a", a), ("b", b)):
-        if min(tensor.stride()) < 0:
-            raise ValueError(f"MFMA GEMM operand {name} must not use negative strides")
-        if tensor.stride(0) != 1 and tensor.stride(1) != 1 and tensor.numel() > 1:
-            raise ValueError(f"MFMA GEMM operand {name} needs one unit-stride dimension")
+    enforce(_operand_rules(a, b))
+
+
+def _checked_output(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None) -> torch.Tensor:
+    """Operand checks of both contracts, then the caller's output buffer (checked) or a fresh one."""
+    enforce(_operand_rules(a, b))
+    shape = (a.size(0), b.size(1))
+    if out is None:
+        return torch.empty(shape, dtype=torch.bfloat16, device=a.device)
+    enforce(output_buffer_rules(out, shape, a.device, "MFMA GEMM"))
+    return out
 
 
 def mfma_gemm(
-    a: torch.Tensor,
-    b: torch.Tensor,
-    *,
-    out: torch.Tensor | None = None,
-    config: str | int | None = None,
+    a: torch.Tensor, b: torch.Tensor, *, out: torch.Tensor | None = None, config: str | int | None = None,
 ) -> torch.Tensor:
     """``a[M,K] @ b[K,N]`` in bf16 under the pinned MFMA contract.
 
@@ -133,27 +152,11 @@ def mfma_gemm(
     buffer with contiguous rows, for instance a narrowed staging view.
     ``config`` names a tile configuration; it never changes a result bit.
     """
-    _validate_operands(a, b)
-    m_size, k_size = a.shape
-    n_size = b.size(1)
-    if out is None:
-        out = torch.empty((m_size, n_size), dtype=torch.bfloat16, device=a.device)
-    else:
-        if tuple(out.shape) != (m_size, n_size):
-            raise ValueError(f"MFMA GEMM output must have shape {(m_size, n_size)}, got {tuple(out.shape)}")
-        if out.dtype != torch.bfloat16:
-            raise TypeError(f"MFMA GEMM output must be BF16, got {out.dtype}")
-        if out.device != a.device:
-            raise RuntimeError("MFMA GEMM output must live on the input device")
-        if out.stride(1) != 1:
-            raise ValueError("MFMA GEMM output rows must be contiguous")
-        if out.requires_grad:
-            raise ValueError("MFMA GEMM output buffer must not require gradients")
-    if m_size == 0 or n_size == 0:
+    out = _checked_output(a, b, out)
+    if out.numel() == 0:
         return out
-    if isinstance(config, str):
-        config = _lib.GEMM_CONFIGS[config]
-    _C.gemm_strided(a, b, out, config=int(config or 0))
+    code = _lib.GEMM_CONFIGS[config] if isinstance(config, str) else int(config or 0)
+    _C.gemm_strided(a, b, out, config=code)
     return out
 
 
@@ -165,22 +168,8 @@ def tree_gemm(a: torch.Tensor, b: torch.Tensor, *, out: torch.Tensor | None = No
     exactly one child of the root, so K-sharded partial results combined by bf16
     adds in a balanced rank tree reproduce the unsharded result.
     """
-    _validate_operands(a, b)
-    m_size, n_size = a.size(0), b.size(1)
-    if out is None:
-        out = torch.empty((m_size, n_size), dtype=torch.bfloat16, device=a.device)
-    else:
-        if tuple(out.shape) != (m_size, n_size):
-            raise ValueError(f"MFMA GEMM output must have shape {(m_size, n_size)}, got {tuple(out.shape)}")
-        if out.dtype != torch.bfloat16:
-            raise TypeError(f"MFMA GEMM output must be BF16, got {out.dtype}")
-        if out.device != a.device:
-            raise RuntimeError("MFMA GEMM output must live on the input device")
-        if out.stride(1) != 1:
-            raise ValueError("MFMA GEMM output rows must be contiguous")
-        if out.requires_grad:
-            raise ValueError("MFMA GEMM output buffer must not require gradients")
-    if m_size == 0 or n_size == 0:
+    out = _checked_output(a, b, out)
+    if out.numel() == 0:
         return out
     return _C.gemm_tree_strided(a, b, out)
 
@@ -190,6 +179,28 @@ def _strict_gemm(a: torch.Tensor, b: torch.Tensor, *, out: torch.Tensor | None =
     if _use_tree():
         return tree_gemm(a, b, out=out)
     return mfma_gemm(a, b, out=out)
+
+
+def _fp32_gemm(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """``a @ b`` accumulated in fp32 and never rounded below it (one rounding to ``out_dtype`` when that is
+    bf16), in the arithmetic family of the selected backend.
+
+    MFMA backend, bf16 operands: the fp32 accumulator of the MFMA chain. k-tree backend, or any fp32 operand:
+    one fp32 fused multiply-add per k, k ascending, from +0 (the chain a k-tree leaf is made of, here over the
+    whole of K) - the arithmetic of the reference's native round-once twin (csrc/musa/det_gemm.mu:25-48).
+    Neither ever runs in place of the other; ``det_gemm_fp32_backend_id`` names the one in use.
+    """
+    if not _use_tree() and a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16:
+        return _C.det_gemm_fwd_out_fp32(a, b) if out_dtype == torch.float32 else _C.det_gemm_fwd(a, b)
+    return _C.det_gemm_seq(a, b, out_dtype)
+
+
+def det_gemm_fp32_backend_id(a_dtype: torch.dtype = torch.bfloat16, b_dtype: torch.dtype = torch.bfloat16) -> str:
+    """Contract id of ``DetGemmOp.forward_fp32`` / ``forward_accum_fp32`` for these operand dtypes."""
+    lib = _lib.load()
+    if not _use_tree() and a_dtype == torch.bfloat16 and b_dtype == torch.bfloat16:
+        return lib.rlk_contract_id().decode()
+    return lib.rlk_det_gemm_seq_contract_id().decode()
 
 
 def _reduction_major(tensor: torch.Tensor) -> torch.Tensor:
@@ -219,39 +230,55 @@ def mfma_linear_weight_gradient(a: torch.Tensor, grad_output: torch.Tensor) -> t
 
 
 # ---------------------------------------------------------------------------
-# Weight-transpose cache (inference only)
+# Prepared (transposed) inference weights and their refresh
 # ---------------------------------------------------------------------------
 
 
-def _tensor_version(tensor: torch.Tensor) -> int | None:
-    try:
-        return int(tensor._version)
-    except RuntimeError:  # inference tensors carry no version counter
-        return None
-
-
-def _cache_key(weight: torch.Tensor):
+def _source_key(weight: torch.Tensor):
     return (weight.data_ptr(), str(weight.device), tuple(weight.shape), weight.dtype)
+
+
+def _live_prepared(weight: torch.Tensor) -> list[torch.Tensor]:
+    """Prepared copies of ``weight`` that are still alive (dead entries are dropped on the way)."""
+    key = _source_key(weight)
+    with _PREPARED_LOCK:
+        refs = _PREPARED_TRANSPOSES.get(key, [])
+        alive = [(ref, ref()) for ref in refs]
+        kept = [ref for ref, buf in alive if buf is not None]
+        if kept:
+            _PREPARED_TRANSPOSES[key] = kept
+        else:
+            _PREPARED_TRANSPOSES.pop(key, None)
+    return [buf for _, buf in alive if buf is not None]
+
+
+def _remember_prepared(weight: torch.Tensor, prepared: torch.Tensor) -> None:
+    key = _source_key(weight)
+    with _PREPARED_LOCK:
+        refs = [ref for ref in _PREPARED_TRANSPOSES.get(key, []) if ref() is not None]
+        if not any(ref() is prepared for ref in refs):
+            refs.append(weakref.ref(prepared))
+        _PREPARED_TRANSPOSES[key] = refs
 
 
 @torch.inference_mode()
 def refresh_cached_weight_transposes(weights: Iterable[object]) -> int:
-    """Re-copy cached ``[K,N]`` transposes after an in-place weight update.
+    """Re-copy, in place, every live prepared ``[K,N]`` buffer of the given ``[N,K]`` weights after an
+    in-place weight update; returns how many weights had one.
 
     Same role as the reference function of this name
-    (rl_engine/backends/rocm/gemm/det_gemm.py:143-159): the buffers keep their
-    addresses so HIP graphs captured against them stay valid.
+    (rl_engine/backends/rocm/gemm/det_gemm.py:143-159): the buffers keep their addresses, so HIP
+    graphs captured against them stay valid. Weights that were never prepared are skipped; the
+    native-layout paths read the weight itself and have nothing to refresh.
     """
     refreshed = 0
     for weight in weights:
         if not isinstance(weight, torch.Tensor) or weight.ndim != 2:
             continue
-        cached = _WEIGHT_TRANSPOSE_CACHE.get(_cache_key(weight))
-        if cached is None:
-            continue
-        cached[1].copy_(weight.t())
-        _WEIGHT_TRANSPOSE_CACHE[_cache_key(weight)] = (_tensor_version(weight), cached[1])
-        refreshed += 1
+        buffers = _live_prepared(weight)
+        for buf in buffers:
+            buf.copy_(weight.t())
+        refreshed += 1 if buffers else 0
     return refreshed
 
 
@@ -259,42 +286,34 @@ def prepare_det_gemm_linear_weight(weight: torch.Tensor, *, out: torch.Tensor | 
     """Materialise a stable contiguous ``[K,N]`` inference weight from ``[N,K]``.
 
     Checks and error types follow the reference
-    (rl_engine/backends/rocm/gemm/det_gemm.py:345-408). The caller owns freshness.
+    (rl_engine/backends/rocm/gemm/det_gemm.py:345-408). The caller owns freshness: call this again
+    with ``out=`` or :func:`refresh_cached_weight_transposes` after the source changes.
     """
-    if weight.dim() != 2:
-        raise ValueError("prepared deterministic linear weights must be 2-D")
-    if weight.dtype != torch.bfloat16:
-        raise TypeError("prepared deterministic linear weights must be BF16")
-    if not weight.is_cuda:
-        raise RuntimeError("prepared deterministic linear weights must be on ROCm")
-    if not weight.is_contiguous():
-        raise ValueError("source deterministic linear weights must be contiguous")
-    expected_shape = (weight.size(1), weight.size(0))
-    if out is None:
-        with torch.inference_mode(False), torch.no_grad():
-            out = torch.empty(expected_shape, dtype=weight.dtype, device=weight.device)
+    what = "prepared deterministic linear weight"
+    enforce([
+        (weight.dim() == 2, ValueError, f"{what}s must be 2-D"),
+        (weight.dtype == torch.bfloat16, TypeError, f"{what}s must be BF16"),
+        (weight.is_cuda, RuntimeError, f"{what}s must be on ROCm"),
+        (weight.is_contiguous(), ValueError, "source deterministic linear weights must be contiguous"),
+    ])  # fmt: skip
+    transposed_shape = tuple(reversed(weight.shape))
+    if out is not None:
+        enforce([
+            (tuple(out.shape) == transposed_shape, ValueError, f"{what} must have shape {transposed_shape}, got {tuple(out.shape)}"),
+            (out.dtype == weight.dtype, TypeError, f"{what} dtype must match its source"),
+            (out.device == weight.device, RuntimeError, f"{what} device must match its source"),
+            (out.is_contiguous(), ValueError, f"{what} must be contiguous"),
+            (not out.requires_grad, ValueError, f"{what} must not require gradients"),
+            (lambda: not torch._C._overlaps(out, weight), ValueError, f"{what} must not alias its source"),
+        ])  # fmt: skip
     else:
-        if tuple(out.shape) != expected_shape:
-            raise ValueError(
-                f"prepared deterministic linear weight must have shape {expected_shape}, got {tuple(out.shape)}"
-            )
-        if out.dtype != weight.dtype:
-            raise TypeError("prepared deterministic linear weight dtype must match its source")
-        if out.device != weight.device:
-            raise RuntimeError("prepared deterministic linear weight device must match its source")
-        if not out.is_contiguous():
-            raise ValueError("prepared deterministic linear weight must be contiguous")
-        if out.requires_grad:
-            raise ValueError("prepared deterministic linear weight must not require gradients")
-        if torch._C._overlaps(out, weight):
-            raise ValueError("prepared deterministic linear weight must not alias its source")
+        # Post-load hooks run under inference mode; an ordinary tensor can be refreshed in place later.
+        with torch.inference_mode(False), torch.no_grad():
+            out = torch.empty(transposed_shape, dtype=weight.dtype, device=weight.device)
     with torch.no_grad():
-        out.copy_(weight.t())
-        cached = _WEIGHT_TRANSPOSE_CACHE.get(_cache_key(weight))
-        if cached is not None:
-            if cached[1] is not out:
-                cached[1].copy_(weight.t())
-            _WEIGHT_TRANSPOSE_CACHE[_cache_key(weight)] = (_tensor_version(weight), cached[1])
+        for buf in [out] + [b for b in _live_prepared(weight) if b is not out]:
+            buf.copy_(weight.t())  # earlier prepared copies of the same source stay coherent
+    _remember_prepared(weight, out)
     return out
 
 
@@ -304,12 +323,8 @@ def prepare_det_gemm_linear_weight(weight: torch.Tensor, *, out: torch.Tensor | 
 
 
 def det_gemm_linear(
-    a: torch.Tensor,
-    weight: torch.Tensor,
-    *,
-    native_op: Callable[[torch.Tensor, torch.Tensor], torch.Tensor] | None = None,
-    out: torch.Tensor | None = None,
-    inference_schedule: bool = False,
+    a: torch.Tensor, weight: torch.Tensor, *, native_op: Callable[[torch.Tensor, torch.Tensor],
+    torch.Tensor] | None = None, out: torch.Tensor | None = None, inference_schedule: bool = False,
 ) -> torch.Tensor:
     """Apply a native ``[N,K]`` weight: ``a @ weight.T``."""
     del native_op, inference_schedule
@@ -318,20 +333,19 @@ def det_gemm_linear(
 
 def det_gemm_linear_prepared(a: torch.Tensor, weight_t: torch.Tensor, *, out: torch.Tensor | None = None) -> torch.Tensor:
     """Apply a lifecycle-managed contiguous ``[K,N]`` inference weight."""
-    if torch.is_grad_enabled() and (a.requires_grad or weight_t.requires_grad):
-        raise RuntimeError("prepared deterministic linear GEMM is inference-only")
-    if not weight_t.is_contiguous():
-        raise ValueError("prepared deterministic linear weight must be contiguous")
-    if out is not None and (torch._C._overlaps(out, a) or torch._C._overlaps(out, weight_t)):
-        raise ValueError("prepared deterministic linear output must not alias its inputs")
+    tracked = torch.is_grad_enabled() and (a.requires_grad or weight_t.requires_grad)
+    enforce([
+        (not tracked, RuntimeError, "prepared deterministic linear GEMM is inference-only"),
+        (weight_t.is_contiguous(), ValueError, "prepared deterministic linear weight must be contiguous"),
+        (lambda: out is None or not (torch._C._overlaps(out, a) or torch._C._overlaps(out, weight_t)),
+         ValueError, "prepared deterministic linear output must not alias its inputs"),
+    ])  # fmt: skip
     return _strict_gemm(a, weight_t, out=out)
 
 
 def det_gemm_linear_input_gradient(
-    grad_output: torch.Tensor,
-    weight: torch.Tensor,
-    *,
-    native_op: Callable[[torch.Tensor, torch.Tensor], torch.Tensor] | None = None,
+    grad_output: torch.Tensor, weight: torch.Tensor, *, native_op: Callable[[torch.Tensor, torch.Tensor],
+    torch.Tensor] | None = None,
 ) -> torch.Tensor:
     """``dX = dY @ weight``."""
     del native_op
@@ -339,10 +353,8 @@ def det_gemm_linear_input_gradient(
 
 
 def det_gemm_linear_weight_gradient(
-    a: torch.Tensor,
-    grad_output: torch.Tensor,
-    *,
-    native_op: Callable[[torch.Tensor, torch.Tensor], torch.Tensor] | None = None,
+    a: torch.Tensor, grad_output: torch.Tensor, *, native_op: Callable[[torch.Tensor, torch.Tensor],
+    torch.Tensor] | None = None,
 ) -> torch.Tensor:
     """``dWeight = dY.T @ X`` in native ``[N,K]`` layout."""
     del native_op
@@ -415,6 +427,12 @@ class MfmaGemmFn(torch.autograd.Function):
         return da, db
 
 
+def _assert_bf16_on_gpu(*tensors: torch.Tensor) -> None:
+    # AssertionError with the reference's two messages (backends/rocm/gemm/det_gemm.py:505-506)
+    assert all(t.dtype == torch.bfloat16 for t in tensors), "BF16 only"
+    assert all(t.is_cuda for t in tensors), "Inputs must be on ROCm device"
+
+
 class RocmDetGemmOp:
     """Batch-invariant deterministic GEMM backed by the gfx950 HIP kernel."""
 
@@ -425,48 +443,46 @@ class RocmDetGemmOp:
         _report_strict_route_once()
 
     def __call__(self, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-        assert a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16, "BF16 only"
-        assert a.is_cuda and b.is_cuda, "Inputs must be on ROCm device"
+        _assert_bf16_on_gpu(a, b)
         return deterministic_gemm(a, b)
 
     def linear(self, a: torch.Tensor, weight: torch.Tensor, *, out: torch.Tensor | None = None) -> torch.Tensor:
         """Apply a native ``[N,K]`` linear weight."""
-        assert a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "BF16 only"
-        assert a.is_cuda and weight.is_cuda, "Inputs must be on ROCm device"
-        a = a.contiguous()
-        weight = weight.contiguous()
-        if out is not None:
-            if torch.is_grad_enabled() and (a.requires_grad or weight.requires_grad):
-                raise RuntimeError("direct-output deterministic GEMM is inference-only")
-            _det_gemm_linear_inference_out(a, weight, out)
-            return out
-        if not torch.is_grad_enabled() or not (a.requires_grad or weight.requires_grad):
-            return _det_gemm_linear_inference(a, weight)
-        return MfmaLinearFn.apply(a, weight)
+        _assert_bf16_on_gpu(a, weight)
+        a, weight = a.contiguous(), weight.contiguous()
+        differentiable = torch.is_grad_enabled() and (a.requires_grad or weight.requires_grad)
+        if out is None:
+            # one opaque custom op for inference (Dynamo / graph capture), autograd otherwise
+            return MfmaLinearFn.apply(a, weight) if differentiable else _det_gemm_linear_inference(a, weight)
+        if differentiable:
+            raise RuntimeError("direct-output deterministic GEMM is inference-only")
+        _det_gemm_linear_inference_out(a, weight, out)
+        return out
 
     def linear_prepared(self, a: torch.Tensor, weight_t: torch.Tensor, *, out: torch.Tensor | None = None) -> torch.Tensor:
         """Apply a post-load prepared ``[K,N]`` weight."""
-        assert a.dtype == torch.bfloat16 and weight_t.dtype == torch.bfloat16, "BF16 only"
-        assert a.is_cuda and weight_t.is_cuda, "Inputs must be on ROCm device"
+        _assert_bf16_on_gpu(a, weight_t)
         return det_gemm_linear_prepared(a.contiguous(), weight_t, out=out)
 
     def forward_fp32(self, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-        """The fp32 accumulator of ``a @ b`` stored without the bf16 rounding."""
-        assert a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16, "BF16 only"
-        assert a.is_cuda and b.is_cuda, "Inputs must be on ROCm device"
-        return _C.det_gemm_fwd_out_fp32(a, b)
+        """``a @ b`` as fp32, never rounded to bf16: the fp32 chain of the selected backend's kernel family
+        (the MFMA accumulator, or the sequential fp32 fused-multiply-add chain when the k-tree is selected)."""
+        _assert_bf16_on_gpu(a, b)
+        return _fp32_gemm(a, b)
 
     def forward_accum_fp32(self, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-        if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
-            raise TypeError("FP32-accumulation GEMM requires BF16 inputs on the gfx950 build")
+        """fp32 accumulation, result in the dtype of ``a``; bf16 or fp32 operands, as in the reference
+        (backends/rocm/gemm/det_gemm.py:548-555). An fp32 operand always takes the sequential fp32 chain."""
+        allowed = (torch.bfloat16, torch.float32)
+        if a.dtype not in allowed or b.dtype not in allowed:
+            raise TypeError("FP32-accumulation GEMM requires BF16 or FP32 inputs")
         assert a.is_cuda and b.is_cuda, "Inputs must be on ROCm device"
-        return _C.det_gemm_fwd_out_fp32(a, b).to(a.dtype)
+        return _fp32_gemm(a, b, a.dtype)
 
     def parameter_vjp_contributions_fp32(self, *, a, b, grad_output):
+        """Per-row outer products ``a_i (x) g_i`` in fp32: the summands of the weight gradient."""
         del b
-        rows_a = a.float()
-        rows_g = grad_output.float()
-        return {"b": rows_a[:, :, None] * rows_g[:, None, :]}
+        return {"b": torch.einsum("mk,mn->mkn", a.float(), grad_output.float())}
 
 
 DetGemmOp = RocmDetGemmOp
@@ -486,6 +502,7 @@ __all__ = [
     "MfmaLinearFn",
     "det_gemm_backend",
     "det_gemm_backend_id",
+    "det_gemm_fp32_backend_id",
     "tree_gemm",
     "det_gemm_fallback_reason",
     "det_gemm_linear",

@@ -527,6 +527,17 @@ def test_weight_transpose_cache_refresh(gemm):
     assert _same_bits(after, gemm.det_gemm_linear(a, w)) and not _same_bits(after, before)
     with pytest.raises(ValueError, match="must not alias"):
         gemm.prepare_det_gemm_linear_weight(w, out=w.view(32, 24))
+    # refresh_cached_weight_transposes re-copies, in place, every live prepared buffer of a weight that changed
+    second = gemm.prepare_det_gemm_linear_weight(w)
+    ptrs = (prepared.data_ptr(), second.data_ptr())
+    w.add_(0.25)
+    other = inputs.randn_bf16(123, 8, 16).to(DEV)  # never prepared: skipped
+    assert gemm.refresh_cached_weight_transposes([w, other, "not a tensor", w[0]]) == 1
+    assert (prepared.data_ptr(), second.data_ptr()) == ptrs  # addresses captured by a graph stay valid
+    assert torch.equal(prepared, w.t()) and torch.equal(second, w.t())
+    assert _same_bits(gemm.det_gemm_linear_prepared(a, second), gemm.det_gemm_linear(a, w))
+    del prepared, second  # dropped buffers are forgotten
+    assert gemm.refresh_cached_weight_transposes([w]) == 0
 
 
 @pytest.mark.parametrize("rows", (16, 48, 300))

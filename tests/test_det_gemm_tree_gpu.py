@@ -311,6 +311,82 @@ def test_tree_backend_routes_the_whole_facade(gemm, oracle, monkeypatch):
     assert gemm.det_gemm_backend() == "hip_mfma"
 
 
+@pytest.mark.parametrize("shape", [(1, 1, 1), (5, 9, 31), (64, 128, 32), (65, 129, 33), (70, 200, 1000), (130, 40, 4096), (3, 300, 97)])
+def test_sequential_fp32_gemm_equals_the_oracle_bit_for_bit(oracle, shape):
+    """rlk_det_gemm_seq: one fused multiply-add per k, ascending. Fully specified, so bit-exact against the
+    oracle: bf16 and fp32 operands in every combination, both output types, strided views."""
+    from rl_engine import _C
+
+    m, n, k = shape
+    g = torch.Generator().manual_seed(9700 + m + n + k)
+    a32 = torch.randn((m, k), generator=g)
+    b32 = torch.randn((n, k), generator=g) * 0.1  # [N, K]
+    a16, b16 = a32.to(torch.bfloat16), b32.to(torch.bfloat16)
+    for a, b in ((a16, b16), (a32, b32), (a16, b32), (a32, b16)):
+        want = oracle.det_gemm_seq_f32(a.float().numpy(), b.float().numpy())
+        got = _C.det_gemm_fwd_fp32(a.to(DEV), b.to(DEV).t())
+        assert got.dtype == torch.float32 and np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32)), (a.dtype, b.dtype)
+        # K-major right-hand side ([K, N] contiguous) and a row-strided left-hand side: same chain, same bits
+        got_kn = _C.det_gemm_fwd_fp32(a.to(DEV), b.to(DEV).t().contiguous())
+        wide = torch.zeros((m, 2 * k), dtype=a.dtype, device=DEV)
+        wide[:, ::2] = a.to(DEV)
+        got_strided = _C.det_gemm_fwd_fp32(wide[:, ::2], b.to(DEV).t())
+        assert torch.equal(got_kn.view(torch.int32), got.view(torch.int32)) and torch.equal(got_strided.view(torch.int32), got.view(torch.int32))
+    # rounded once to the dtype of A
+    want16 = oracle.f32_to_bf16(oracle.det_gemm_seq_f32(a16.float().numpy(), b16.float().numpy()))
+    got16 = _C.det_gemm_accum_fwd_fp32(a16.to(DEV), b16.to(DEV).t())
+    assert got16.dtype == torch.bfloat16 and np.array_equal(inputs.bits(got16), want16)
+    assert np.array_equal(want16, oracle.det_gemm_seq(inputs.bits(a16), inputs.bits(b16)))  # the bf16 sequential GEMM
+    # a row alone has the bits it has in the batch
+    row = m // 2
+    alone = _C.det_gemm_fwd_fp32(a32[row : row + 1].to(DEV), b32.to(DEV).t())
+    full = _C.det_gemm_fwd_fp32(a32.to(DEV), b32.to(DEV).t())
+    assert torch.equal(alone.view(torch.int32), full[row : row + 1].view(torch.int32))
+
+
+def test_sequential_fp32_gemm_order_and_fused_step_known_answers():
+    from rl_engine import _C
+
+    ones = torch.ones((1, 4), device=DEV)
+    col = torch.tensor([[2.0**24], [1.0], [1.0], [1.0]], device=DEV)
+    assert float(_C.det_gemm_fwd_fp32(ones, col)) == 2.0**24  # ascending: every +1 is rounded away
+    assert float(_C.det_gemm_fwd_fp32(ones, col.flip(0))) == 2.0**24 + 4.0
+    x = 1.0 + 2.0**-12
+    a = torch.tensor([[-(1.0 + 2.0**-11), x]], device=DEV)
+    b = torch.tensor([[1.0], [x]], device=DEV)
+    assert float(_C.det_gemm_fwd_fp32(a, b)) == 2.0**-24  # the step is fused: one rounding per term
+    assert _C.det_gemm_fwd_fp32(torch.empty((3, 0), device=DEV), torch.empty((0, 5), device=DEV)).abs().sum().item() == 0.0
+    with pytest.raises(RuntimeError, match="K mismatch"):
+        _C.det_gemm_fwd_fp32(torch.ones((2, 3), device=DEV), torch.ones((4, 2), device=DEV))
+    with pytest.raises(RuntimeError, match="bf16 or fp32"):
+        _C.det_gemm_fwd_fp32(torch.ones((2, 3), device=DEV, dtype=torch.float16), torch.ones((3, 2), device=DEV))
+
+
+def test_fp32_result_paths_never_mix_contracts(gemm, oracle, monkeypatch):
+    """DetGemmOp.forward_fp32 / forward_accum_fp32: the MFMA accumulator under the MFMA backend, the sequential
+    fp32 chain under the k-tree backend and for any fp32 operand; the reported id says which."""
+    a = inputs.randn_bf16(9710, 33, 264)
+    b = inputs.randn_bf16(9711, 264, 70, 0.05)  # [K, N]
+    seq = oracle.det_gemm_seq_f32(a.float().numpy(), b.t().contiguous().float().numpy())
+    op = gemm.DetGemmOp()
+    mfma = op.forward_fp32(a.to(DEV), b.to(DEV))
+    assert gemm.det_gemm_fp32_backend_id() == "rlkernel.det_gemm.hip_mfma16x16x32_gfx950.v1"
+    assert _same_bits(mfma.to(torch.bfloat16), gemm.mfma_gemm(a.to(DEV), b.to(DEV)))
+    assert _same_bits(op.forward_accum_fp32(a.to(DEV), b.to(DEV)), gemm.mfma_gemm(a.to(DEV), b.to(DEV)))
+    # fp32 operands: accepted, as in the reference, and always the sequential chain
+    got32 = op.forward_accum_fp32(a.float().to(DEV), b.float().to(DEV))
+    assert got32.dtype == torch.float32 and np.array_equal(got32.cpu().numpy().view(np.uint32), seq.view(np.uint32))
+    assert gemm.det_gemm_fp32_backend_id(torch.float32, torch.float32) == "rlkernel.det_gemm.hip_seqfma32_gfx950.v1"
+    with pytest.raises(TypeError, match="BF16 or FP32"):
+        op.forward_accum_fp32(a.to(DEV).half(), b.to(DEV).half())
+    monkeypatch.setattr(gemm, "_REQUESTED_BACKEND", "hip_tree")
+    assert gemm.det_gemm_fp32_backend_id() == "rlkernel.det_gemm.hip_seqfma32_gfx950.v1"
+    tree32 = op.forward_fp32(a.to(DEV), b.to(DEV))
+    assert np.array_equal(tree32.cpu().numpy().view(np.uint32), seq.view(np.uint32))
+    assert np.array_equal(inputs.bits(op.forward_accum_fp32(a.to(DEV), b.to(DEV))), oracle.f32_to_bf16(seq))
+    monkeypatch.setattr(gemm, "_REQUESTED_BACKEND", "auto")
+
+
 def test_tree_gemm_is_graph_capturable(gemm):
     a = inputs.randn_bf16(9900, 40, 1024).to(DEV)
     w = inputs.randn_bf16(9901, 200, 1024, 0.02).to(DEV)

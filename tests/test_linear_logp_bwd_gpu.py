@@ -5,7 +5,8 @@ that were themselves rounded to bf16 once, so against the exact (fp64) gradient 
 oracle every element must lie within
     half a bf16 ulp of itself  +  (2^-8 + K 2^-24 + 2e-5) * sum_k |dz_k| |operand_k|
 (the second term: dz rounding, fp32 accumulation over K terms, fp32 exp / lse).
-grad_bias is fp32 and sums the bf16 dz: within 2^-8 * sum_t |dz| + fp32 accumulation.
+grad_bias is fp32 and sums the unrounded fp32 dz (as the reference does): within
+(2e-5 + T 2^-24) * sum_t |dz|, i.e. fp32 exp / lse and fp32 accumulation only.
 Determinism, batch invariance of grad_hidden rows and configuration neutrality are
 bit-exact."""
 
@@ -97,7 +98,7 @@ def _assert_grad_parity(oracle, c, lse, grads, *, g_lse=True):
     check(inputs.bits(gw), dz.T @ hf, np.abs(dz).T @ np.abs(hf), t, "grad_weight")
     if gb is not None:
         exact = dz.sum(axis=0)
-        bound = (slack + t * 2.0**-24) * np.abs(dz).sum(axis=0) + 1e-30
+        bound = (2e-5 + t * 2.0**-24) * np.abs(dz).sum(axis=0) + 1e-30  # no bf16 rounding of dz in this sum
         worst = float((np.abs(gb.double().cpu().numpy() - exact) / bound).max())
         assert worst <= 1.0, f"grad_bias: error is {worst:.3f}x the bound"
     # the reference's own bf16-dz formulation as a second, looser witness (its ws1 bf16 tolerance)

@@ -113,6 +113,36 @@ def test_row_alone_equals_row_in_batch_with_bias_temperature_padding(logp_mod):
     assert float((picked - logp.double()).abs().max()) < 1e-4
 
 
+@pytest.mark.parametrize("shape", [(40, 3000, 256, 2990), (1100, 2500, 128, 2500), (300, 4099, 320, 4000), (1, 1024, 64, 1024), (2050, 1030, 64, 1001)])
+def test_logits_come_out_of_the_same_pass_bit_for_bit(logp_mod, shape):
+    """return_logits: the fp32 logits are the accumulators the reduction sees (bias added, padded lanes -inf,
+    no temperature), stored by the fused kernel itself: equal to the fp32-output GEMM plus bias bit for bit,
+    for the stream-group grid (up to 1024 tokens) and the split grid, aligned and unaligned vocabulary sizes,
+    every configuration; logp and lse keep their bits."""
+    from rl_engine import _C, _lib
+
+    n, v, d, real = shape
+    h, w, target = inputs.logp_inputs(n, vocab=v, hidden=d, seed=4900 + n, rms_norm=False)
+    target = target % real
+    g = torch.Generator().manual_seed(4901 + n)
+    bias = (torch.randn(v, generator=g) * 0.3).to(DEV)
+    temp = (0.5 + torch.rand(n, generator=g)).to(DEV)
+    h_d, w_d, t_d = h.to(DEV), w.to(DEV), target.to(DEV)
+    plain = _C.det_gemm_fwd_out_fp32(h_d, w_d.t())
+    for extra, want in (({}, plain), ({"bias": bias, "temperature": temp, "real_vocab_size": real}, plain + bias)):
+        want = want.clone()
+        if extra:
+            want[:, real:] = float("-inf")
+        base = logp_mod.deterministic_linear_logp(h_d, w_d, t_d, **extra)
+        for name in ("auto", "256", "128", "64", "16", "64_streams", "256_streams"):
+            lp, lse, logits = logp_mod.deterministic_linear_logp(h_d, w_d, t_d, return_logits=True, config=name, **extra)
+            assert logits.dtype == torch.float32 and logits.shape == (n, v)
+            assert _same_bits(logits, want), (name, sorted(extra))
+            assert _same_bits(lp, base[0]) and _same_bits(lse, base[1]), (name, sorted(extra))
+        staged = _lib.LOGP_CONFIGS["64"] | _lib.FORCE_STAGED
+        assert _same_bits(logp_mod.deterministic_linear_logp(h_d, w_d, t_d, return_logits=True, config=staged, **extra)[2], want)
+
+
 @pytest.mark.parametrize(
     "shape",
     [(1, 5000, 256, 4900), (17, 3072, 128, 3000), (64, 9001, 320, 9001), (33, 1024, 64, 1000), (130, 4608, 128, 4500), (700, 2300, 192, 2290)],

@@ -146,6 +146,37 @@ def test_gemm_ref_and_seq_agree_to_one_ulp_on_config1_shape(oracle):
     assert oracle.bf16_ulp_distance(ref, seq)[big].max() <= 1
 
 
+def test_sequential_fp32_gemm_is_pinned(oracle):
+    """oracle.det_gemm_seq_f32 (fp32 operands, fp32 result, one fused multiply-add per k): rounded to bf16 it is
+    the sequential bf16 GEMM on bf16-valued operands; one-hot rows select columns exactly; integer sums are
+    exact; a sum whose order matters (2^24 + 1 + 1 ...) comes out as the ascending chain gives it and not as a
+    pairwise or descending sum would; and it stays within the fp32 accumulation bound of the fp64 value on
+    general fp32 operands."""
+    rng = np.random.default_rng(21)
+    a_bits, bt_bits = oracle.randn_bf16(rng, (7, 200)), oracle.randn_bf16(rng, (5, 200), 0.02)
+    af, btf = oracle.bf16_to_f32(a_bits), oracle.bf16_to_f32(bt_bits)
+    assert np.array_equal(oracle.f32_to_bf16(oracle.det_gemm_seq_f32(af, btf)), oracle.det_gemm_seq(a_bits, bt_bits))
+    eye = np.zeros((3, 200), np.float32)
+    eye[0, 0] = eye[1, 77] = eye[2, 199] = 1.0
+    assert np.array_equal(oracle.det_gemm_seq_f32(eye, btf), btf[:, [0, 77, 199]].T)
+    # order: ((2^24 + 1) + 1) + 1 stays 2^24 in an ascending chain (each +1 is lost to rounding to even),
+    # while 1 + 1 + 1 + 2^24 (descending k) or a pairwise sum would give 2^24 + 4 / + 2
+    col = np.array([[2.0**24, 1.0, 1.0, 1.0]], np.float32)
+    ones = np.ones((1, 4), np.float32)
+    assert float(oracle.det_gemm_seq_f32(ones, col)[0, 0]) == 2.0**24
+    assert float(oracle.det_gemm_seq_f32(ones, col[:, ::-1].copy())[0, 0]) == 2.0**24 + 4.0
+    # fused step: a*b + c with a single rounding. (1 + 2^-12)^2 - (1 + 2^-11) = 2^-24 exactly; an unfused
+    # product rounds to 1 + 2^-11 first and gives 0
+    x = np.float32(1.0 + 2.0**-12)
+    got = oracle.det_gemm_seq_f32(np.array([[-(1.0 + 2.0**-11), x]], np.float32), np.array([[1.0, x]], np.float32))
+    assert float(got[0, 0]) == 2.0**-24
+    a32 = rng.standard_normal((9, 333)).astype(np.float32)
+    b32 = rng.standard_normal((4, 333)).astype(np.float32)
+    exact = a32.astype(np.float64) @ b32.astype(np.float64).T
+    bound = 333 * 2.0**-24 * (np.abs(a32).astype(np.float64) @ np.abs(b32).astype(np.float64).T)
+    assert np.all(np.abs(oracle.det_gemm_seq_f32(a32, b32) - exact) <= bound)
+
+
 # ---------------------------------------------------------------------------
 # k-tree contract
 # ---------------------------------------------------------------------------
