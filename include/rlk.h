@@ -335,6 +335,12 @@ int rlk_logits_tile_stats(const void* logits, int dtype, int64_t row_stride, con
                           int64_t V, int64_t vocab_start, int64_t real_vocab, int num_tiles, float* tile_max,
                           float* tile_sum, void* stream);
 
+/* Reduction contract identifier of rlk_logits_tile_stats / rlk_logp_from_logits (which lanes fold which
+ * columns of a tile, and in which order the partial results merge). No counterpart in the reference, whose
+ * tile-stats kernel documents no order beyond its tile boundaries
+ * (csrc/rocm/logprob/hip_deterministic_logp_kernel.hip:389-467). */
+const char* rlk_logits_logp_contract_id(void);
+
 /* Bytes of workspace rlk_logp_from_logits needs. */
 size_t rlk_logp_from_logits_workspace_bytes(int T, int num_tiles);
 

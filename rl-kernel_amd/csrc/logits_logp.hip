@@ -19,15 +19,18 @@
 //   tile t  = columns [t * V / tiles, (t + 1) * V / tiles) cut at the real vocabulary
 //   vector g = columns [8 g, 8 g + 8) of the row;
 //             columns outside the tile count as -inf
-//   lane l of the tile's wave takes vectors g0 + l, g0 + l + 64, ... ascending
+//   a tile belongs to 16 lanes; lane l of them takes vectors g0 + l, g0 + l + 16, ... ascending
 //             (g0 = first vector touching the tile) with state (m, s) = (-inf, 0):
-//             t = max of the vector;  n = max(m, t);
+//             n = max(m, the eight y);
 //             if n > -inf: s = s * e(m - n) + ((e(y0 - n) + e(y1 - n)) + ...);  m = n
-//   the 64 lane states merge in an xor butterfly (offsets 32, 16, 8, 4, 2, 1):
-//             M = max(m_a, m_b);  S = s_a * e(m_a - M) + s_b * e(m_b - M)   (-inf sides skipped)
+//   the 16 lane states merge in an xor butterfly (offsets 8, 4, 2, 1):
+//             M = max(m_a, m_b);  S = s_a * e(m_a - M) + s_b * e(m_b - M)   (-inf sides skipped,
+//             the lower lane's term first)
 //   tile_max = M, tile_sum = S (0 when M is not finite)
 //   lse = merge over tiles ascending (same formula as the fused forward's split merge)
 //   e(x) = v_exp_f32(x * log2(e)) with an unfused fp32 multiply.
+// (Four tiles share a wave, so one butterfly serves four tiles; a wave per tile spent as many
+// instructions on its 64-lane butterfly as on the tile's logits.)
 #include "linear_logp_common.h"
 #include "rlk_host.h"
 
@@ -97,66 +100,144 @@ struct TileStatsArgs {
   int num_tiles, tiles_per_group;
 };
 
-// The (m, s) state of one lane over its vectors of one tile. FAST: every vector of the row is
-// a whole, 16-byte aligned vector (decided per row, so the branch is uniform).
-template <int ELEM, bool HAS_TEMP, bool FAST>
-__device__ __forceinline__ void tile_lane_state(const typename LogitElem<ELEM>::type* row_ptr, int cols, int lo_col,
-                                                int hi_col, float inv_t, int lane, float& m, float& s) {
-  constexpr int VEC = LogitElem<ELEM>::kVec;
-  constexpr int kBatch = 4;
-  const int g0 = lo_col / VEC;
-  const int g1 = (hi_col + VEC - 1) / VEC;
-  // Four vectors of a lane are loaded before any is folded, so a wave keeps 4 KiB (8 KiB for
-  // fp32) in flight; the folds still run in ascending vector order. A lane past the last
-  // vector re-reads the last one with every column masked, which leaves (m, s) untouched.
-  for (int base = g0; base < g1; base += 64 * kBatch) {
-    float y[kBatch][VEC];
+// The eight values of vector g of a row, widened to fp32. ALIGNED: every row is made of whole,
+// 16-byte aligned vectors (decided once on the host), so a vector is one or two 16-byte loads from a
+// uniform row base plus a 32-bit lane offset; otherwise element by element, columns past the row as 0.
+template <int ELEM, bool ALIGNED>
+struct RawVector;
+
+template <bool ALIGNED>
+struct RawVector<RLK_DTYPE_BF16, ALIGNED> {
+  u32x4_t w;
+  __device__ __forceinline__ void load(const uint16_t* row, int g, int cols) {
+    if constexpr (ALIGNED) {
+      w = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const char*>(row) + (uint32_t)g * 16u);
+    } else {
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      if (base + 64 * u >= g1) break;  // uniform
-      const int g = base + 64 * u + lane;
-      const int gc = g < g1 ? g : g1 - 1;
-      load_logit_vector<ELEM>(row_ptr, gc * VEC, cols, FAST, y[u]);
-    }
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      if (base + 64 * u >= g1) break;  // uniform
-      const int g = base + 64 * u + lane;
-      const int lo = lo_col - g * VEC;
-      const int hi = g < g1 ? hi_col - g * VEC : lo;  // columns [lo, hi) of the vector count
-      if (lo > 0 || hi < VEC) {                        // only vectors that straddle a tile edge
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) y[u][i] = (i >= lo && i < hi) ? y[u][i] : kNegInf;
+      for (int i = 0; i < 4; ++i) {
+        const int c = g * 8 + 2 * i;
+        const uint32_t lo = c < cols ? row[c] : 0u, hi = c + 1 < cols ? row[c + 1] : 0u;
+        w[i] = lo | (hi << 16);
       }
-      float vmax = kNegInf;
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) {
-        const float v = HAS_TEMP ? y[u][i] * inv_t : y[u][i];  // -inf stays -inf (temperature > 0)
-        y[u][i] = v;
-        vmax = fmaxf(vmax, v);
-      }
-      const float n = fmaxf(m, vmax);
-      float sum = pinned_exp(y[u][0] - n);
-#pragma unroll
-      for (int i = 1; i < VEC; ++i) sum = sum + pinned_exp(y[u][i] - n);
-      const float scaled = s * pinned_exp(m - n);
-      s = (n > kNegInf) ? (scaled + sum) : s;
-      m = n;
     }
   }
+  __device__ __forceinline__ void unpack(float (&y)[8]) const {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      y[2 * i] = __uint_as_float(w[i] << 16);
+      y[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+};
+
+template <bool ALIGNED>
+struct RawVector<RLK_DTYPE_FP16, ALIGNED> {
+  _Float16 h[8];
+  __device__ __forceinline__ void load(const _Float16* row, int g, int cols) {
+    if constexpr (ALIGNED) {
+      const u32x4_t w = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const char*>(row) + (uint32_t)g * 16u);
+      __builtin_memcpy(h, &w, 16);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) h[i] = g * 8 + i < cols ? row[g * 8 + i] : (_Float16)0.f;
+    }
+  }
+  __device__ __forceinline__ void unpack(float (&y)[8]) const {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = (float)h[i];
+  }
+};
+
+template <bool ALIGNED>
+struct RawVector<RLK_DTYPE_FP32, ALIGNED> {
+  f32x4_t lo, hi;
+  __device__ __forceinline__ void load(const float* row, int g, int cols) {
+    if constexpr (ALIGNED) {
+      const char* p = reinterpret_cast<const char*>(row) + (uint32_t)g * 32u;
+      lo = reinterpret_cast<const f32x4_t*>(p)[0];
+      hi = reinterpret_cast<const f32x4_t*>(p)[1];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        lo[i] = g * 8 + i < cols ? row[g * 8 + i] : 0.f;
+        hi[i] = g * 8 + 4 + i < cols ? row[g * 8 + 4 + i] : 0.f;
+      }
+    }
+  }
+  __device__ __forceinline__ void unpack(float (&y)[8]) const {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      y[i] = lo[i];
+      y[4 + i] = hi[i];
+    }
+  }
+};
+
+// max(a, b, c) in one instruction. (fmaxf on values that come out of integer shifts costs an extra
+// canonicalising instruction per operand; v_max3_f32 needs none. For the non-NaN values of this contract it
+// returns what nested fmaxf returns.)
+__device__ __forceinline__ float max3_f32(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
 }
 
-template <int ELEM, bool HAS_TEMP>
+// One step of a lane's online chain: the eight scaled logits of a vector folded into (m, s).
+// (Measured without effect on the kernel's time once its instruction count was halved: a fused
+// exp2(y * log2e - n * log2e), and skipping the rescale of s while no lane's maximum moves.)
+__device__ __forceinline__ void fold_logit_vector(const float (&y)[8], float& m, float& s) {
+  const float n = max3_f32(max3_f32(max3_f32(max3_f32(y[0], y[1], y[2]), y[3], y[4]), y[5], y[6]), y[7], m);
+  float sum = pinned_exp(y[0] - n);
+#pragma unroll
+  for (int i = 1; i < 8; ++i) sum = sum + pinned_exp(y[i] - n);
+  const float scaled = s * pinned_exp(m - n);
+  s = (n > kNegInf) ? (scaled + sum) : s;
+  m = n;
+}
+
+// Value of lane (l ^ OFFSET) for OFFSET 1, 2 (DPP quad permutes) and 4, 8 (ds_swizzle xor mode).
+template <int OFFSET>
+__device__ __forceinline__ float xor_lane(float v) {
+  const int bits = __float_as_int(v);
+  int out;
+  if constexpr (OFFSET == 1) {
+    out = __builtin_amdgcn_update_dpp(bits, bits, 0xB1, 0xf, 0xf, false);  // quad_perm [1, 0, 3, 2]
+  } else if constexpr (OFFSET == 2) {
+    out = __builtin_amdgcn_update_dpp(bits, bits, 0x4E, 0xf, 0xf, false);  // quad_perm [2, 3, 0, 1]
+  } else {
+    out = __builtin_amdgcn_ds_swizzle(bits, (OFFSET << 10) | 0x1f);  // and 0x1f, or 0, xor OFFSET
+  }
+  return __int_as_float(out);
+}
+
+template <int OFFSET>
+__device__ __forceinline__ void merge_lane_states(int lane, float& m, float& s) {
+  const float om = xor_lane<OFFSET>(m);
+  const float os = xor_lane<OFFSET>(s);
+  const float n = fmaxf(m, om);
+  const float mine = (m > kNegInf) ? s * pinned_exp(m - n) : 0.f;
+  const float theirs = (om > kNegInf) ? os * pinned_exp(om - n) : 0.f;
+  // The lower lane's term goes first on both sides, so both lanes add in the same order.
+  s = (lane & OFFSET) ? (theirs + mine) : (mine + theirs);
+  m = n;
+}
+
+constexpr int kTileLanes = 16;                    // lanes that share a tile
+constexpr int kTilesPerWave = kWave / kTileLanes;  // 4
+
+template <int ELEM, bool HAS_TEMP, bool ALIGNED>
 __global__ __launch_bounds__(256) void logits_tile_stats_kernel(TileStatsArgs a) {
   using L = LogitElem<ELEM>;
   using E = typename L::type;
-  constexpr int VEC = L::kVec;
+  constexpr int VEC = 8, kBatch = 4;
+  constexpr int kStep = kTileLanes * kBatch;  // vectors of a tile per batch
   const int row = blockIdx.x;
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int l16 = lane & (kTileLanes - 1);
+  const int grp = lane / kTileLanes;
   const E* row_ptr = reinterpret_cast<const E*>(a.logits) + (int64_t)row * a.row_stride;
   const int cols = (int)a.V;
-  const bool fast = (reinterpret_cast<uintptr_t>(row_ptr) & 15) == 0 && (cols % VEC) == 0;
   const float inv_t = HAS_TEMP ? 1.0f / a.temperature[row] : 1.0f;
   const int tile_size = cols / a.num_tiles;
   const int64_t real_span = a.real_vocab - a.vocab_start;
@@ -166,37 +247,88 @@ __global__ __launch_bounds__(256) void logits_tile_stats_kernel(TileStatsArgs a)
 
   const int tile_first = blockIdx.y * a.tiles_per_group;
   const int tile_last = tile_first + a.tiles_per_group < a.num_tiles ? tile_first + a.tiles_per_group : a.num_tiles;
-  for (int tile = tile_first + wave; tile < tile_last; tile += 4) {
-    const int col_begin = tile * tile_size;
-    const int col_end = col_begin + tile_size;
-    const int real_end = col_end < real_cols ? col_end : real_cols;
+  // A wave takes four consecutive tiles at a time, one per group of 16 lanes.
+  for (int t0 = tile_first + wave * kTilesPerWave; t0 < tile_last; t0 += 4 * kTilesPerWave) {
+    const int tile = t0 + grp;
+    const bool have = tile < tile_last;
+    const int lo_col = tile * tile_size;
+    const int col_end = lo_col + tile_size;
+    int hi_col = col_end < real_cols ? col_end : real_cols;
+    if (!have || hi_col < lo_col) hi_col = lo_col;  // no columns: every vector below is masked out
+    const int g0 = lo_col / VEC;
+    const int g1 = hi_col > lo_col ? (hi_col + VEC - 1) / VEC : g0;
+    const int g_last = g1 > g0 ? g1 - 1 : (have ? g0 : 0);  // a valid vector to clamp loads to
+    // Batches in which all four vectors of every lane are whole vectors of the lane's tile (only the very
+    // first vector of a tile may start inside the vector) run without clamps and with one mask.
+    const int g_whole = (hi_col % VEC) ? g1 - 1 : g1;
+    const int my_clean = g_whole > g0 ? (g_whole - g0) / kStep : 0;
+    const int my_slots = (g1 - g0 + kTileLanes - 1) / kTileLanes;  // vector slots of 16 lanes this tile needs
+    int clean = __builtin_amdgcn_readlane(my_clean, 0), slots = __builtin_amdgcn_readlane(my_slots, 0);
+#pragma unroll
+    for (int other = kTileLanes; other < kWave; other += kTileLanes) {  // uniform over the wave's four tiles
+      const int c = __builtin_amdgcn_readlane(my_clean, other), t = __builtin_amdgcn_readlane(my_slots, other);
+      clean = c < clean ? c : clean;
+      slots = t > slots ? t : slots;
+    }
+
     float m = kNegInf, s = 0.f;
-    if (real_end > col_begin) {
-      if (fast) {
-        tile_lane_state<ELEM, HAS_TEMP, true>(row_ptr, cols, col_begin, real_end, inv_t, lane, m, s);
-      } else {
-        tile_lane_state<ELEM, HAS_TEMP, false>(row_ptr, cols, col_begin, real_end, inv_t, lane, m, s);
+    int g = g0 + l16;  // this lane's next vector
+    for (int b = 0; b < clean; ++b, g += kStep) {
+      RawVector<ELEM, ALIGNED> raw[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) raw[u].load(row_ptr, g + u * kTileLanes, cols);
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        float y[VEC];
+        raw[u].unpack(y);
+        if (u == 0 && b == 0) {  // the tile may start inside its first vector (lane 0 of the 16)
+          const int lo = lo_col - g * VEC;
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) y[i] = (i >= lo) ? y[i] : kNegInf;
+        }
+        if (HAS_TEMP) {
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) y[i] = y[i] * inv_t;  // -inf stays -inf (temperature > 0)
+        }
+        fold_logit_vector(y, m, s);
       }
     }
+    for (int b = clean; b * kBatch < slots; ++b, g += kStep) {  // the rest: clamped loads, both edges masked
+      RawVector<ELEM, ALIGNED> raw[kBatch];
 #pragma unroll
-    for (int offset = 32; offset > 0; offset >>= 1) {
-      const float om = __shfl_xor(m, offset, 64);
-      const float os = __shfl_xor(s, offset, 64);
-      const float n = fmaxf(m, om);
-      const float mine = (m > kNegInf) ? s * pinned_exp(m - n) : 0.f;
-      const float theirs = (om > kNegInf) ? os * pinned_exp(om - n) : 0.f;
-      // The lower lane's term goes first on both sides, so both lanes add in the same order.
-      s = (lane & offset) ? (theirs + mine) : (mine + theirs);
-      m = n;
+      for (int u = 0; u < kBatch; ++u) {
+        const int gu = g + u * kTileLanes;
+        raw[u].load(row_ptr, gu < g1 ? gu : g_last, cols);
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        if (b * kBatch + u >= slots) break;  // uniform: no tile of this wave reaches this slot
+        const int gu = g + u * kTileLanes;
+        float y[VEC];
+        raw[u].unpack(y);
+        const int lo = lo_col - gu * VEC;
+        const int hi = gu < g1 ? hi_col - gu * VEC : lo;  // columns [lo, hi) of the vector count
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) y[i] = (i >= lo && i < hi) ? y[i] : kNegInf;
+        if (HAS_TEMP) {
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) y[i] = y[i] * inv_t;
+        }
+        fold_logit_vector(y, m, s);  // a vector of -inf leaves (m, s) as they are
+      }
     }
-    if (lane == 0) {
+    merge_lane_states<8>(lane, m, s);
+    merge_lane_states<4>(lane, m, s);
+    merge_lane_states<2>(lane, m, s);
+    merge_lane_states<1>(lane, m, s);
+    if (l16 == 0 && have) {
       const bool finite = m > kNegInf && m < -kNegInf;
       const int64_t at = (int64_t)row * a.out_row_stride + (int64_t)tile * a.out_tile_stride;
       a.out_max[at] = m;
       a.out_sum[at] = finite ? s : 0.f;
       if (a.out_target) {
         float zt = 0.f;
-        if (target_local >= col_begin && target_local < real_end) {
+        if (target_local >= lo_col && target_local < hi_col) {
           zt = L::to_float(row_ptr[target_local]);
           if (HAS_TEMP) zt = zt * inv_t;
         }
@@ -283,11 +415,11 @@ __global__ __launch_bounds__(256) void logits_backward_kernel(LogitsBackwardArgs
 
 static int tiles_per_group_for(int T, int num_tiles) {
   // Enough workgroups to fill 256 CUs several times over when T is small; one workgroup
-  // (4 waves) per row once T alone does that. A group is a multiple of 4 tiles (one per wave).
+  // (4 waves) per row once T alone does that. A group is a multiple of 16 tiles (four per wave).
   int groups = 1;
-  while ((int64_t)T * groups < 4096 && groups * 4 < num_tiles) groups *= 2;
+  while ((int64_t)T * groups < 4096 && groups * 16 < num_tiles) groups *= 2;
   int per = (num_tiles + groups - 1) / groups;
-  per = (per + 3) / 4 * 4;
+  per = (per + 15) / 16 * 16;
   return per;
 }
 
@@ -315,11 +447,18 @@ hipError_t logits_tile_stats_launch(const void* logits, int dtype, int64_t row_s
   const int groups = (num_tiles + a.tiles_per_group - 1) / a.tiles_per_group;
   const dim3 grid((unsigned)T, (unsigned)groups);
   const bool has_temp = temperature != nullptr;
+  // every row made of whole, 16-byte aligned vectors: vector loads (the same arithmetic either way)
+  const int64_t elem_bytes = dtype == RLK_DTYPE_FP32 ? 4 : 2;
+  const bool aligned = (reinterpret_cast<uintptr_t>(logits) & 15) == 0 && (row_stride * elem_bytes) % 16 == 0 && V % 8 == 0;
 #define RLK_LAUNCH_TILE_STATS(ELEM)                                                                          \
-  if (has_temp) {                                                                                            \
-    hipLaunchKernelGGL((logits_tile_stats_kernel<ELEM, true>), grid, dim3(256), 0, stream, a);               \
+  if (aligned && has_temp) {                                                                                 \
+    hipLaunchKernelGGL((logits_tile_stats_kernel<ELEM, true, true>), grid, dim3(256), 0, stream, a);         \
+  } else if (aligned) {                                                                                      \
+    hipLaunchKernelGGL((logits_tile_stats_kernel<ELEM, false, true>), grid, dim3(256), 0, stream, a);        \
+  } else if (has_temp) {                                                                                     \
+    hipLaunchKernelGGL((logits_tile_stats_kernel<ELEM, true, false>), grid, dim3(256), 0, stream, a);        \
   } else {                                                                                                   \
-    hipLaunchKernelGGL((logits_tile_stats_kernel<ELEM, false>), grid, dim3(256), 0, stream, a);              \
+    hipLaunchKernelGGL((logits_tile_stats_kernel<ELEM, false, false>), grid, dim3(256), 0, stream, a);       \
   }
   switch (dtype) {
     case RLK_DTYPE_BF16:

@@ -417,6 +417,8 @@ int rlk_logits_tile_stats(const void* logits, int dtype, int64_t row_stride, con
   return err == hipSuccess ? RLK_OK : device_error("rlk_logits_tile_stats", err);
 }
 
+const char* rlk_logits_logp_contract_id(void) { return "rlkernel.logits_logp.hip_tiles_x16lanes_gfx950.v2"; }
+
 size_t rlk_logp_from_logits_workspace_bytes(int T, int num_tiles) {
   if (T <= 0 || num_tiles <= 0) return 0;
   return (size_t)3 * (size_t)num_tiles * (size_t)T * sizeof(float);

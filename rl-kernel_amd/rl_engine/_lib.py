@@ -69,6 +69,7 @@ EXPORTED_SYMBOLS = (
     "rlk_linear_logp_bwd_workspace_bytes",
     "rlk_linear_logp_bwd",
     "rlk_logits_tile_stats",
+    "rlk_logits_logp_contract_id",
     "rlk_logp_from_logits_workspace_bytes",
     "rlk_logp_from_logits",
     "rlk_logits_logp_backward",
@@ -156,6 +157,8 @@ def load() -> ctypes.CDLL:
 
     lib.rlk_logits_tile_stats.restype = i32
     lib.rlk_logits_tile_stats.argtypes = [vp, i32, i64, vp, i32, i64, i64, i64, i32, vp, vp, vp]
+    lib.rlk_logits_logp_contract_id.restype = c.c_char_p
+    lib.rlk_logits_logp_contract_id.argtypes = []
     lib.rlk_logp_from_logits_workspace_bytes.restype = sz
     lib.rlk_logp_from_logits_workspace_bytes.argtypes = [i32, i32]
     lib.rlk_logp_from_logits.restype = i32

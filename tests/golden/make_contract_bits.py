@@ -65,6 +65,26 @@ def contract_bits() -> dict:
     grad_h, grad_w, _ = _C.fused_linear_logp_bwd(h, w, t, lse, g, None)
     out[lib.rlk_linear_logp_contract_id().decode()]["small_linear_logp.grad_hidden"] = _sha(grad_h)
     out[lib.rlk_linear_logp_contract_id().decode()]["small_linear_logp.grad_weight"] = _sha(grad_w)
+    # bias gradient (fp32 sums of the unrounded d(logits) in the fixed token tree) on the padded case
+    bias = torch.from_numpy(d["bias"]).to(dev)
+    temp = torch.from_numpy(d["temperature"]).to(dev)
+    _, _, grad_b = _C.fused_linear_logp_bwd(h, w, t % 1900, lse2, g, None, bias, temp, 1900, need_grad_bias=True)
+    out[lib.rlk_linear_logp_contract_id().decode()]["small_linear_logp.grad_bias_bias_temp_pad"] = _sha(grad_b)
+    # log-probabilities from materialised logits (the fp32 logits of the same case, and their bf16 rounding)
+    logits = _C.det_gemm_fwd_out_fp32(h, w.t())
+    vocab = logits.size(1)
+    tiles = next(n for n in (64, 16, 8, 1) if vocab % n == 0)
+    entries = {}
+    for name, z in (("fp32", logits), ("bf16", logits.to(torch.bfloat16))):
+        lp, ls = _C.hip_deterministic_logp_from_logits(z, t, 0, vocab, tiles)
+        tmax, tsum = _C.hip_deterministic_logp_tile_stats(z, 0, vocab - 37, tiles, temperature=temp)
+        entries[f"small_linear_logp.from_{name}_logits.logp"] = _sha(lp)
+        entries[f"small_linear_logp.from_{name}_logits.lse"] = _sha(ls)
+        entries[f"small_linear_logp.from_{name}_logits.tile_max_temp_pad"] = _sha(tmax)
+        entries[f"small_linear_logp.from_{name}_logits.tile_sum_temp_pad"] = _sha(tsum)
+    out[lib.rlk_logits_logp_contract_id().decode()] = entries
+    # the sequential fp32 chain (fully specified: the CPU suite checks the stored hash against the oracle)
+    out[lib.rlk_det_gemm_seq_contract_id().decode()] = {"config1_det_gemm_fp32": _sha(_C.det_gemm_fwd_fp32(a, b))}
     # gated FFN on the same hidden states: packed gate/up projection + SwiGLU, then down
     from rl_engine.ops.ffn import qwen3_ffn_packed_inference
 

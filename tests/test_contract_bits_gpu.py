@@ -36,3 +36,15 @@ def test_stored_k_tree_bits_are_the_oracle_bits(oracle):
     a, b = inputs.config1()
     want = oracle.k_tree_gemm(inputs.bits(a), inputs.bits(b.t().contiguous()))
     assert hashlib.sha256(want.tobytes()).hexdigest() == stored["rlkernel.det_gemm.hip_ktree32_gfx950.v1"]["config1_det_gemm"]
+
+
+def test_stored_sequential_chain_bits_are_the_oracle_bits(oracle):
+    # Fully specified as well: one fp32 fused multiply-add per k, ascending.
+    import hashlib
+
+    import inputs
+
+    stored = json.loads((GOLDEN / "contract_bits.json").read_text())
+    a, b = inputs.config1()
+    want = oracle.det_gemm_seq_f32(a.float().numpy(), b.t().contiguous().float().numpy())
+    assert hashlib.sha256(want.tobytes()).hexdigest() == stored["rlkernel.det_gemm.hip_seqfma32_gfx950.v1"]["config1_det_gemm_fp32"]
