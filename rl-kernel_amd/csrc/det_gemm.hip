@@ -22,9 +22,12 @@ enum : int {
   kLoopPingPongKMajor = 3,   // weight K-major
   kLoopPingPongXKMajor = 4,  // activation K-major
   kLoopPingPongBothKMajor = 5,
-  kLoopSolo = 6  // four waves, one per SIMD
+  kLoopSolo = 6,  // four waves, one per SIMD
+  kLoopStagedKMajor = 7  // register-staged, weight K-major (the small tiles)
 };
-constexpr bool loop_weight_kmajor(int loop) { return loop == kLoopPingPongKMajor || loop == kLoopPingPongBothKMajor; }
+constexpr bool loop_weight_kmajor(int loop) {
+  return loop == kLoopPingPongKMajor || loop == kLoopPingPongBothKMajor || loop == kLoopStagedKMajor;
+}
 constexpr bool loop_act_kmajor(int loop) { return loop == kLoopPingPongXKMajor || loop == kLoopPingPongBothKMajor; }
 
 template <class S, int LOOP, bool OUT_F32, int KS = 1, int NS = 2>
@@ -50,6 +53,8 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
   f32x4_t acc[S::TN][S::TM];
   if constexpr (LOOP == kLoopSolo) {
     tile_mainloop_solo<S>(W, X, n0, m0, K, lds, acc);
+  } else if constexpr (LOOP == kLoopStagedKMajor) {
+    tile_mainloop_staged_kmajor<S, KS>(W, X, n0, m0, K, lds, acc);
   } else if constexpr (LOOP >= kLoopPingPongKMajor) {
     tile_mainloop_pingpong<S, loop_weight_kmajor(LOOP), loop_act_kmajor(LOOP), PlainRowMap<S>, KS, NS>(W, X, n0, m0, K,
                                                                                                         lds, acc);
@@ -230,6 +235,17 @@ static hipError_t launch_deep(const MatView& W, const MatView& X, void* C, int64
                  : launch_tile<S, kLoopPingPong, false, KS, NS>(W, X, C, ldc, M, N, K, stream);
 }
 
+// The register-staged K-major-weight loop of a small tile with as many K tiles per stage as 128 KiB of LDS
+// hold (four for 64 x 64, two for the 128-token tiles): a long reduction wants several K tiles in flight per
+// workgroup.
+template <class S>
+static hipError_t launch_staged_kmajor(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
+                                       bool out_f32, hipStream_t stream) {
+  constexpr int kKs = 128 * 1024 / (2 * S::kStageBytes) >= 4 ? 4 : 2;
+  return out_f32 ? launch_tile<S, kLoopStagedKMajor, true, kKs, 2>(W, X, C, ldc, M, N, K, stream)
+                 : launch_tile<S, kLoopStagedKMajor, false, kKs, 2>(W, X, C, ldc, M, N, K, stream);
+}
+
 // Tile shapes. Which one runs is a pure performance choice (see det_gemm_tile.h).
 using Shape256x256 = TileShape<256, 256, 4, 2>;
 using Shape256x256Solo = TileShape<256, 256, 2, 2>;
@@ -334,18 +350,24 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
       // N = 4096, K = 151936) the 64-token tile doubles the workgroups (2.15 -> 2.0 ms: every
       // workgroup of a feature tile still streams the whole 78 MB weight panel).
       struct Shape {
-        int config, bm;
+        int config, bn, bm;
         double quality;
       };
-      const Shape shapes[] = {{RLK_GEMM_CFG_256x256, 256, 1.00}, {RLK_GEMM_CFG_256x128, 128, 0.65},
-                              {RLK_GEMM_CFG_256x64, 64, 0.50}};
+      // The 64- and 128-feature tiles (register-staged K-major weight, native activations only) give a long
+      // reduction against few output tiles, e.g. grad_hidden of the LogP backward up to about a thousand
+      // tokens (N = 4096, K = 151936), a workgroup per CU: every workgroup then streams a narrow slice of the
+      // weight instead of a 256-column one (1.9 -> 0.9 ms at 256 tokens, 1.8 -> 1.3 ms at 512).
+      const Shape shapes[] = {{RLK_GEMM_CFG_256x256, 256, 256, 1.00}, {RLK_GEMM_CFG_256x128, 256, 128, 0.65},
+                              {RLK_GEMM_CFG_256x64, 256, 64, 0.50},   {RLK_GEMM_CFG_128x128, 128, 128, 0.52},
+                              {RLK_GEMM_CFG_128x64, 128, 64, 0.36},   {RLK_GEMM_CFG_64x64, 64, 64, 0.25}};
       double best = 1e300;
       for (const Shape& c : shapes) {
         if (c.config == RLK_GEMM_CFG_256x64 && x_kmajor) continue;
-        const int64_t tiles = tile_count(M, N, c.bm, 256);
+        if (c.bn <= 128 && (x_kmajor || !w_kmajor)) continue;
+        const int64_t tiles = tile_count(M, N, c.bm, c.bn);
         const int64_t full = tiles / 256;
         const double part = (double)(tiles - full * 256) / 256.0;
-        const double t = ((double)full + (part > 0.0 ? (part > 0.9 ? part : 0.9) : 0.0)) * (256.0 * c.bm) / c.quality;
+        const double t = ((double)full + (part > 0.0 ? (part > 0.9 ? part : 0.9) : 0.0)) * ((double)c.bn * c.bm) / c.quality;
         if (t < best * 0.999) {
           best = t;
           config = c.config;
@@ -359,6 +381,15 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
         return launch_shape<Shape256x128>(W, X, C, ldc, M, N, K, false, loop, true, out_f32, stream);
       case RLK_GEMM_CFG_256x64:
         if (!x_kmajor) return launch_shape<Shape256x64>(W, X, C, ldc, M, N, K, false, loop, true, out_f32, stream);
+        break;
+      case RLK_GEMM_CFG_64x64:
+        if (w_kmajor && x_native) return launch_staged_kmajor<Shape64x64>(W, X, C, ldc, M, N, K, out_f32, stream);
+        break;
+      case RLK_GEMM_CFG_128x64:
+        if (w_kmajor && x_native) return launch_staged_kmajor<Shape128x64>(W, X, C, ldc, M, N, K, out_f32, stream);
+        break;
+      case RLK_GEMM_CFG_128x128:
+        if (w_kmajor && x_native) return launch_staged_kmajor<Shape128x128>(W, X, C, ldc, M, N, K, out_f32, stream);
         break;
       default:
         break;  // an explicitly requested other shape runs the element-wise loader below

@@ -126,6 +126,189 @@ struct Stager {
   }
 };
 
+// Swizzle of the 16-byte chunk position inside a K row of a K-major stage (a 64-wide column of 64 K rows
+// of 128 bytes): keeps both the 16-byte stores / direct loads and the transposing fragment reads free of
+// bank conflicts.
+__device__ __forceinline__ int kmajor_swizzle(int k_row) { return 2 * (((k_row >> 1) & 1) ^ ((k_row >> 3) & 3)); }
+
+// The MFMA fragment of 16-row tile `j16` of a K-major column for K step `step`: ds_read_b64_tr_b16 hands lane r
+// of a 16-lane group the four K values of row r out of 4 K rows x 16 rows.
+__device__ __forceinline__ u32x4_t read_kmajor_fragment(const char* col, int j16, int step, int l16, int grp) {
+  typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+  typedef __attribute__((address_space(3))) bf16x4_t* lds_bf16x4_ptr_t;
+  u32x2_t half[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int k_row = step * 32 + grp * 8 + h * 4 + (l16 >> 2);
+    const int chunk = (2 * j16 + ((l16 & 3) >> 1)) ^ kmajor_swizzle(k_row);
+    const char* p = col + k_row * kRowBytes + chunk * 16 + (l16 & 1) * 8;
+    half[h] = __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr_t)p));
+  }
+  return u32x4_t{half[0].x, half[0].y, half[1].x, half[1].y};
+}
+
+// Global -> register staging of one K tile of a K-major weight operand (w[k * ld + n], features contiguous):
+// a thread's chunk is 8 consecutive features at one k, stored into the K-major stage layout above.
+// Needs N % 8 == 0, 16-byte aligned rows and K % 64 == 0 (no K tail).
+template <int ITERS, int CHUNKS, int THREADS>
+struct KMajorStager {
+  const bf16_bits* src[ITERS];  // chunk source at k0 = 0
+  int lds_off[ITERS];
+  u32x4_t regs[ITERS];
+  int64_t ld;
+
+  __device__ __forceinline__ void init(const MatView& w, int n0, int tid) {
+    ld = w.k_stride;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      int ci = tid + i * THREADS;
+      if (CHUNKS % THREADS != 0 && ci >= CHUNKS) ci = CHUNKS - 1;  // duplicate work, same value
+      const int col = ci / (kTileK * kRowChunks);
+      const int k = (ci / kRowChunks) % kTileK;
+      const int c = ci % kRowChunks;
+      int n = n0 + col * 64 + c * kChunkElems;
+      n = n + kChunkElems <= w.rows ? n : w.rows - kChunkElems;  // features past the edge are computed, never stored
+      src[i] = w.ptr + (int64_t)k * ld + n;
+      lds_off[i] = col * (kTileK * kRowBytes) + k * kRowBytes + ((c ^ kmajor_swizzle(k)) << 4);
+    }
+  }
+  __device__ __forceinline__ void load(int k0) {
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) regs[i] = *reinterpret_cast<const u32x4_t*>(src[i] + (int64_t)k0 * ld);
+  }
+  __device__ __forceinline__ void store(char* lds_stage, int tid) {
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      if (CHUNKS % THREADS == 0 || tid + i * THREADS < CHUNKS)
+        *reinterpret_cast<u32x4_t*>(lds_stage + lds_off[i]) = regs[i];
+    }
+  }
+};
+
+template <int V>
+struct IntTag {
+  static constexpr int value = V;
+};
+
+// The register-staged loop with a K-major weight operand (B[K, N], N contiguous) for the small tiles, which
+// have no direct-to-LDS K-major loop: 16-byte loads of eight features at one k, the K-major stage layout and
+// transposing fragment reads; activations as in tile_mainloop_staged. With this operand MFMA tile jn of a
+// wave holds features (wave_n * TN + jn) * 16 + (lane >> 4) * 4 + q. Same MFMA chain: same bits.
+// A stage holds KS consecutive K tiles, and the loads of two stages are in flight while a third is
+// multiplied: these tiles serve long reductions against few outputs (one workgroup per CU), where one K
+// tile in flight per workgroup would make every iteration a memory round trip. Every load is issued
+// unconditionally (past the end it repeats the last K tile and its data is dropped), so the waits the
+// compiler places count loads on one straight path.
+// The last stage may hold fewer than KS tiles. Needs BN % 64 == 0, K % 64 == 0, N % 8 == 0;
+// 2 * KS * kStageBytes of LDS.
+template <class S, int KS>
+__device__ __forceinline__ void tile_mainloop_staged_kmajor(const MatView& W, const MatView& X, int n0, int m0, int K,
+                                                            char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
+  static_assert(S::BN % 64 == 0, "whole 64-feature columns");
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_n = wave % S::WN;
+  const int wave_m = wave / S::WN;
+
+  // Addresses and LDS offsets of this thread's chunks; the data lives in the two register sets below.
+  KMajorStager<S::kWIters, S::kWChunks, S::kThreads> sw;
+  Stager<S::kXIters, S::kXChunks, S::kThreads, true> sx;
+  sw.init(W, n0, tid);
+  sx.init(X, m0, tid, [](int r) { return r; });
+  u32x4_t wr[2][KS][S::kWIters], xr[2][KS][S::kXIters];
+
+#pragma unroll
+  for (int jn = 0; jn < S::TN; ++jn)
+#pragma unroll
+    for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const int l16 = lane & 15;
+  const int grp = lane >> 4;
+  const int frag_lo = (grp ^ (l16 & 7)) << 4;
+  const int x_row_base = S::BN * kRowBytes + (wave_m * 16 * S::TM + l16) * kRowBytes;
+  constexpr int kSpan = KS * S::kStageBytes;
+  const int k_tiles = K / kTileK;
+  const int stages = (k_tiles + KS - 1) / KS;
+
+  auto load_stage = [&](auto set, int st) __attribute__((always_inline)) {
+    constexpr int R = decltype(set)::value;
+#pragma unroll
+    for (int q = 0; q < KS; ++q) {
+      int t = st * KS + q;
+      t = t < k_tiles ? t : k_tiles - 1;
+      const int k0 = t * kTileK;
+#pragma unroll
+      for (int i = 0; i < S::kWIters; ++i)
+        wr[R][q][i] = *reinterpret_cast<const u32x4_t*>(sw.src[i] + (int64_t)k0 * sw.ld);
+#pragma unroll
+      for (int i = 0; i < S::kXIters; ++i)
+        xr[R][q][i] = *reinterpret_cast<const u32x4_t*>(sx.src[i] + k0 + sx.chunk_k[i]);
+    }
+  };
+  // A tile past the end lands in a slot that is never multiplied.
+  auto store_stage = [&](auto set, char* dst) __attribute__((always_inline)) {
+    constexpr int R = decltype(set)::value;
+#pragma unroll
+    for (int q = 0; q < KS; ++q) {
+      char* tile = dst + q * S::kStageBytes;
+#pragma unroll
+      for (int i = 0; i < S::kWIters; ++i)
+        if (S::kWChunks % S::kThreads == 0 || tid + i * S::kThreads < S::kWChunks)
+          *reinterpret_cast<u32x4_t*>(tile + sw.lds_off[i]) = wr[R][q][i];
+#pragma unroll
+      for (int i = 0; i < S::kXIters; ++i)
+        if (S::kXChunks % S::kThreads == 0 || tid + i * S::kThreads < S::kXChunks)
+          *reinterpret_cast<u32x4_t*>(tile + S::BN * kRowBytes + sx.lds_off[i]) = xr[R][q][i];
+    }
+  };
+  auto multiply_stage = [&](const char* cur, int st) __attribute__((always_inline)) {
+#pragma unroll
+    for (int q = 0; q < KS; ++q) {
+      if (st * KS + q >= k_tiles) break;
+      const char* tile = cur + q * S::kStageBytes;
+#pragma unroll
+      for (int s = 0; s < kTileK / kMfmaK; ++s) {
+        u32x4_t wf[S::TN], xf[S::TM];
+#pragma unroll
+        for (int jn = 0; jn < S::TN; ++jn) {
+          const int t16 = wave_n * S::TN + jn;  // 16-feature tile of the workgroup tile
+          wf[jn] = read_kmajor_fragment(tile + (t16 >> 2) * (kTileK * kRowBytes), t16 & 3, s, l16, grp);
+        }
+#pragma unroll
+        for (int jm = 0; jm < S::TM; ++jm)
+          xf[jm] = *reinterpret_cast<const u32x4_t*>(tile + x_row_base + jm * 16 * kRowBytes + (frag_lo ^ (s << 6)));
+#pragma unroll
+        for (int jn = 0; jn < S::TN; ++jn)
+#pragma unroll
+          for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = mfma_16x16x32(wf[jn], xf[jm], acc[jn][jm]);
+      }
+    }
+  };
+
+  using Set0 = IntTag<0>;
+  using Set1 = IntTag<1>;
+  load_stage(Set0{}, 0);
+  load_stage(Set1{}, 1);
+  store_stage(Set0{}, lds);
+  __syncthreads();
+  // Entering an even stage st: LDS half 0 holds it, register set 1 holds stage st + 1 (loads in flight).
+  // The loop body has no exit in its middle: a path on which other loads are pending at the loop head
+  // would make the compiler wait for all of them there.
+  int st = 0;
+  for (; st + 1 < stages; st += 2) {
+    load_stage(Set0{}, st + 2);
+    multiply_stage(lds, st);
+    store_stage(Set1{}, lds + kSpan);
+    __syncthreads();
+    load_stage(Set1{}, st + 3);
+    multiply_stage(lds + kSpan, st + 1);
+    store_stage(Set0{}, lds);
+    __syncthreads();
+  }
+  if (st < stages) multiply_stage(lds, st);
+}
+
 // Runs the whole K loop for one (feature tile, token tile) and leaves the fp32
 // accumulators in registers. acc[jn][jm][q] is feature
 //   n0 + wave_n*16*TN + (lane>>4)*4*TN + jn*4 + q
@@ -279,7 +462,7 @@ __device__ __forceinline__ void wg_barrier() {
 // tokens contiguous: the transposed operands of a weight gradient). Its stage keeps
 // 64-token columns of 64 K rows; a wave group must own whole columns, so BM % 128 == 0,
 // and M % 8 == 0.
-__device__ __forceinline__ int kmajor_swizzle(int k_row) { return 2 * (((k_row >> 1) & 1) ^ ((k_row >> 3) & 3)); }
+// (kmajor_swizzle is defined with the register-staged K-major loop above.)
 
 // Which weight row an LDS row of the native (reduction-contiguous) weight stage holds, split
 // into a block-uniform part and a part that depends on the lane's row inside the block.
@@ -545,18 +728,8 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
   // K-major fragments: the transposing read takes, from lane r of a 16-lane group, the address
   // of 4 features (tokens) at K row (r >> 2), positions 4 (r & 3) .. +3 of MFMA tile `j16` of a
   // 64-wide column.
-  typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
-  typedef __attribute__((address_space(3))) bf16x4_t* lds_bf16x4_ptr_t;
   auto read_kmajor = [&](const char* col, int j16, int step) -> u32x4_t {
-    u32x2_t half[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int k_row = step * 32 + grp * 8 + h * 4 + (l16 >> 2);
-      const int chunk = (2 * j16 + ((l16 & 3) >> 1)) ^ kmajor_swizzle(k_row);
-      const char* p = col + k_row * kRowBytes + chunk * 16 + (l16 & 1) * 8;
-      half[h] = __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr_t)p));
-    }
-    return u32x4_t{half[0].x, half[0].y, half[1].x, half[1].y};
+    return read_kmajor_fragment(col, j16, step, l16, grp);
   };
   auto read_w_kmajor = [&](const char* st, int jn, int step) -> u32x4_t {
     return read_kmajor(st + wave_n * (64 * kRowBytes), jn, step);

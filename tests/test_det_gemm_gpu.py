@@ -347,7 +347,8 @@ def test_kmajor_weight_fast_path_gives_the_same_bits(gemm, native, shape):
     bt = inputs.randn_bf16(54, n, k, 0.02).to(DEV)  # [N,K]
     b = bt.t().contiguous()  # [K,N]
     expected = gemm.mfma_gemm(a, bt.t(), config="16x16")
-    for name in ("auto", "256x256", "256x128", "256x64", "128x128"):
+    # (128x128, 128x64 and 64x64 with a K-major weight: the register-staged K-major loop)
+    for name in ("auto", "256x256", "256x128", "256x64", "128x128", "128x64", "64x64"):
         for _ in range(2):
             assert _same_bits(gemm.mfma_gemm(a, b, config=name), expected), name
     # the activation as a K-major view (tokens contiguous: the operands of a weight gradient),
