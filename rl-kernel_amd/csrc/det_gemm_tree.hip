@@ -695,66 +695,81 @@ __global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_skinny_ke
   }
 }
 
-// The same split for more rows, on the matrix pipe: a workgroup of 16 waves takes 16 rows x 64
-// columns, wave w evaluates node w at depth 4 with one v_mfma_f32_16x16x1_4b_f32 per k (the row
-// operand of block 0 broadcast to the four 16-column blocks), operands straight from global
-// memory into registers (a lane streams the weight row of its own column and the A row
-// lane % 16), no LDS stage and no barrier until the 16 nodes are folded. 16 x the workgroups of
-// the tiled kernel: for row counts whose tiles do not fill the chip.
-constexpr int kTreeNodeLevels = 6;  // tree levels below a wave's node (K <= 32768)
+// The same split for more rows, on the matrix pipe: a workgroup of 16 waves takes 16 rows, wave w evaluates
+// node w at depth 4 with one v_mfma_f32_16x16x1_4b_f32 per k, operands straight from global memory into
+// registers (a lane streams the weight row of its own column and the A row lane % 16), no LDS stage and no
+// barrier until the 16 nodes are folded. 16 x the workgroups of the tiled kernel: for row counts whose tiles
+// do not fill the chip. The four 16 x 16 blocks of the instruction are
+//   KB = 1: four groups of 16 columns (64 columns per workgroup), the row operand of block 0 broadcast;
+//   KB = 4: the four grandchildren (depth 6) of the wave's node for one group of 16 columns, every block
+//           with its own k range; the lane then folds its four blocks in tree order. Four times the
+//           workgroups and a quarter of the leaves per lane: for narrow N, where 64-column workgroups
+//           would leave most CUs idle and a lane's chain of leaves (one memory round trip each) decides.
+// CHUNKS = leaf length / 8. The leaves of a node are fetched two leaves ahead (one where the registers of a
+// third leaf would spill: 64 columns with leaves of 32); every fetch is
+// issued unconditionally (past the node's end it repeats the last leaf), so that the waits the compiler
+// places count loads along one straight path.
+constexpr int kTreeNodeLevels = 6;  // tree levels below a node, KB = 1 (K <= 32768)
 
+template <int KB, int CHUNKS>
 __global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_nodes_kernel(
     MatView A, MatView B, bf16_bits* __restrict__ C, int64_t ldc, int M, int N, int K, int depth) {
-  __shared__ uint32_t nodes[kTreeSkinnyWaves][8][64];
+  constexpr int kLevels = KB == 4 ? kTreeNodeLevels - 2 : kTreeNodeLevels;
+  constexpr int kKeep = KB == 4 ? 2 : 8;  // packed registers a wave hands to the fold
+  constexpr int kTreeNodeAhead = (KB == 1 && CHUNKS == 4) ? 1 : 2;
+  __shared__ uint32_t nodes[kTreeSkinnyWaves][kKeep][64];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int n0 = blockIdx.x * 64, m0 = blockIdx.y * 16;
-  const int col = n0 + lane;
+  const int n0 = blockIdx.x * (KB == 4 ? 16 : 64), m0 = blockIdx.y * 16;
+  const int col = n0 + (KB == 4 ? (lane & 15) : lane);
   const int a_index = m0 + (lane & 15);
   const bf16_bits* wrow = B.ptr + (int64_t)(col < N ? col : N - 1) * B.row_stride;
   const bf16_bits* arow = A.ptr + (int64_t)(a_index < M ? a_index : M - 1) * A.row_stride;
-  const int len = K >> depth;                          // leaf length, 8 ... 32, a multiple of 8
-  const int leaves = 1 << (depth - kTreeSkinnySplit);  // leaves under this wave's node
-  const int first = wave * leaves * len;
+  constexpr int len = 8 * CHUNKS;  // leaf length
+  const int node_depth = kTreeSkinnySplit + (KB == 4 ? 2 : 0);
+  const int leaves = 1 << (depth - node_depth);  // leaves under this lane's node
+  const int first = (KB == 4 ? 4 * wave + (lane >> 4) : wave) * leaves * len;
 
-  uint32_t slot[kTreeNodeLevels][8];
+  uint32_t slot[kLevels][8];
   uint32_t cur[8];
-  u32x4_t w_now[4], w_next[4], a_now[4], a_next[4];
-  auto fetch = [&](int lo, u32x4_t (&w)[4], u32x4_t (&a)[4]) {
+  u32x4_t wq[kTreeNodeAhead + 1][CHUNKS], aq[kTreeNodeAhead + 1][CHUNKS];
+  auto fetch = [&](int leaf, u32x4_t (&w)[CHUNKS], u32x4_t (&a)[CHUNKS]) __attribute__((always_inline)) {
+    const int lo = first + (leaf < leaves ? leaf : leaves - 1) * len;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      if (8 * c < len) {
-        w[c] = *reinterpret_cast<const u32x4_t*>(wrow + lo + 8 * c);
-        a[c] = *reinterpret_cast<const u32x4_t*>(arow + lo + 8 * c);
-      }
+    for (int c = 0; c < CHUNKS; ++c) {
+      w[c] = *reinterpret_cast<const u32x4_t*>(wrow + lo + 8 * c);
+      a[c] = *reinterpret_cast<const u32x4_t*>(arow + lo + 8 * c);
     }
   };
-  fetch(first, w_now, a_now);
+#pragma unroll
+  for (int p = 0; p < kTreeNodeAhead; ++p) fetch(p, wq[p], aq[p]);
   for (int i = 0; i < leaves; ++i) {
-    const int lo = first + i * len;
-    if (i + 1 < leaves) fetch(lo + len, w_next, a_next);
+    fetch(i + kTreeNodeAhead, wq[kTreeNodeAhead], aq[kTreeNodeAhead]);
     f32x16_t acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.f;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      if (8 * c < len) {
+    for (int c = 0; c < CHUNKS; ++c) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const uint32_t wb = w_now[c][e >> 1], ab = a_now[c][e >> 1];
-          const float b = __uint_as_float((e & 1) ? (wb & 0xffff0000u) : (wb << 16));
-          const float a = __uint_as_float((e & 1) ? (ab & 0xffff0000u) : (ab << 16));
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t wb = wq[0][c][e >> 1], ab = aq[0][c][e >> 1];
+        const float b = __uint_as_float((e & 1) ? (wb & 0xffff0000u) : (wb << 16));
+        const float a = __uint_as_float((e & 1) ? (ab & 0xffff0000u) : (ab << 16));
+        if constexpr (KB == 4) {
+          acc = __builtin_amdgcn_mfma_f32_16x16x1f32(a, b, acc, 0, 0, 0);
+        } else {
           acc = __builtin_amdgcn_mfma_f32_16x16x1f32(a, b, acc, 2, 0, 0);
         }
       }
     }
 #pragma unroll
     for (int q = 0; q < 8; ++q) cur[q] = pack_bf16x2(acc[2 * q], acc[2 * q + 1]);
+    // Leaf i closes one node per trailing one bit of i; then it waits at the level of its lowest zero bit.
     int level = 0;
     for (int j = i; j & 1; j >>= 1, ++level) {
 #pragma unroll
-      for (int l = 0; l < kTreeNodeLevels; ++l) {
+      for (int l = 0; l < kLevels; ++l) {
         if (l == level) {
 #pragma unroll
           for (int r = 0; r < 8; ++r) cur[r] = bf16x2_add(slot[l][r], cur[r]);
@@ -763,29 +778,39 @@ __global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_nodes_ker
     }
     if (i + 1 < leaves) {
 #pragma unroll
-      for (int l = 0; l < kTreeNodeLevels; ++l) {
+      for (int l = 0; l < kLevels; ++l) {
         if (l == level) {
 #pragma unroll
           for (int r = 0; r < 8; ++r) slot[l][r] = cur[r];
         }
       }
+    }
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        w_now[c] = w_next[c];
-        a_now[c] = a_next[c];
+    for (int p = 0; p < kTreeNodeAhead; ++p) {
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c) {
+        wq[p][c] = wq[p + 1][c];
+        aq[p][c] = aq[p + 1][c];
       }
     }
   }
+  // Accumulator r: block r / 4; row 4 (lane / 16) + r % 4, column lane % 16 of the block.
+  // cur[q] packs accumulators 2 q, 2 q + 1 (two consecutive rows of one column), block q / 2.
+  if constexpr (KB == 4) {
+    // blocks 0..3 are the node's grandchildren left to right: (0 + 1) + (2 + 3)
 #pragma unroll
-  for (int r = 0; r < 8; ++r) nodes[wave][r][lane] = cur[r];
+    for (int h = 0; h < 2; ++h)
+      nodes[wave][h][lane] = bf16x2_add(bf16x2_add(cur[h], cur[2 + h]), bf16x2_add(cur[4 + h], cur[6 + h]));
+  } else {
+#pragma unroll
+    for (int r = 0; r < 8; ++r) nodes[wave][r][lane] = cur[r];
+  }
   __syncthreads();
   if (wave != 0) return;
-  // Accumulator r: block r / 4 (16 columns each); row 4 (lane / 16) + r % 4, column lane % 16.
-  // cur[q] packs accumulators 2 q, 2 q + 1 (two consecutive rows of one column).
   const int out_col = n0 + (lane & 15);
   const int out_row = m0 + 4 * (lane >> 4);
 #pragma unroll
-  for (int q = 0; q < 8; ++q) {
+  for (int q = 0; q < kKeep; ++q) {
     uint32_t v[kTreeSkinnyWaves];
 #pragma unroll
     for (int w = 0; w < kTreeSkinnyWaves; ++w) v[w] = nodes[w][q][lane];
@@ -793,12 +818,26 @@ __global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_nodes_ker
     for (int width = kTreeSkinnyWaves / 2; width >= 1; width /= 2)
 #pragma unroll
       for (int w = 0; w < width; ++w) v[w] = bf16x2_add(v[2 * w], v[2 * w + 1]);
-    const int c = out_col + 16 * (q >> 1);
+    const int c = out_col + (KB == 4 ? 0 : 16 * (q >> 1));
     const int r = out_row + 2 * (q & 1);
     if (c < N) {
       if (r < M) C[(int64_t)r * ldc + c] = (bf16_bits)(v[0] & 0xffffu);
       if (r + 1 < M) C[(int64_t)(r + 1) * ldc + c] = (bf16_bits)(v[0] >> 16);
     }
+  }
+}
+
+template <int KB>
+static void launch_nodes(const MatView& A, const MatView& B, bf16_bits* out, int64_t ldc, int M, int N, int K, int depth,
+                         hipStream_t stream) {
+  constexpr int kCols = KB == 4 ? 16 : 64;
+  const dim3 grid((unsigned)((N + kCols - 1) / kCols), (unsigned)((M + 15) / 16)), block(64 * kTreeSkinnyWaves);
+  auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, block, 0, stream, A, B, out, ldc, M, N, K, depth); };
+  switch ((K >> depth) / 8) {  // leaf length 8 ... 32
+    case 1: launch(det_gemm_tree_nodes_kernel<KB, 1>); break;
+    case 2: launch(det_gemm_tree_nodes_kernel<KB, 2>); break;
+    case 3: launch(det_gemm_tree_nodes_kernel<KB, 3>); break;
+    default: launch(det_gemm_tree_nodes_kernel<KB, 4>); break;
   }
 }
 
@@ -861,20 +900,28 @@ hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int
   const bool nodes_ok = a_chunked && b_chunked && depth >= kTreeSkinnySplit &&
                         depth - kTreeSkinnySplit <= kTreeNodeLevels && (M + 15) / 16 <= 65535;
   if (config == RLK_TREE_CFG_NODES && !nodes_ok) return hipErrorInvalidValue;
+  // The node-per-wave kernel splits a node over the four blocks of its instruction where 64-column workgroups
+  // would not give every CU one; that needs two more tree levels above the leaves.
+  const int64_t wide_groups = (int64_t)((N + 63) / 64) * ((M + 15) / 16);
+  const bool split_blocks = nodes_ok && wide_groups < 256 && depth >= kTreeSkinnySplit + 2;
   if (config == RLK_TREE_CFG_AUTO && nodes_ok && M > 8) {
     // Node-per-wave kernel against the tiled one (fitted to the Qwen3-8B projections at 8 ... 4096 rows):
-    // the first runs at about 40 TFLOP/s on rows padded to 16 whatever the grid; the second needs about
+    // the first runs at about 50 TFLOP/s on rows padded to 16 whatever the grid; the second needs about
     // 2.25 us per leaf per round of 512 tiles and reaches about 80 TFLOP/s once the chip is full.
     const double work = 2.0 * N * (double)K;
-    const double t_nodes = work * (16.0 * ((M + 15) / 16)) / 40e12;
+    const double t_nodes = work * (16.0 * ((M + 15) / 16)) / 50e12;
     const double rounds = (double)((tiles64 + 511) / 512);
     const double t_tiled_latency = rounds * (double)(1 << depth) * 2.25e-6;
     const double t_tiled_rate = work * M / 80e12;
     if (t_nodes < (t_tiled_latency > t_tiled_rate ? t_tiled_latency : t_tiled_rate)) config = RLK_TREE_CFG_NODES;
   }
+  // Up to 8 rows and narrow N (from HBM, Qwen3-8B down at one token 76 -> 39 us, o_proj 24 -> 15 us; the wide
+  // projections measure the same on either kernel): the split blocks shorten a lane's chain of leaves to a
+  // quarter, which the vector-ALU kernel's wave halves only halve.
+  if (config == RLK_TREE_CFG_AUTO && M <= 8 && split_blocks && N <= kTreeHalvesMaxN) config = RLK_TREE_CFG_NODES;
   if (config == RLK_TREE_CFG_NODES) {
-    hipLaunchKernelGGL(det_gemm_tree_nodes_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((M + 15) / 16)),
-                       dim3(64 * kTreeSkinnyWaves), 0, stream, A, B, out, ldc, M, N, K, depth);
+    if (split_blocks) launch_nodes<4>(A, B, out, ldc, M, N, K, depth, stream);
+    else launch_nodes<1>(A, B, out, ldc, M, N, K, depth, stream);
     return hipGetLastError();
   }
   if (skinny_ok && (config == RLK_TREE_CFG_SKINNY || (config == RLK_TREE_CFG_AUTO && (M <= 8 || !nodes_ok)))) {

@@ -210,8 +210,9 @@ def test_skinny_kernel_folds_the_depth_4_nodes_to_the_same_bits(oracle):
 
 
 def test_node_per_wave_kernel_computes_the_same_bits(oracle):
-    # 16 rows x 64 columns per workgroup, one depth-4 node per wave on the fp32 matrix pipe: any row
-    # count, ragged M and N, against the vector-ALU kernel; one case against the oracle.
+    # 16 rows per workgroup, one depth-4 node per wave on the fp32 matrix pipe: any row count, ragged M and N,
+    # against the vector-ALU kernel; one case against the oracle. Narrow problems split a node over the four
+    # blocks of the instruction (16 columns per workgroup), problems of 256 and more 64-column groups do not.
     from rl_engine import _C
 
     def run(a_d, b_kn, config):
@@ -223,6 +224,10 @@ def test_node_per_wave_kernel_computes_the_same_bits(oracle):
             a = inputs.randn_bf16(9900 + k + m, m, k).to(DEV)
             w = inputs.randn_bf16(9901 + k + m, n, k, 0.02).to(DEV)
             assert _same_bits(run(a, w.t(), 4), run(a, w.t(), 1)), (m, k, n)
+    for m, n, k in ((40, 5500, 4096), (16, 16400, 2048), (33, 5504, 6144)):  # 258, 257 and 258 groups of 64 columns
+        a = inputs.randn_bf16(9920 + m, m, k).to(DEV)
+        w = inputs.randn_bf16(9921 + m, n, k, 0.02).to(DEV)
+        assert _same_bits(run(a, w.t(), 4), run(a, w.t(), 1)), (m, k, n)
     a = inputs.randn_bf16(9910, 37, 4096)
     w = inputs.randn_bf16(9911, 70, 4096, 0.02)
     assert np.array_equal(inputs.bits(run(a.to(DEV), w.to(DEV).t(), 4)), _oracle_tree(oracle, a, w))
