@@ -482,6 +482,17 @@ def main() -> int:
                      "frac_of_fp32_mfma_peak": round(flops_d / ms_tree_down * 1e-9 / 157.3, 4)},
             "contract": _lib.load().rlk_det_gemm_tree_contract_id().decode(),
         }
+        # the sequential fp32 chain (fp32-result GEMM of the default backend): vector ALU, one fma per k
+        from rl_engine import _C as _c_seq
+
+        ms_seq = _time_calls(lambda: _c_seq.det_gemm_fwd_fp32(x[:1024], w_gu.t()), 3, 1)
+        result["det_gemm_seq"] = {
+            "workload": "X[1024,4096]xW[24576,4096]^T, fp32 result, one fp32 fused multiply-add per k in ascending order",
+            "ms": round(ms_seq, 3), "tflops": round(2.0 * 1024 * 2 * INTER * HIDDEN / ms_seq * 1e-9, 1),
+            "bound": "fp32 vector ALU (157.3 TFLOP/s)",
+            "frac_of_fp32_valu_peak": round(2.0 * 1024 * 2 * INTER * HIDDEN / ms_seq * 1e-9 / 157.3, 4),
+            "contract": _lib.load().rlk_det_gemm_seq_contract_id().decode(),
+        }
         decode = []
         for ts in (1, 16, 64):
             for name, act, w, out in (("gate_up", x, w_gu, out_gu), ("down", h, w_d, out_d)):
@@ -521,6 +532,26 @@ def main() -> int:
             "frac_of_mfma_peak": round(3 * fl_lp / ms_bwd * 1e-9 / PEAK_BF16_TFLOPS, 4),
         }
         del lse_lp, g_lp
+        # the same pass with the fp32 logits stored (return_logits=True) against the plain forward, at 2048 tokens
+        hid_s, tgt_s = hid[:2048].contiguous(), tgt[:2048].contiguous()
+        ms_plain = _time_calls(lambda: deterministic_linear_logp(hid_s, w_lm, tgt_s), 10, 4)
+        ms_logits = _time_calls(lambda: deterministic_linear_logp(hid_s, w_lm, tgt_s, return_logits=True), 10, 4)
+        result["linear_logp"]["return_logits"] = {
+            "workload": "T=2048: LogP forward, and the same launch storing logits[2048,151936] as fp32 (1.24 GB written)",
+            "ms_plain": round(ms_plain, 3), "ms_with_logits": round(ms_logits, 3), "ratio": round(ms_logits / ms_plain, 3),
+        }
+        # the backward below the token count where its GEMMs fill the chip: 256 tokens
+        hid_b, tgt_b = hid[:256].contiguous(), tgt[:256].contiguous()
+        _, lse_b = _C.fused_linear_logp(hid_b, w_lm, tgt_b)
+        g_b = torch.randn((256,), generator=gen, device=dev)
+        ms_bs = _time_calls(lambda: _C.fused_linear_logp_bwd(hid_b, w_lm, tgt_b, lse_b, g_b, None), 10, 4)
+        result["linear_logp"]["backward_256_tokens"] = {
+            "workload": "T=256: d(logits) recompute -> grad_hidden[256,4096] (reduction over 151936) and grad_weight[151936,4096]",
+            "ms": round(ms_bs, 3),
+            "min_hbm_bytes": 3 * 2.0 * VOCAB * HIDDEN,  # the weight read twice, its gradient written once
+            "frac_of_hbm_peak": round(3 * 2.0 * VOCAB * HIDDEN / ms_bs * 1e-6 / PEAK_HBM_GBPS, 4),
+        }
+        del hid_s, tgt_s, hid_b, tgt_b, lse_b, g_b
         # the stage that reuses materialised logits: one pass over [8192, 151936] bf16
         logits = randn(tl, VOCAB, 4.0)
         ms_fl = _time_calls(lambda: _C.hip_deterministic_logp_from_logits(logits, tgt, 0, VOCAB, 64), 10, 4)
