@@ -77,7 +77,7 @@ def _parse():
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-T table")
     ap.add_argument("--rotate-weights", action="store_true",
                     help="gate_up_tN / down_tN legs: launch over copies of the weight (~1.3 GB in rotation) so that it is read from HBM")
-    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|gate_up_tN|down_tN|logp|logp_decode|logp_mid|logp_bwd|from_logits|ffn|tree|tree_down|tree_decode|copy|power (used for profiling)")
+    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|gate_up_tN|down_tN|logp|logp_decode|logp_mid|logp_logits|logp_bwd|logp_bwd_256|from_logits|ffn|tree|tree_down|tree_decode|copy|power (used for profiling)")
     return ap.parse_args()
 
 
@@ -282,14 +282,16 @@ def main() -> int:
         print(json.dumps({"leg": args.only, "ms": ms, "tflops": flops / ms * 1e-9,
                           "launches": args.steps + args.warmup}))
         return 0
-    if args.only in ("logp_bwd", "from_logits"):
+    if args.only in ("logp_bwd", "logp_bwd_256", "logp_logits", "from_logits"):
         from rl_engine import _C
 
-        tl = 8192
+        tl = {"logp_bwd_256": 256, "logp_logits": 2048}.get(args.only, 8192)
         hid = randn(tl, HIDDEN)
         w_lm = randn(VOCAB, HIDDEN, 0.02)
         tgt = torch.randint(0, VOCAB, (tl,), generator=gen, device=dev)
-        if args.only == "logp_bwd":
+        if args.only == "logp_logits":  # the forward that also stores the fp32 logits
+            ms = _time_calls(lambda: deterministic_linear_logp(hid, w_lm, tgt, return_logits=True), args.steps, args.warmup)
+        elif args.only.startswith("logp_bwd"):
             _, lse = _C.fused_linear_logp(hid, w_lm, tgt)
             g = torch.randn((tl,), generator=gen, device=dev)
             ms = _time_calls(lambda: _C.fused_linear_logp_bwd(hid, w_lm, tgt, lse, g, None), args.steps, args.warmup)
