@@ -28,22 +28,15 @@ import torch
 from rl_engine import _C, _lib
 from rl_engine._checks import enforce, output_buffer_rules
 
-_BACKEND_ENV = "RL_KERNEL_DET_GEMM_BACKEND"
-_AUTO_BACKEND = "auto"
 _HIP_BACKEND = "hip_mfma"
 _TREE_BACKEND = "hip_tree"
-# Names the reference accepts (rl_engine/backends/rocm/gemm/det_gemm.py:33-48) select the
-# contract that plays the same role here; "auto" is the MFMA contract on gfx950.
-_BACKEND_ALIASES = {
+# RL_KERNEL_DET_GEMM_BACKEND: every value the reference accepts (rl_engine/backends/rocm/gemm/det_gemm.py:33-48)
+# selects the contract that plays the same role here; "auto" is the MFMA contract on gfx950.
+_CONTRACT_OF_REQUEST = {
+    "auto": _HIP_BACKEND, _HIP_BACKEND: _HIP_BACKEND, "mfma": _HIP_BACKEND, "triton_mfma": _HIP_BACKEND,
+    _TREE_BACKEND: _TREE_BACKEND, "tree": _TREE_BACKEND, "triton_tree": _TREE_BACKEND, "triton": _TREE_BACKEND,
     "rocm": _TREE_BACKEND,
-    "triton": _TREE_BACKEND,
-    "tree": _TREE_BACKEND,
-    "triton_tree": _TREE_BACKEND,
-    "mfma": _HIP_BACKEND,
-    "triton_mfma": _HIP_BACKEND,
-}
-_ROUTE_REPORTED = False
-_ROUTE_REPORT_LOCK = Lock()
+}  # fmt: skip
 # Prepared [K,N] copies by source weight: what refresh_cached_weight_transposes re-copies. The kernels read
 # the native [N,K] layout directly, so no transpose is ever made behind the caller's back; the only
 # transposed buffers alive are the ones prepare_det_gemm_linear_weight handed out. They are held weakly:
@@ -53,26 +46,26 @@ _PREPARED_LOCK = Lock()
 
 
 def _resolve_backend_request(value: str) -> str:
-    value = value.strip().lower()
-    value = _BACKEND_ALIASES.get(value, value)
-    if value not in {_AUTO_BACKEND, _HIP_BACKEND, _TREE_BACKEND}:
+    """The request as written (normalised), refused when it names no contract of this build."""
+    key = value.strip().lower()
+    if key not in _CONTRACT_OF_REQUEST:
         raise RuntimeError(
-            f"{_BACKEND_ENV} must be '{_AUTO_BACKEND}', '{_TREE_BACKEND}' or '{_HIP_BACKEND}' "
-            f"on the gfx950 build, got {value!r}"
+            f"RL_KERNEL_DET_GEMM_BACKEND must be 'auto', '{_TREE_BACKEND}' or '{_HIP_BACKEND}' "
+            f"on the gfx950 build, got {key!r}"
         )
-    return value
+    return "auto" if key == "auto" else _CONTRACT_OF_REQUEST[key]
 
 
 def _requested_backend() -> str:
-    return _resolve_backend_request(os.getenv(_BACKEND_ENV, _AUTO_BACKEND))
+    return _resolve_backend_request(os.getenv("RL_KERNEL_DET_GEMM_BACKEND", "auto"))
 
 
-_REQUESTED_BACKEND = _requested_backend()
+_REQUESTED_BACKEND = _requested_backend()  # read once, at import, as in the reference
 
 
 def det_gemm_backend() -> str:
     """Name of the strict GEMM implementation in use."""
-    return _TREE_BACKEND if _REQUESTED_BACKEND == _TREE_BACKEND else _HIP_BACKEND
+    return _CONTRACT_OF_REQUEST[_REQUESTED_BACKEND]
 
 
 def _use_tree() -> bool:
@@ -89,19 +82,18 @@ def det_gemm_backend_id() -> str:
     return (lib.rlk_det_gemm_tree_contract_id() if _use_tree() else lib.rlk_contract_id()).decode()
 
 
+_route_line_pending = [True]  # one route line per process (RL_KERNEL_ROUTE_REPORT), whoever constructs first
+
+
 def _report_strict_route_once() -> None:
-    global _ROUTE_REPORTED
     if os.getenv("RL_KERNEL_ROUTE_REPORT", "").strip().lower() not in {"1", "true", "yes", "on"}:
         return
-    with _ROUTE_REPORT_LOCK:
-        if _ROUTE_REPORTED:
-            return
-        _ROUTE_REPORTED = True
-    print(
-        f"[RL-Kernel][route] mode={os.getenv('RL_KERNEL_MODE', 'strict')} module=gemm "
-        f"requested={_REQUESTED_BACKEND} actual={det_gemm_backend_id()} fallback=false",
-        flush=True,
-    )
+    with _PREPARED_LOCK:
+        first, _route_line_pending[0] = _route_line_pending[0], False
+    if first:
+        mode = os.getenv("RL_KERNEL_MODE", "strict")
+        print(f"[RL-Kernel][route] mode={mode} module=gemm requested={_REQUESTED_BACKEND} "
+              f"actual={det_gemm_backend_id()} fallback=false", flush=True)  # fmt: skip
 
 
 # ---------------------------------------------------------------------------
