@@ -100,6 +100,10 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_partial_kernel(LogpAr
     }
 
     const int col0 = v0 + stream * 16;  // first column of this lane's run
+    const int span0 = v0 + wave_n * 64;  // first column of the wave's four runs
+    // whole spans into 16-byte aligned rows are stored by the four lanes of a token together (wave uniform)
+    const bool span_stores = a.logits != nullptr && span0 + 64 <= a.V && (a.logits_ld & 3) == 0 &&
+                             (reinterpret_cast<uintptr_t>(a.logits) & 15) == 0;
     float bias_run[16];
 #pragma unroll
     for (int c = 0; c < 16; ++c) bias_run[c] = 0.f;
@@ -114,7 +118,9 @@ __global__ __launch_bounds__(S::kThreads) void linear_logp_partial_kernel(LogpAr
       for (int c = 0; c < 16; ++c) y[c] = biased_logit(acc[c >> 2][jm][c & 3], a.bias != nullptr, bias_run[c], col0 + c, a.vocab_limit);
       if (a.logits) {  // the same accumulators the reduction sees, stored before the temperature
         const int m = m0 + tok_local + jm * 16;
-        if (m < a.T) store_logit_run(a.logits + (int64_t)m * a.logits_ld, col0, a.V, y);
+        float* row = a.logits + (int64_t)(m < a.T ? m : 0) * a.logits_ld;
+        if (span_stores) store_logit_span(row, span0, grp, m < a.T, y);
+        else if (m < a.T) store_logit_run(row, col0, a.V, y);
       }
       if (a.temperature) {
 #pragma unroll

@@ -55,6 +55,44 @@ __device__ __forceinline__ void store_logit_run(float* __restrict__ row, int col
   }
 }
 
+// The same store for the four lanes of one token together (lanes l, l + 16, l + 32, l + 48 of a wave hold the four
+// adjacent 16-column runs of the token's 64-column span that starts at span0): the 4 x 4 grid of 16-byte chunks is
+// transposed between the lanes (two butterfly stages of lane swaps over distances 32 and 16: the chunk that lane
+// g held at position c ends at lane c, position g), so that store q of lane g writes bytes [64 q + 16 g, + 16) of
+// the span and one instruction covers whole 64-byte sectors instead of a quarter of each. Every lane of the wave
+// must call it (the swaps read the other lanes whatever their `live`); needs span0 + 64 <= V and 16-byte aligned
+// rows, both uniform over the wave. The values stored are the ones store_logit_run stores.
+__device__ __forceinline__ void store_logit_span(float* __restrict__ row, int span0, int grp, bool live,
+                                                 const float (&u)[16]) {
+  uint32_t w[4][4];  // [chunk][word]
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[c][e] = __float_as_uint(u[4 * c + e]);
+#pragma unroll
+  for (int c = 0; c < 2; ++c)  // lane bit 5 <-> chunk bit 1
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const auto r = __builtin_amdgcn_permlane32_swap(w[c][e], w[c + 2][e], false, false);
+      w[c][e] = r[0];
+      w[c + 2][e] = r[1];
+    }
+#pragma unroll
+  for (int c = 0; c < 4; c += 2)  // lane bit 4 <-> chunk bit 0
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const auto r = __builtin_amdgcn_permlane16_swap(w[c][e], w[c + 1][e], false, false);
+      w[c][e] = r[0];
+      w[c + 1][e] = r[1];
+    }
+  if (live) {
+    float* dst = row + span0 + 4 * grp;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      *reinterpret_cast<u32x4_t*>(dst + 16 * q) = u32x4_t{w[q][0], w[q][1], w[q][2], w[q][3]};
+  }
+}
+
 // One step of a stream's online chain: the 16 scaled logits y of the stream's run in one
 // tile are folded into the running (max, sum), exponentials added in ascending column order;
 // `tl` is the target's position inside the run (outside [0, 16): not in this run). A run that
