@@ -77,7 +77,7 @@ def _parse():
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-T table")
     ap.add_argument("--rotate-weights", action="store_true",
                     help="gate_up_tN / down_tN legs: launch over copies of the weight (~1.3 GB in rotation) so that it is read from HBM")
-    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|gate_up_tN|down_tN|logp|logp_decode|logp_mid|logp_logits|logp_bwd|logp_bwd_256|from_logits|ffn|tree|tree_down|tree_decode|copy|power (used for profiling)")
+    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|gate_up_tN|down_tN|logp|logp_decode|logp_mid|logp_logits|logp_bwd|logp_bwd_256|from_logits|from_logits_bwd|ffn|tree|tree_down|tree_decode|copy|power (used for profiling)")
     return ap.parse_args()
 
 
@@ -282,7 +282,7 @@ def main() -> int:
         print(json.dumps({"leg": args.only, "ms": ms, "tflops": flops / ms * 1e-9,
                           "launches": args.steps + args.warmup}))
         return 0
-    if args.only in ("logp_bwd", "logp_bwd_256", "logp_logits", "from_logits"):
+    if args.only in ("logp_bwd", "logp_bwd_256", "logp_logits", "from_logits", "from_logits_bwd"):
         from rl_engine import _C
 
         tl = {"logp_bwd_256": 256, "logp_logits": 2048}.get(args.only, 8192)
@@ -295,6 +295,12 @@ def main() -> int:
             _, lse = _C.fused_linear_logp(hid, w_lm, tgt)
             g = torch.randn((tl,), generator=gen, device=dev)
             ms = _time_calls(lambda: _C.fused_linear_logp_bwd(hid, w_lm, tgt, lse, g, None), args.steps, args.warmup)
+        elif args.only == "from_logits_bwd":
+            logits = randn(tl, VOCAB, 4.0)
+            lse = torch.full((tl,), 12.0, device=dev)
+            g = torch.randn((tl,), generator=gen, device=dev)
+            zero = torch.zeros((tl,), device=dev)
+            ms = _time_calls(lambda: _C.hip_deterministic_logp_backward(logits, lse, g, zero, tgt, 0, VOCAB, False), args.steps, args.warmup)
         else:
             logits = randn(tl, VOCAB, 4.0)
             ms = _time_calls(lambda: _C.hip_deterministic_logp_from_logits(logits, tgt, 0, VOCAB, 64), args.steps, args.warmup)
@@ -566,7 +572,19 @@ def main() -> int:
             "gbps": round(by_fl / ms_fl * 1e-6, 1),
             "frac_of_hbm_peak": round(by_fl / ms_fl * 1e-6 / PEAK_HBM_GBPS, 4),
         }
-        del logits
+        # its backward: one read of the logits and one write of their gradient
+        lse_fl = torch.full((tl,), 12.0, device=dev)
+        g_fl = torch.randn((tl,), generator=gen, device=dev)
+        z_fl = torch.zeros((tl,), device=dev)
+        ms_fb = _time_calls(lambda: _C.hip_deterministic_logp_backward(logits, lse_fl, g_fl, z_fl, tgt, 0, VOCAB, False), 10, 4)
+        result["linear_logp"]["from_logits_backward"] = {
+            "workload": "bf16 logits[8192,151936] + lse -> bf16 d(logits) (coef * (onehot - p))",
+            "ms": round(ms_fb, 3),
+            "bound": "hbm",
+            "gbps": round(2 * by_fl / ms_fb * 1e-6, 1),
+            "frac_of_hbm_peak": round(2 * by_fl / ms_fb * 1e-6 / PEAK_HBM_GBPS, 4),
+        }
+        del logits, lse_fl, g_fl, z_fl
         # rollout scale: 64 rollouts x 1024 tokens through the fused LogP, then the GRPO ratio / k3-KL epilogue
         from rl_engine.ops.loss import grpo_ratio_kl_loss
 
