@@ -222,6 +222,11 @@ __device__ __forceinline__ void merge_lane_states(int lane, float& m, float& s) 
   m = n;
 }
 
+template <bool V>
+struct BoolConstant {
+  static constexpr bool value = V;
+};
+
 constexpr int kTileLanes = 16;                    // lanes that share a tile
 constexpr int kTilesPerWave = kWave / kTileLanes;  // 4
 
@@ -273,15 +278,21 @@ __global__ __launch_bounds__(256) void logits_tile_stats_kernel(TileStatsArgs a)
 
     float m = kNegInf, s = 0.f;
     int g = g0 + l16;  // this lane's next vector
-    for (int b = 0; b < clean; ++b, g += kStep) {
-      RawVector<ELEM, ALIGNED> raw[kBatch];
+    // Clean batches, the loads rotating through the four raw vectors: a vector's registers are free once it is
+    // unpacked, and the same vector of the next batch is fetched into them before the fold, so a lane always
+    // has three or four loads in flight instead of none while it folds the end of a batch.
+    RawVector<ELEM, ALIGNED> raw[kBatch];
+    if (clean > 0) {
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) raw[u].load(row_ptr, g + u * kTileLanes, cols);
+    }
+    auto clean_batch = [&](auto more, bool first) __attribute__((always_inline)) {
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) {
         float y[VEC];
         raw[u].unpack(y);
-        if (u == 0 && b == 0) {  // the tile may start inside its first vector (lane 0 of the 16)
+        if constexpr (decltype(more)::value) raw[u].load(row_ptr, g + kStep + u * kTileLanes, cols);
+        if (u == 0 && first) {  // the tile may start inside its first vector (lane 0 of the 16)
           const int lo = lo_col - g * VEC;
 #pragma unroll
           for (int i = 0; i < VEC; ++i) y[i] = (i >= lo) ? y[i] : kNegInf;
@@ -292,9 +303,13 @@ __global__ __launch_bounds__(256) void logits_tile_stats_kernel(TileStatsArgs a)
         }
         fold_logit_vector(y, m, s);
       }
+    };
+    for (int b = 0; b + 1 < clean; ++b, g += kStep) clean_batch(BoolConstant<true>{}, b == 0);
+    if (clean > 0) {
+      clean_batch(BoolConstant<false>{}, clean == 1);
+      g += kStep;
     }
     for (int b = clean; b * kBatch < slots; ++b, g += kStep) {  // the rest: clamped loads, both edges masked
-      RawVector<ELEM, ALIGNED> raw[kBatch];
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) {
         const int gu = g + u * kTileLanes;
