@@ -56,8 +56,11 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
   } else if constexpr (LOOP == kLoopStagedKMajor) {
     tile_mainloop_staged_kmajor<S, KS>(W, X, n0, m0, K, lds, acc);
   } else if constexpr (LOOP >= kLoopPingPongKMajor) {
-    tile_mainloop_pingpong<S, loop_weight_kmajor(LOOP), loop_act_kmajor(LOOP), PlainRowMap<S>, KS, NS>(W, X, n0, m0, K,
-                                                                                                        lds, acc);
+    // whole K tiles through the ping-pong loop, the rest of a reduction length that 64 does not divide behind it
+    const int k_whole = K & ~(kTileK - 1);
+    tile_mainloop_pingpong<S, loop_weight_kmajor(LOOP), loop_act_kmajor(LOOP), PlainRowMap<S>, KS, NS>(
+        W, X, n0, m0, k_whole, lds, acc);
+    if (k_whole != K) tile_tail_step<S, loop_weight_kmajor(LOOP), loop_act_kmajor(LOOP)>(W, X, n0, m0, k_whole, K, lds, acc);
   } else if constexpr (LOOP == kLoopPingPong) {
     tile_mainloop_pingpong<S, false, false, PlainRowMap<S>, KS, NS>(W, X, n0, m0, K, lds, acc);
   } else {
@@ -338,8 +341,11 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
   const bool allow_pingpong = (config & RLK_GEMM_CFG_FORCE_STAGED) == 0;
   config &= ~RLK_GEMM_CFG_FORCE_STAGED;
   const bool w_kmajor = !w_native && view_is_kmajor_fast(W), x_kmajor = !x_native && view_is_kmajor_fast(X);
-  if (allow_pingpong && (K % kTileK) == 0 && (w_kmajor || x_kmajor) && (w_native || w_kmajor) &&
-      (x_native || x_kmajor)) {
+  // A reduction length that 64 does not divide (the token count of a weight gradient) runs its whole K tiles in
+  // the same loops and the rest in a register-staged step behind them; a native operand of the pair then
+  // needs whole 16-byte chunks (K % 8 == 0).
+  const bool k_fits = K >= kTileK && ((K % kTileK) == 0 || (w_kmajor && x_kmajor) || (K % kChunkElems) == 0);
+  if (allow_pingpong && k_fits && (w_kmajor || x_kmajor) && (w_native || w_kmajor) && (x_native || x_kmajor)) {
     const int loop = w_kmajor ? (x_kmajor ? kLoopPingPongBothKMajor : kLoopPingPongKMajor) : kLoopPingPongXKMajor;
     // Only the shapes with 64-feature wave columns have the transposing loop, and a K-major
     // activation needs at least 128 tokens per tile.

@@ -147,12 +147,14 @@ __device__ __forceinline__ u32x4_t read_kmajor_fragment(const char* col, int j16
   return u32x4_t{half[0].x, half[0].y, half[1].x, half[1].y};
 }
 
-// Global -> register staging of one K tile of a K-major weight operand (w[k * ld + n], features contiguous):
-// a thread's chunk is 8 consecutive features at one k, stored into the K-major stage layout above.
-// Needs N % 8 == 0, 16-byte aligned rows and K % 64 == 0 (no K tail).
+// Global -> register staging of one K tile of a K-major operand (w[k * ld + n], rows contiguous; the weight
+// B[K, N], or an activation stored token-contiguous): a thread's chunk is 8 consecutive rows at one k, stored
+// into the K-major stage layout above. Needs rows % 8 == 0 and 16-byte aligned K rows. load<true> fills the
+// K rows at and past K with zeros (their address is clamped to K row 0, which always exists).
 template <int ITERS, int CHUNKS, int THREADS>
 struct KMajorStager {
-  const bf16_bits* src[ITERS];  // chunk source at k0 = 0
+  const bf16_bits* src[ITERS];  // chunk source at K row 0
+  int krow[ITERS];              // K row of the chunk inside a tile
   int lds_off[ITERS];
   u32x4_t regs[ITERS];
   int64_t ld;
@@ -168,13 +170,25 @@ struct KMajorStager {
       const int c = ci % kRowChunks;
       int n = n0 + col * 64 + c * kChunkElems;
       n = n + kChunkElems <= w.rows ? n : w.rows - kChunkElems;  // features past the edge are computed, never stored
-      src[i] = w.ptr + (int64_t)k * ld + n;
+      src[i] = w.ptr + n;
+      krow[i] = k;
       lds_off[i] = col * (kTileK * kRowBytes) + k * kRowBytes + ((c ^ kmajor_swizzle(k)) << 4);
     }
   }
-  __device__ __forceinline__ void load(int k0) {
+  template <bool TAIL>
+  __device__ __forceinline__ void load(int k0, int K) {
 #pragma unroll
-    for (int i = 0; i < ITERS; ++i) regs[i] = *reinterpret_cast<const u32x4_t*>(src[i] + (int64_t)k0 * ld);
+    for (int i = 0; i < ITERS; ++i) {
+      const int k = k0 + krow[i];
+      if constexpr (TAIL) {
+        const bool ok = k < K;
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(src[i] + (int64_t)(ok ? k : 0) * ld);
+        const u32x4_t z = {0u, 0u, 0u, 0u};
+        regs[i] = ok ? v : z;
+      } else {
+        regs[i] = *reinterpret_cast<const u32x4_t*>(src[i] + (int64_t)k * ld);
+      }
+    }
   }
   __device__ __forceinline__ void store(char* lds_stage, int tid) {
 #pragma unroll
@@ -199,8 +213,9 @@ struct IntTag {
 // tile in flight per workgroup would make every iteration a memory round trip. Every load is issued
 // unconditionally (past the end it repeats the last K tile and its data is dropped), so the waits the
 // compiler places count loads on one straight path.
-// The last stage may hold fewer than KS tiles. Needs BN % 64 == 0, K % 64 == 0, N % 8 == 0;
-// 2 * KS * kStageBytes of LDS.
+// The last stage may hold fewer than KS tiles, and the last K tile fewer than 64 K values (the rest is
+// filled with zeros in both operands, as in every other loop). Needs BN % 64 == 0, N % 8 == 0, K % 8 == 0
+// (the activation chunks); 2 * KS * kStageBytes of LDS.
 template <class S, int KS>
 __device__ __forceinline__ void tile_mainloop_staged_kmajor(const MatView& W, const MatView& X, int n0, int m0, int K,
                                                             char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
@@ -228,22 +243,30 @@ __device__ __forceinline__ void tile_mainloop_staged_kmajor(const MatView& W, co
   const int frag_lo = (grp ^ (l16 & 7)) << 4;
   const int x_row_base = S::BN * kRowBytes + (wave_m * 16 * S::TM + l16) * kRowBytes;
   constexpr int kSpan = KS * S::kStageBytes;
-  const int k_tiles = K / kTileK;
+  const int k_tiles = (K + kTileK - 1) / kTileK;
   const int stages = (k_tiles + KS - 1) / KS;
 
+  // K values at and past K (the tail of the last tile) read a clamped address and become zeros.
   auto load_stage = [&](auto set, int st) __attribute__((always_inline)) {
     constexpr int R = decltype(set)::value;
+    const u32x4_t zero = {0u, 0u, 0u, 0u};
 #pragma unroll
     for (int q = 0; q < KS; ++q) {
       int t = st * KS + q;
       t = t < k_tiles ? t : k_tiles - 1;
       const int k0 = t * kTileK;
 #pragma unroll
-      for (int i = 0; i < S::kWIters; ++i)
-        wr[R][q][i] = *reinterpret_cast<const u32x4_t*>(sw.src[i] + (int64_t)k0 * sw.ld);
+      for (int i = 0; i < S::kWIters; ++i) {
+        const int k = k0 + sw.krow[i];
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(sw.src[i] + (int64_t)(k < K ? k : 0) * sw.ld);
+        wr[R][q][i] = k < K ? v : zero;
+      }
 #pragma unroll
-      for (int i = 0; i < S::kXIters; ++i)
-        xr[R][q][i] = *reinterpret_cast<const u32x4_t*>(sx.src[i] + k0 + sx.chunk_k[i]);
+      for (int i = 0; i < S::kXIters; ++i) {
+        const int k = k0 + sx.chunk_k[i];  // K % 8 == 0: a chunk is all in or all out
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(sx.src[i] + (k < K ? k : 0));
+        xr[R][q][i] = k < K ? v : zero;
+      }
     }
   };
   // A tile past the end lands in a slot that is never multiplied.
@@ -862,6 +885,91 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
   }
   __builtin_amdgcn_s_waitcnt(kWaitAll0);
   wg_barrier();  // callers reuse the LDS after the loop
+}
+
+// ---------------------------------------------------------------------------
+// The last, partial K tile behind a ping-pong loop that has a K-major operand.
+//
+// Direct-to-LDS loads move whole 64-wide K tiles; a reduction length that is not a multiple of 64 (the token
+// count of a weight gradient) used to send the whole GEMM to the element-wise loader. Instead the ping-pong
+// loop runs over the K / 64 whole tiles and this step adds the rest to the same accumulators: both operands of
+// K values [k0, K) go through registers (16-byte chunks, zeros at and past K, addresses clamped into the
+// matrix), into stage 0 in the layout the loop uses, and through the same fragment reads and two MFMA steps.
+// The chain of an output element is the one every other loop runs: K tiles ascending, the tail zero-filled
+// to a multiple of 64 in both operands. A native operand needs K % 8 == 0 (a chunk is all in or all out).
+// Call it after the loop (which ends on a barrier); it ends on a barrier as well.
+// ---------------------------------------------------------------------------
+// Everything here is derived from a thread index the compiler cannot see through, so that none of the step's
+// addresses is computed ahead of the main loop and kept alive across it (which made the 256 x 256 kernels
+// spill hundreds of registers inside that loop).
+template <class S, bool WK, bool XK>
+__device__ __forceinline__ void tile_tail_step(const MatView& W, const MatView& X, int n0, int m0, int k0, int K,
+                                               char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
+  static_assert(!WK || S::TN == 4, "K-major weights need 64-feature wave columns");
+  static_assert(!XK || S::BM % 128 == 0, "K-major activations need whole 64-token columns per wave group");
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_n = wave % S::WN;
+  const int wave_m = wave / S::WN;
+  char* x_stage = lds + S::BN * kRowBytes;
+
+  if constexpr (WK) {
+    KMajorStager<S::kWIters, S::kWChunks, S::kThreads> sw;
+    sw.init(W, n0, tid);
+    sw.template load<true>(k0, K);
+    sw.store(lds, tid);
+  } else {
+    Stager<S::kWIters, S::kWChunks, S::kThreads, true> sw;
+    sw.init(W, n0, tid, [](int r) { return weight_row_of_lds_row<S>(r); });
+    sw.template load<true>(k0, K);
+    sw.store(lds, tid);
+  }
+  if constexpr (XK) {
+    KMajorStager<S::kXIters, S::kXChunks, S::kThreads> sx;
+    sx.init(X, m0, tid);
+    sx.template load<true>(k0, K);
+    sx.store(x_stage, tid);
+  } else {
+    Stager<S::kXIters, S::kXChunks, S::kThreads, true> sx;
+    sx.init(X, m0, tid, [](int r) { return r; });
+    sx.template load<true>(k0, K);
+    sx.store(x_stage, tid);
+  }
+  __syncthreads();
+
+  const int l16 = lane & 15;
+  const int grp = lane >> 4;
+  const int frag_lo = (grp ^ (l16 & 7)) << 4;
+  const int w_row_base = (wave_n * 16 * S::TN + l16) * kRowBytes;
+  const int x_row_base = (wave_m * 16 * S::TM + l16) * kRowBytes;
+#pragma unroll
+  for (int s = 0; s < kTileK / kMfmaK; ++s) {
+    u32x4_t wf[S::TN], xf[S::TM];
+#pragma unroll
+    for (int jn = 0; jn < S::TN; ++jn) {
+      if constexpr (WK) {
+        wf[jn] = read_kmajor_fragment(lds + wave_n * (64 * kRowBytes), jn, s, l16, grp);
+      } else {
+        wf[jn] = *reinterpret_cast<const u32x4_t*>(lds + w_row_base + jn * 16 * kRowBytes + (frag_lo ^ (s << 6)));
+      }
+    }
+#pragma unroll
+    for (int jm = 0; jm < S::TM; ++jm) {
+      if constexpr (XK) {
+        const int col = wave_m * (S::TM / 4) + (jm >> 2);
+        xf[jm] = read_kmajor_fragment(x_stage + col * (64 * kRowBytes), jm & 3, s, l16, grp);
+      } else {
+        xf[jm] = *reinterpret_cast<const u32x4_t*>(x_stage + x_row_base + jm * 16 * kRowBytes + (frag_lo ^ (s << 6)));
+      }
+    }
+#pragma unroll
+    for (int jn = 0; jn < S::TN; ++jn)
+#pragma unroll
+      for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = mfma_16x16x32(wf[jn], xf[jm], acc[jn][jm]);
+  }
+  __syncthreads();
 }
 
 // ---------------------------------------------------------------------------

@@ -335,7 +335,8 @@ def test_operand_layouts_give_the_same_bits(gemm, native, shape):
     assert _same_bits(native.det_gemm_fwd_rhs_transposed(a, unaligned), expected)
 
 
-@pytest.mark.parametrize("shape", [(512, 1024, 4096), (300, 1000, 192), (1000, 2056, 320), (64, 8, 64), (7, 1024, 1024), (2048, 4096, 1024)])
+@pytest.mark.parametrize("shape", [(512, 1024, 4096), (300, 1000, 192), (1000, 2056, 320), (64, 8, 64), (7, 1024, 1024), (2048, 4096, 1024),
+                                   (520, 1024, 200), (264, 520, 1000), (16, 128, 72)])  # the last three: K % 64 != 0, a zero-filled tail tile
 def test_kmajor_weight_fast_path_gives_the_same_bits(gemm, native, shape):
     """B[K,N] with N contiguous (the `a @ b`, prepared-weight and input-gradient
     form) and token-contiguous activations are read through transposing LDS loads. Each must
@@ -368,6 +369,26 @@ def test_kmajor_weight_fast_path_gives_the_same_bits(gemm, native, shape):
     acc_nk = native.det_gemm_fwd_out_fp32(a, bt.t())
     assert torch.equal(acc_kn.view(torch.int32), acc_nk.view(torch.int32))
     assert _same_bits(acc_kn.to(torch.bfloat16), expected)
+
+
+@pytest.mark.parametrize("tokens", (64, 65, 100, 257, 1000, 4095))
+def test_weight_gradient_at_any_token_count_keeps_the_bits(gemm, native, oracle, tokens):
+    """dW = dY^T @ X reduces over the tokens with both operands K-major. A token count that 64 does not divide
+    runs its whole K tiles in the transposing ping-pong loop and the rest in a zero-filled tail step: the bits
+    of the element loader (forced 16x16 tile on transposed copies), whatever the tile."""
+    n, k = 384, 520
+    x = inputs.randn_bf16(71, tokens, k).to(DEV)
+    dy = inputs.randn_bf16(72, tokens, n, 0.05).to(DEV)
+    expected = gemm.mfma_gemm(dy.t().contiguous(), x.t().contiguous().t(), config="16x16")  # [n, tokens] @ [tokens, k]
+    for name in ("auto", "256x256", "256x128"):
+        assert _same_bits(gemm.mfma_gemm(dy.t(), x, config=name), expected), name
+    assert _same_bits(native.det_gemm_db_transposed(x, dy), expected)
+    assert _same_bits(gemm.det_gemm_linear_weight_gradient(x, dy), expected)
+    # the mixed pairs need whole 16-byte chunks of the native operand
+    if tokens % 8 == 0:
+        assert _same_bits(gemm.mfma_gemm(dy.t().contiguous(), x, config="256x256"), expected)
+        assert _same_bits(gemm.mfma_gemm(dy.t(), x.t().contiguous().t(), config="256x256"), expected)
+    _assert_parity(oracle, expected, dy.t().contiguous().cpu(), x.t().contiguous().cpu(), f"weight gradient, {tokens} tokens")
 
 
 @pytest.mark.parametrize("k", (1, 8, 31, 32, 33, 65, 100, 1000))
