@@ -58,8 +58,15 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
   } else if constexpr (LOOP >= kLoopPingPongKMajor) {
     // whole K tiles through the ping-pong loop, the rest of a reduction length that 64 does not divide behind it
     const int k_whole = K & ~(kTileK - 1);
-    tile_mainloop_pingpong<S, loop_weight_kmajor(LOOP), loop_act_kmajor(LOOP), PlainRowMap<S>, KS, NS>(
-        W, X, n0, m0, k_whole, lds, acc);
+    if (k_whole > 0) {
+      tile_mainloop_pingpong<S, loop_weight_kmajor(LOOP), loop_act_kmajor(LOOP), PlainRowMap<S>, KS, NS>(
+          W, X, n0, m0, k_whole, lds, acc);
+    } else {  // fewer than 64 K values: the tail step is the whole reduction
+#pragma unroll
+      for (int jn = 0; jn < S::TN; ++jn)
+#pragma unroll
+        for (int jm = 0; jm < S::TM; ++jm) acc[jn][jm] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
     if (k_whole != K) tile_tail_step<S, loop_weight_kmajor(LOOP), loop_act_kmajor(LOOP)>(W, X, n0, m0, k_whole, K, lds, acc);
   } else if constexpr (LOOP == kLoopPingPong) {
     tile_mainloop_pingpong<S, false, false, PlainRowMap<S>, KS, NS>(W, X, n0, m0, K, lds, acc);
@@ -344,7 +351,7 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
   // A reduction length that 64 does not divide (the token count of a weight gradient) runs its whole K tiles in
   // the same loops and the rest in a register-staged step behind them; a native operand of the pair then
   // needs whole 16-byte chunks (K % 8 == 0).
-  const bool k_fits = K >= kTileK && ((K % kTileK) == 0 || (w_kmajor && x_kmajor) || (K % kChunkElems) == 0);
+  const bool k_fits = K >= 1 && ((K % kTileK) == 0 || (w_kmajor && x_kmajor) || (K % kChunkElems) == 0);
   if (allow_pingpong && k_fits && (w_kmajor || x_kmajor) && (w_native || w_kmajor) && (x_native || x_kmajor)) {
     const int loop = w_kmajor ? (x_kmajor ? kLoopPingPongBothKMajor : kLoopPingPongKMajor) : kLoopPingPongXKMajor;
     // Only the shapes with 64-feature wave columns have the transposing loop, and a K-major

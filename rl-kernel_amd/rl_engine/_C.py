@@ -205,10 +205,10 @@ det_gemm_seq_fp32 = det_gemm_fwd_fp32
 def _reduction_major(t: torch.Tensor) -> torch.Tensor:
     """``t.t()`` ready for a GEMM whose reduction runs over ``t``'s rows.
 
-    A row-major ``t[M, C]`` with ``C % 8 == 0``, ``M >= 64`` and 16-byte aligned rows is
-    passed as the plain view ``t.t()``: the library reads such a K-major operand through
-    transposing LDS loads, whole 64-row tiles directly and the rest of an ``M`` that 64 does
-    not divide through registers. Anything else gets a value-preserving copy with the
+    A row-major ``t[M, C]`` with ``C % 8 == 0`` and 16-byte aligned rows is passed as the
+    plain view ``t.t()``: the library reads such a K-major operand through transposing LDS
+    loads, whole 64-row tiles directly and the rest of an ``M`` that 64 does not divide
+    through registers. Anything else gets a value-preserving copy with the
     reduction axis contiguous.
     """
     tt = t.t()
@@ -217,7 +217,7 @@ def _reduction_major(t: torch.Tensor) -> torch.Tensor:
     if (
         t.stride(1) == 1
         and t.size(1) % 8 == 0
-        and t.size(0) >= 64
+        and t.size(0) >= 1
         and t.stride(0) % 8 == 0
         and t.data_ptr() % 16 == 0
     ):

@@ -371,7 +371,7 @@ def test_kmajor_weight_fast_path_gives_the_same_bits(gemm, native, shape):
     assert _same_bits(acc_kn.to(torch.bfloat16), expected)
 
 
-@pytest.mark.parametrize("tokens", (64, 65, 100, 257, 1000, 4095))
+@pytest.mark.parametrize("tokens", (1, 7, 63, 64, 65, 100, 257, 1000, 4095))
 def test_weight_gradient_at_any_token_count_keeps_the_bits(gemm, native, oracle, tokens):
     """dW = dY^T @ X reduces over the tokens with both operands K-major. A token count that 64 does not divide
     runs its whole K tiles in the transposing ping-pong loop and the rest in a zero-filled tail step: the bits
