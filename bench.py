@@ -559,6 +559,13 @@ def main() -> int:
             "min_hbm_bytes": 3 * 2.0 * VOCAB * HIDDEN,  # the weight read twice, its gradient written once
             "frac_of_hbm_peak": round(3 * 2.0 * VOCAB * HIDDEN / ms_bs * 1e-6 / PEAK_HBM_GBPS, 4),
         }
+        # a token count that 64 does not divide: the weight gradient reduces over it (whole K tiles + a tail step)
+        hid_r, tgt_r = hid[:8191].contiguous(), tgt[:8191].contiguous()
+        _, lse_r = _C.fused_linear_logp(hid_r, w_lm, tgt_r)
+        g_r = torch.randn((8191,), generator=gen, device=dev)
+        ms_br = _time_calls(lambda: _C.fused_linear_logp_bwd(hid_r, w_lm, tgt_r, lse_r, g_r, None), 4, 2)
+        result["linear_logp"]["backward_8191_tokens"] = {"ms": round(ms_br, 3), "ratio_to_8192_tokens": round(ms_br / ms_bwd, 3)}
+        del hid_r, tgt_r, lse_r, g_r
         del hid_s, tgt_s, hid_b, tgt_b, lse_b, g_b
         # the stage that reuses materialised logits: one pass over [8192, 151936] bf16
         logits = randn(tl, VOCAB, 4.0)
