@@ -307,8 +307,10 @@ int pick_det_gemm_config(int M, int N, int K) {
   };
   // 192 x 256 (three quarters of the large tile at 0.89 of its throughput) fills the rounds that
   // N / 256 leaves half empty: gate_up at 1024 tokens is 512 tiles = two full rounds instead of
-  // 384 = one and a half (169 -> 152 us), qkv at 3072 tokens 150 -> 128 us. Only where 192 divides N:
-  // a ragged last feature tile costs a whole tile time.
+  // 384 = one and a half (169 -> 152 us), qkv at 3072 tokens 150 -> 128 us. Where 192 does not divide N the
+  // last feature tile is partly empty and the shape counts as 0.85: it still wins where it turns a round and a
+  // fraction into less (N = 5120 at 4096 tokens 293 -> 256 us, N = 10240 at 2048 tokens 190 -> 162 us, N = 2560 at
+  // 8192 tokens 347 -> 308 us) and loses the tie against 256 x 128 at N = 4096, 2048 tokens (177 against 166 us).
   static const Candidate kCandidates[] = {
       {RLK_GEMM_CFG_256x256, 256, 256, 1.00}, {RLK_GEMM_CFG_192x256, 192, 256, 0.89},
       {RLK_GEMM_CFG_256x128, 256, 128, 0.65},
@@ -319,12 +321,13 @@ int pick_det_gemm_config(int M, int N, int K) {
   int best = RLK_GEMM_CFG_64x64;
   double best_time = 1e300;
   for (const Candidate& c : kCandidates) {
-    if (c.config == RLK_GEMM_CFG_192x256 && (N % 192 != 0 || K % kTileK != 0)) continue;
+    if (c.config == RLK_GEMM_CFG_192x256 && K % kTileK != 0) continue;
+    const double quality = (c.config == RLK_GEMM_CFG_192x256 && N % 192 != 0) ? 0.85 : c.quality;
     const int64_t tiles = tile_count(M, N, c.bm, c.bn);
     const int64_t full = tiles / kCus;
     const double part = (double)(tiles - full * kCus) / kCus;
     const double rounds = (double)full + (part > 0.0 ? (part > 0.9 ? part : 0.9) : 0.0);
-    const double t = rounds * (double)(c.bn * c.bm) / c.quality;
+    const double t = rounds * (double)(c.bn * c.bm) / quality;
     if (t < best_time * 0.999) {
       best_time = t;
       best = c.config;
