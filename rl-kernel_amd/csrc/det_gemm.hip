@@ -23,10 +23,12 @@ enum : int {
   kLoopPingPongXKMajor = 4,  // activation K-major
   kLoopPingPongBothKMajor = 5,
   kLoopSolo = 6,  // four waves, one per SIMD
-  kLoopStagedKMajor = 7  // register-staged, weight K-major (the small tiles)
+  kLoopStagedKMajor = 7,     // register-staged, weight K-major (the small tiles), K % 64 == 0
+  kLoopStagedKMajorTail = 8  // the same with a zero-filled last K tile
 };
 constexpr bool loop_weight_kmajor(int loop) {
-  return loop == kLoopPingPongKMajor || loop == kLoopPingPongBothKMajor || loop == kLoopStagedKMajor;
+  return loop == kLoopPingPongKMajor || loop == kLoopPingPongBothKMajor || loop == kLoopStagedKMajor ||
+         loop == kLoopStagedKMajorTail;
 }
 constexpr bool loop_act_kmajor(int loop) { return loop == kLoopPingPongXKMajor || loop == kLoopPingPongBothKMajor; }
 
@@ -53,8 +55,8 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
   f32x4_t acc[S::TN][S::TM];
   if constexpr (LOOP == kLoopSolo) {
     tile_mainloop_solo<S>(W, X, n0, m0, K, lds, acc);
-  } else if constexpr (LOOP == kLoopStagedKMajor) {
-    tile_mainloop_staged_kmajor<S, KS>(W, X, n0, m0, K, lds, acc);
+  } else if constexpr (LOOP == kLoopStagedKMajor || LOOP == kLoopStagedKMajorTail) {
+    tile_mainloop_staged_kmajor<S, KS, LOOP == kLoopStagedKMajorTail>(W, X, n0, m0, K, lds, acc);
   } else if constexpr (LOOP >= kLoopPingPongKMajor) {
     // whole K tiles through the ping-pong loop, the rest of a reduction length that 64 does not divide behind it
     const int k_whole = K & ~(kTileK - 1);
@@ -252,6 +254,9 @@ template <class S>
 static hipError_t launch_staged_kmajor(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
                                        bool out_f32, hipStream_t stream) {
   constexpr int kKs = 128 * 1024 / (2 * S::kStageBytes) >= 4 ? 4 : 2;
+  if (K % kTileK != 0)
+    return out_f32 ? launch_tile<S, kLoopStagedKMajorTail, true, kKs, 2>(W, X, C, ldc, M, N, K, stream)
+                   : launch_tile<S, kLoopStagedKMajorTail, false, kKs, 2>(W, X, C, ldc, M, N, K, stream);
   return out_f32 ? launch_tile<S, kLoopStagedKMajor, true, kKs, 2>(W, X, C, ldc, M, N, K, stream)
                  : launch_tile<S, kLoopStagedKMajor, false, kKs, 2>(W, X, C, ldc, M, N, K, stream);
 }

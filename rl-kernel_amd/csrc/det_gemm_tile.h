@@ -216,7 +216,7 @@ struct IntTag {
 // The last stage may hold fewer than KS tiles, and the last K tile fewer than 64 K values (the rest is
 // filled with zeros in both operands, as in every other loop). Needs BN % 64 == 0, N % 8 == 0, K % 8 == 0
 // (the activation chunks); 2 * KS * kStageBytes of LDS.
-template <class S, int KS>
+template <class S, int KS, bool RAGGED>
 __device__ __forceinline__ void tile_mainloop_staged_kmajor(const MatView& W, const MatView& X, int n0, int m0, int K,
                                                             char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
   static_assert(S::BN % 64 == 0, "whole 64-feature columns");
@@ -246,7 +246,9 @@ __device__ __forceinline__ void tile_mainloop_staged_kmajor(const MatView& W, co
   const int k_tiles = (K + kTileK - 1) / kTileK;
   const int stages = (k_tiles + KS - 1) / KS;
 
-  // K values at and past K (the tail of the last tile) read a clamped address and become zeros.
+  // RAGGED: K values at and past K (the tail of the last tile) read a clamped address and become zeros. The
+  // choice is made at compile time: a select behind every load, or a branch around the loads, costs the loop
+  // with whole tiles 15 % (the waits in front of the selects flatten its two stages of loads in flight).
   auto load_stage = [&](auto set, int st) __attribute__((always_inline)) {
     constexpr int R = decltype(set)::value;
     const u32x4_t zero = {0u, 0u, 0u, 0u};
@@ -258,14 +260,22 @@ __device__ __forceinline__ void tile_mainloop_staged_kmajor(const MatView& W, co
 #pragma unroll
       for (int i = 0; i < S::kWIters; ++i) {
         const int k = k0 + sw.krow[i];
-        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(sw.src[i] + (int64_t)(k < K ? k : 0) * sw.ld);
-        wr[R][q][i] = k < K ? v : zero;
+        if constexpr (RAGGED) {
+          const u32x4_t v = *reinterpret_cast<const u32x4_t*>(sw.src[i] + (int64_t)(k < K ? k : 0) * sw.ld);
+          wr[R][q][i] = k < K ? v : zero;
+        } else {
+          wr[R][q][i] = *reinterpret_cast<const u32x4_t*>(sw.src[i] + (int64_t)k * sw.ld);
+        }
       }
 #pragma unroll
       for (int i = 0; i < S::kXIters; ++i) {
         const int k = k0 + sx.chunk_k[i];  // K % 8 == 0: a chunk is all in or all out
-        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(sx.src[i] + (k < K ? k : 0));
-        xr[R][q][i] = k < K ? v : zero;
+        if constexpr (RAGGED) {
+          const u32x4_t v = *reinterpret_cast<const u32x4_t*>(sx.src[i] + (k < K ? k : 0));
+          xr[R][q][i] = k < K ? v : zero;
+        } else {
+          xr[R][q][i] = *reinterpret_cast<const u32x4_t*>(sx.src[i] + k);
+        }
       }
     }
   };
