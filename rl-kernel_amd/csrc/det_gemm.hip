@@ -349,8 +349,47 @@ static bool view_is_kmajor_fast(const MatView& v) {
          (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0 && (v.rows % kChunkElems) == 0;
 }
 
+// A token count just above a multiple of 256 (4097, 8200 ...) gives the large tiles a last row of token tiles that
+// is nearly empty; when that row is what opens another round of workgroups, the few tokens cost a whole tile
+// time (down at 4097 tokens: 272 tiles = two rounds instead of one, 0.54 against 0.27 ms). Rows are independent,
+// so the remainder can run as a launch of its own on the few-token kernels without changing a bit. Returns
+// whether that pays: the round the remainder opens, priced at 11 + 21 K / 1024 us for a 256 x 256 tile
+// (measured on gate_up across K), against the few-token launch, which streams the weight once.
+static bool remainder_launch_pays(int M, int N, int K, int rest, bool fast_few_tokens, bool w_kmajor) {
+  const int64_t feature_tiles = (N + 255) / 256;
+  const int64_t rounds_all = (feature_tiles * ((M + 255) / 256) + 255) / 256;
+  const int64_t rounds_main = (feature_tiles * (M / 256) + 255) / 256;
+  if (rounds_all == rounds_main) return false;  // the remainder's tiles fit beside the last round
+  const double round_us = 11.0 + 21.0 * K / 1024.0;
+  double rest_us;
+  if (w_kmajor) {
+    rest_us = 10.0 + 0.4 * (K / 64.0);  // register-staged small tiles: a chain of K tiles
+  } else if (fast_few_tokens) {
+    rest_us = 8.0 + 2.0 * N * (double)K / 4.5e6 * (rest <= 16 ? 1.0 : 1.5);  // the weight once at 4.5 TB/s
+  } else {
+    return false;
+  }
+  return rest_us < 0.8 * round_us;
+}
+
 hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
                            bool out_f32, int config, hipStream_t stream) {
+  if (config == RLK_GEMM_CFG_AUTO && M > 256 && M % 256 >= 1 && M % 256 <= 64) {
+    const int rest = M % 256;
+    const bool natives = view_is_vectorizable(W) && view_is_vectorizable(X) && K % kTileK == 0 && K >= 1024;
+    const bool kmajor_w = !view_is_vectorizable(W) && view_is_kmajor_fast(W) && view_is_vectorizable(X) &&
+                          K % kChunkElems == 0;
+    if ((natives || kmajor_w) && remainder_launch_pays(M, N, K, rest, natives, kmajor_w)) {
+      MatView head = X, tail = X;
+      head.rows = M - rest;
+      tail.rows = rest;
+      tail.ptr = X.ptr + (int64_t)(M - rest) * X.row_stride;
+      hipError_t err = det_gemm_launch(W, head, C, ldc, M - rest, N, K, out_f32, config, stream);
+      if (err != hipSuccess) return err;
+      char* c_tail = reinterpret_cast<char*>(C) + (int64_t)(M - rest) * ldc * (out_f32 ? 4 : 2);
+      return det_gemm_launch(W, tail, c_tail, ldc, rest, N, K, out_f32, config, stream);
+    }
+  }
   const bool w_native = view_is_vectorizable(W), x_native = view_is_vectorizable(X);
   const bool vec = w_native && x_native && (K % kChunkElems) == 0;
   const bool allow_pingpong = (config & RLK_GEMM_CFG_FORCE_STAGED) == 0;

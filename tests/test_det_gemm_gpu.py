@@ -391,6 +391,27 @@ def test_weight_gradient_at_any_token_count_keeps_the_bits(gemm, native, oracle,
     _assert_parity(oracle, expected, dy.t().contiguous().cpu(), x.t().contiguous().cpu(), f"weight gradient, {tokens} tokens")
 
 
+def test_a_remainder_of_tokens_launched_on_its_own_changes_no_bit(gemm):
+    """513 tokens against 32768 features: the three token rows of 256 x 256 tiles would be 384 tiles, a round and
+    a half; the automatic choice launches the last token separately on the few-token kernel. Rows are
+    independent: every row equals the forced single launch, for the native and the K-major weight."""
+    m, n, k = 513, 32768, 1024
+    a = inputs.randn_bf16(81, m, k).to(DEV)
+    w = inputs.randn_bf16(82, n, k, 0.02).to(DEV)
+    whole = gemm.mfma_gemm(a, w.t(), config="256x256")
+    assert _same_bits(gemm.mfma_gemm(a, w.t()), whole)
+    staging = torch.zeros((m, n + 8), dtype=torch.bfloat16, device=DEV)
+    gemm.mfma_gemm(a, w.t(), out=staging[:, :n])
+    assert _same_bits(staging[:, :n], whole) and bool((staging[:, n:] == 0).all())
+    w_kn = w.t().contiguous()  # [K, N]: the K-major weight
+    assert _same_bits(gemm.mfma_gemm(a[:, :], w_kn), whole)
+    m2, n2, k2 = 4097, 4096, 4096  # the down-projection case: 272 tiles
+    a2 = inputs.randn_bf16(83, m2, k2).to(DEV)
+    w2 = inputs.randn_bf16(84, n2, k2, 0.02).to(DEV)
+    assert _same_bits(gemm.mfma_gemm(a2, w2.t()), gemm.mfma_gemm(a2, w2.t(), config="256x256"))
+    assert _same_bits(gemm.mfma_gemm(a2, w2.t().contiguous()), gemm.mfma_gemm(a2, w2.t(), config="256x256"))
+
+
 @pytest.mark.parametrize("k", (1, 8, 31, 32, 33, 65, 100, 1000))
 def test_ragged_k_equals_zero_padded_k(gemm, k):
     a = inputs.randn_bf16(61, 9, k).to(DEV)
