@@ -15,7 +15,7 @@ PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "librlk_gfx950.so"
 OBJ_DIR = PKG_DIR / "build"  # object files (git-ignored)
-SOURCES = ["det_gemm.hip", "det_gemm_stream.hip", "det_gemm_tree.hip", "det_gemm_seq.hip", "linear_logp.hip",
+SOURCES = ["det_gemm.hip", "det_gemm_stream.hip", "det_gemm_shortk.hip", "det_gemm_tree.hip", "det_gemm_seq.hip", "linear_logp.hip",
     "linear_logp_bwd.hip", "logits_logp.hip", "swiglu.hip", "grpo.hip", "rlk_api.hip"]
 
 HIPCC_FLAGS = [

@@ -390,6 +390,16 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
       return det_gemm_launch(W, tail, c_tail, ldc, rest, N, K, out_f32, config, stream);
     }
   }
+  if ((config & ~RLK_GEMM_CFG_FORCE_STAGED) == RLK_GEMM_CFG_SHORTK) {
+    // Serves a K-major token operand with K <= 256 only (and has no register-staged form); anything else runs
+    // the picked tile kernel (same bits).
+    if (config == RLK_GEMM_CFG_SHORTK && det_gemm_shortk_supported(W, X, M, N, K))
+      return det_gemm_shortk_launch(W, X, C, ldc, M, N, K, out_f32, stream);
+    config = RLK_GEMM_CFG_AUTO | (config & RLK_GEMM_CFG_FORCE_STAGED);
+  }
+  // A weight gradient of up to 256 tokens with many output rows: the feature operand stays in registers.
+  if (config == RLK_GEMM_CFG_AUTO && det_gemm_shortk_supported(W, X, M, N, K) && det_gemm_shortk_pays(M, N))
+    return det_gemm_shortk_launch(W, X, C, ldc, M, N, K, out_f32, stream);
   const bool w_native = view_is_vectorizable(W), x_native = view_is_vectorizable(X);
   const bool vec = w_native && x_native && (K % kChunkElems) == 0;
   const bool allow_pingpong = (config & RLK_GEMM_CFG_FORCE_STAGED) == 0;

@@ -63,6 +63,13 @@ hipError_t det_gemm_stream_launch(const MatView& W, const MatView& X, void* C, i
 hipError_t det_gemm_stream_gated_launch(const MatView& W, const MatView& X, void* Y, int64_t ldy, int M, int I, int K,
                                         hipStream_t stream);
 
+// A reduction of 64 ... 256 values (K % 64 == 0) against a K-major token operand (x[k * ld + m], 16-byte aligned
+// K rows, M % 8 == 0): the feature operand (any strides) stays in registers, the tokens stream through LDS.
+bool det_gemm_shortk_supported(const MatView& W, const MatView& X, int M, int N, int K);
+bool det_gemm_shortk_pays(int M, int N);  // enough token tiles per workgroup to amortise its start
+hipError_t det_gemm_shortk_launch(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
+                                  bool out_f32, hipStream_t stream);
+
 hipError_t fill_zero_launch(void* dst, int64_t rows, int64_t cols, int64_t ld, int elem_bytes,
                             hipStream_t stream);
 

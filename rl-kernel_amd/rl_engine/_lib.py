@@ -39,6 +39,7 @@ GEMM_CONFIGS = {
     "stream64": 14,
     "256x256_solo": 15,
     "192x256": 16,
+    "shortk": 17,
 }
 # OR-ed into a GEMM or LogP configuration: register-staged main loop (bit-neutral).
 FORCE_STAGED = 0x100

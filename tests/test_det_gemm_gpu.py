@@ -391,6 +391,47 @@ def test_weight_gradient_at_any_token_count_keeps_the_bits(gemm, native, oracle,
     _assert_parity(oracle, expected, dy.t().contiguous().cpu(), x.t().contiguous().cpu(), f"weight gradient, {tokens} tokens")
 
 
+@pytest.mark.parametrize("tokens", (64, 128, 192, 256))
+@pytest.mark.parametrize("rows,feats", ((1000, 520), (4160, 768), (8, 16), (72, 250)))
+def test_short_reduction_streaming_kernel_keeps_the_bits(native, tokens, rows, feats):
+    """A weight gradient of up to 256 tokens, dW[rows, feats] = dY[tokens, rows]^T @ X[tokens, feats], on the kernel
+    that keeps the feature operand in registers and streams the K-major token operand: the bits of the element
+    loader (forced 16x16 tile on transposed copies) for bf16 and fp32 results, whole and partial feature blocks
+    and token tiles, a native feature operand, and an output whose rows are not 16-byte aligned."""
+    from rl_engine import _lib
+
+    shortk = _lib.GEMM_CONFIGS["shortk"]
+    reference = _lib.GEMM_CONFIGS["16x16"] | _lib.FORCE_STAGED
+
+    def bits(t):
+        return t.contiguous().view(torch.int32 if t.dtype == torch.float32 else torch.int16)
+
+    dy = inputs.randn_bf16(91, tokens, rows, 0.05).to(DEV)
+    x = inputs.randn_bf16(92, tokens, feats).to(DEV)
+    for dtype in (torch.bfloat16, torch.float32):
+        expected = torch.empty((rows, feats), dtype=dtype, device=DEV)
+        native.gemm_strided(dy.t().contiguous(), x.t().contiguous().t(), expected, config=reference)
+        got = torch.full((rows, feats), 7.0, dtype=dtype, device=DEV)
+        native.gemm_strided(dy.t(), x, got, config=shortk)
+        assert torch.equal(bits(got), bits(expected)), dtype
+        # feature operand in the native layout (its transposed copy)
+        got.fill_(7.0)
+        native.gemm_strided(dy.t(), x.t().contiguous().t(), got, config=shortk)
+        assert torch.equal(bits(got), bits(expected)), ("native feature operand", dtype)
+        # rows of the output that start at odd elements: the element-wise stores, nothing written beside them
+        wide = torch.full((rows, feats + 3), 7.0, dtype=dtype, device=DEV)
+        native.gemm_strided(dy.t(), x, wide[:, 1 : feats + 1], config=shortk)
+        assert torch.equal(bits(wide[:, 1 : feats + 1]), bits(expected)), ("unaligned rows", dtype)
+        assert bool((wide[:, 0] == 7.0).all()) and bool((wide[:, feats + 1 :] == 7.0).all())
+    # the automatic choice and the wrappers of the weight gradient land on the same bits
+    expected = torch.empty((rows, feats), dtype=torch.bfloat16, device=DEV)
+    native.gemm_strided(dy.t().contiguous(), x.t().contiguous().t(), expected, config=reference)
+    auto = torch.empty_like(expected)
+    native.gemm_strided(dy.t(), x, auto)
+    assert _same_bits(auto, expected)
+    assert _same_bits(native.det_gemm_db_transposed(x, dy), expected)
+
+
 def test_a_remainder_of_tokens_launched_on_its_own_changes_no_bit(gemm):
     """513 tokens against 32768 features: the three token rows of 256 x 256 tiles would be 384 tiles, a round and
     a half; the automatic choice launches the last token separately on the few-token kernel. Rows are
