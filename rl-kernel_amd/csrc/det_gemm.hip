@@ -86,6 +86,51 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
   if constexpr (loop_weight_kmajor(LOOP)) {
     // No run permutation on this path: MFMA tile jn holds features jn*16 + (lane>>4)*4 + q.
     const int n_tile = n0 + wave_n * 16 * S::TN + (lane >> 4) * 4;
+    if constexpr (!OUT_F32 && S::TN == 4) {
+      // bf16 results of a wave whose 64 features all lie inside N, rows 16-byte aligned (both uniform over the
+      // wave): a lane holds four 8-byte pieces of a token's row, 32 bytes apart. A 4 x 4 transpose of the pieces
+      // between the four lanes of a token (two butterfly stages of lane swaps over distances 32 and 16: the
+      // piece that lane g held at position c ends at lane c, position g) gives every lane the 16 consecutive
+      // features 16 g .. 16 g + 15, stored as two 16-byte halves: 128 contiguous bytes per token and instruction
+      // pair instead of 32 per instruction.
+      const int n_wave = n0 + wave_n * 64;
+      const bool whole_span = n_wave + 64 <= N && (reinterpret_cast<uintptr_t>(C) & 15) == 0 && (ldc & 7) == 0;
+      if (whole_span) {
+        const int grp = lane >> 4;
+#pragma unroll
+        for (int jm = 0; jm < S::TM; ++jm) {
+          uint32_t w[4][2];
+#pragma unroll
+          for (int jn = 0; jn < 4; ++jn) {
+            w[jn][0] = pack_bf16x2(acc[jn][jm][0], acc[jn][jm][1]);
+            w[jn][1] = pack_bf16x2(acc[jn][jm][2], acc[jn][jm][3]);
+          }
+#pragma unroll
+          for (int c = 0; c < 2; ++c)  // lane bit 5 <-> piece bit 1
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+              const auto r = __builtin_amdgcn_permlane32_swap(w[c][e], w[c + 2][e], false, false);
+              w[c][e] = r[0];
+              w[c + 2][e] = r[1];
+            }
+#pragma unroll
+          for (int c = 0; c < 4; c += 2)  // lane bit 4 <-> piece bit 0
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+              const auto r = __builtin_amdgcn_permlane16_swap(w[c][e], w[c + 1][e], false, false);
+              w[c][e] = r[0];
+              w[c + 1][e] = r[1];
+            }
+          const int m = m_lane + jm * 16;
+          if (m < M) {
+            bf16_bits* dst = reinterpret_cast<bf16_bits*>(C) + (int64_t)m * ldc + n_wave + grp * 16;
+            *reinterpret_cast<u32x4_t*>(dst) = u32x4_t{w[0][0], w[0][1], w[1][0], w[1][1]};
+            *reinterpret_cast<u32x4_t*>(dst + 8) = u32x4_t{w[2][0], w[2][1], w[3][0], w[3][1]};
+          }
+        }
+        return;
+      }
+    }
 #pragma unroll
     for (int jm = 0; jm < S::TM; ++jm) {
       const int m = m_lane + jm * 16;
@@ -427,8 +472,8 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
       // reduction against few output tiles, e.g. grad_hidden of the LogP backward up to about a thousand
       // tokens (N = 4096, K = 151936), a workgroup per CU: every workgroup then streams a narrow slice of the
       // weight instead of a 256-column one (1.9 -> 0.9 ms at 256 tokens, 1.8 -> 1.3 ms at 512).
-      const Shape shapes[] = {{RLK_GEMM_CFG_256x256, 256, 256, 1.00}, {RLK_GEMM_CFG_256x128, 256, 128, 0.65},
-                              {RLK_GEMM_CFG_256x64, 256, 64, 0.50},   {RLK_GEMM_CFG_128x128, 128, 128, 0.52},
+      const Shape shapes[] = {{RLK_GEMM_CFG_256x256, 256, 256, 1.00}, {RLK_GEMM_CFG_256x128, 256, 128, 0.70},
+                              {RLK_GEMM_CFG_256x64, 256, 64, 0.56},   {RLK_GEMM_CFG_128x128, 128, 128, 0.52},
                               {RLK_GEMM_CFG_128x64, 128, 64, 0.36},   {RLK_GEMM_CFG_64x64, 64, 64, 0.25}};
       double best = 1e300;
       for (const Shape& c : shapes) {

@@ -22,12 +22,9 @@ constexpr int kShortKTokens = 64;     // tokens of one streamed tile (one K-majo
 constexpr int kShortKFeatures = 256;  // features of a workgroup: 64 per wave
 constexpr int kShortKXcds = 8;
 
-// The fragments of 16-token sub-tile j of a stage. The restrict qualifiers (true: nothing writes the stage
-// while it is read) also give these reads alias scopes; the compiler waits for every direct-to-LDS load in
-// flight in front of an LDS read it knows nothing about, which would undo the prefetch.
+// The fragments of 16-token sub-tile j of a stage (KT K-major columns of 64 K rows, one per K tile).
 template <int STEPS>
-__device__ __forceinline__ void read_shortk_subtile(const char* __restrict__ stage, int j, int l16, int grp,
-                                                    u32x4_t (&__restrict__ dst)[STEPS]) {
+__device__ __forceinline__ void read_shortk_subtile(const char* stage, int j, int l16, int grp, u32x4_t (&dst)[STEPS]) {
 #pragma unroll
   for (int s = 0; s < STEPS; ++s)
     dst[s] = read_kmajor_fragment(stage + (s >> 1) * (kTileK * kRowBytes), j, s & 1, l16, grp);

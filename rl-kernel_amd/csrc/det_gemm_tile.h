@@ -133,7 +133,13 @@ __device__ __forceinline__ int kmajor_swizzle(int k_row) { return 2 * (((k_row >
 
 // The MFMA fragment of 16-row tile `j16` of a K-major column for K step `step`: ds_read_b64_tr_b16 hands lane r
 // of a 16-lane group the four K values of row r out of 4 K rows x 16 rows.
-__device__ __forceinline__ u32x4_t read_kmajor_fragment(const char* col, int j16, int step, int l16, int grp) {
+// `col` is restrict-qualified (nothing writes the column while this function reads it) for what that does to the
+// generated waits: in front of an LDS read that carries no alias information (this intrinsic, unlike a plain
+// vector load) the compiler waits for every direct-to-LDS load in flight, which made a wave that prefetches the
+// next stage wait for it before reading the current one. With the qualifier the reads carry an alias scope and
+// only the hand-placed waits of the loops remain, as for the native layout.
+__device__ __forceinline__ u32x4_t read_kmajor_fragment(const char* __restrict__ col, int j16, int step, int l16,
+                                                        int grp) {
   typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
   typedef __attribute__((address_space(3))) bf16x4_t* lds_bf16x4_ptr_t;
   u32x2_t half[2];
