@@ -165,6 +165,42 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
     return;
   }
 
+  if constexpr (!OUT_F32 && S::TN == 4) {
+    // bf16 results of a wave whose 64 features all lie inside N, rows 16-byte aligned (both uniform over the wave):
+    // a lane holds the 16 consecutive features 16 g .. 16 g + 15 of a token as two 16-byte halves, so a store
+    // instruction would write 16-byte pieces 32 bytes apart. Two lane swaps (over distance 16 between the halves,
+    // then over distance 32) rotate (half, lane bit 5, lane bit 4) into (lane bit 4, half, lane bit 5): store s of
+    // lane g then holds features 32 s + 8 g .. + 7, 64 contiguous bytes per token and instruction.
+    const int n_wave = n0 + wave_n * 64;
+    const bool whole_span = n_wave + 64 <= N && (reinterpret_cast<uintptr_t>(C) & 15) == 0 && (ldc & 7) == 0;
+    if (whole_span) {
+      const int grp = lane >> 4;
+#pragma unroll
+      for (int jm = 0; jm < S::TM; ++jm) {
+        uint32_t half[2][4];
+#pragma unroll
+        for (int jn = 0; jn < 4; ++jn) {
+          half[jn >> 1][2 * (jn & 1)] = pack_bf16x2(acc[jn][jm][0], acc[jn][jm][1]);
+          half[jn >> 1][2 * (jn & 1) + 1] = pack_bf16x2(acc[jn][jm][2], acc[jn][jm][3]);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const auto r = __builtin_amdgcn_permlane16_swap(half[0][e], half[1][e], false, false);
+          const auto t = __builtin_amdgcn_permlane32_swap(r[0], r[1], false, false);
+          half[0][e] = t[0];
+          half[1][e] = t[1];
+        }
+        const int m = m_lane + jm * 16;
+        if (m < M) {
+          bf16_bits* dst = reinterpret_cast<bf16_bits*>(C) + (int64_t)m * ldc + n_wave + grp * 8;
+          *reinterpret_cast<u32x4_t*>(dst) = u32x4_t{half[0][0], half[0][1], half[0][2], half[0][3]};
+          *reinterpret_cast<u32x4_t*>(dst + 32) = u32x4_t{half[1][0], half[1][1], half[1][2], half[1][3]};
+        }
+      }
+      return;
+    }
+  }
+
 #pragma unroll
   for (int jm = 0; jm < S::TM; ++jm) {
     const int m = m_lane + jm * 16;
