@@ -77,7 +77,7 @@ def _parse():
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-T table")
     ap.add_argument("--rotate-weights", action="store_true",
                     help="gate_up_tN / down_tN legs: launch over copies of the weight (~1.3 GB in rotation) so that it is read from HBM")
-    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|gate_up_tN|down_tN|logp|logp_decode|logp_mid|logp_logits|logp_bwd|logp_bwd_256|from_logits|from_logits_bwd|ffn|tree|tree_down|tree_decode|copy|power (used for profiling)")
+    ap.add_argument("--only", default="", help="run a single leg and print its JSON: gate_up|down|gate_up_tN|down_tN|logp|logp_decode|logp_mid|logp_logits|logp_bwd|logp_bwd_256|from_logits|from_logits_bwd|ffn|tree|tree_down|tree_decode|copy|power|host (used for profiling)")
     return ap.parse_args()
 
 
@@ -170,6 +170,47 @@ def main() -> int:
         gate_up()
         down()
 
+    if args.only == "host":
+        # Eager host cost per call of the Python entry points (facade -> ctypes -> launch) on tiny operands:
+        # `steps` calls are queued without waiting for the GPU and the wall clock is divided by their number;
+        # torch.matmul on the same operands is there for scale.
+        import time
+
+        from rl_engine import _C
+        from rl_engine.ops.ffn import qwen3_ffn_packed_inference
+        from rl_engine.ops.gemm import deterministic_gemm
+        from rl_engine.ops.gemm.det_gemm import det_gemm_linear
+        from rl_engine.ops.logprob import deterministic_linear_logp
+
+        x1, w_s = randn(1, 512), randn(512, 512, 0.02)
+        b_s = w_s.t().contiguous()
+        out_s = torch.empty((1, 512), dtype=torch.bfloat16, device=dev)
+        h4, w_v = randn(4, 512), randn(4096, 512, 0.02)
+        t4 = torch.randint(0, 4096, (4,), device=dev)
+        w_gu_s, w_d_s = randn(2 * 1024, 512, 0.02), randn(512, 1024, 0.02)
+        calls = {
+            "torch.matmul": lambda: torch.matmul(x1, b_s),
+            "_C.gemm_strided(out=)": lambda: _C.gemm_strided(x1, b_s, out_s),
+            "_C.det_gemm_fwd": lambda: _C.det_gemm_fwd(x1, b_s),
+            "deterministic_gemm": lambda: deterministic_gemm(x1, b_s),
+            "det_gemm_linear": lambda: det_gemm_linear(x1, w_s),
+            "_C.fused_linear_logp": lambda: _C.fused_linear_logp(h4, w_v, t4),
+            "deterministic_linear_logp": lambda: deterministic_linear_logp(h4, w_v, t4),
+            "qwen3_ffn_packed_inference": lambda: qwen3_ffn_packed_inference(x1, w_gu_s, w_d_s),
+        }
+        n = max(args.steps, 1000)
+        result = {}
+        for name, fn in calls.items():
+            for _ in range(50):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                fn()
+            result[name] = round((time.perf_counter() - t0) / n * 1e6, 1)
+            torch.cuda.synchronize()
+        print(json.dumps({"leg": "host", "calls": n, "us_per_call": result}))
+        return 0
     if args.only == "copy":
         # Calibration leg for the FETCH_SIZE / WRITE_SIZE counters: one plain device
         # copy kernel of known size (1 GiB read + 1 GiB written per launch).
