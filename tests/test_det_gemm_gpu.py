@@ -432,6 +432,31 @@ def test_short_reduction_streaming_kernel_keeps_the_bits(native, tokens, rows, f
     assert _same_bits(native.det_gemm_db_transposed(x, dy), expected)
 
 
+@pytest.mark.parametrize("tokens,rows,feats", ((128, 24576, 4096), (256, 24648, 4136), (64, 40000, 1024), (192, 16392, 520)))
+def test_short_reduction_kernel_over_many_token_tiles_per_workgroup(native, tokens, rows, feats):
+    """Shapes that give a workgroup of the streaming kernel 6 ... 40 token tiles, so the ring wraps and the
+    counted waits reach their steady state: whole chunks (every store a whole line, loads counted past the
+    stores), a result with a partial last token tile and a partial last feature block (guarded stores,
+    conservative waits), and the automatic choice (which takes this kernel at these sizes) against a forced tile
+    kernel."""
+    from rl_engine import _lib
+
+    dy = inputs.randn_bf16(93, tokens, rows, 0.05).to(DEV)
+    x = inputs.randn_bf16(94, tokens, feats).to(DEV)
+    expected = torch.empty((rows, feats), dtype=torch.bfloat16, device=DEV)
+    native.gemm_strided(dy.t(), x, expected, config=_lib.GEMM_CONFIGS["256x256"])
+    for config in ("shortk", "auto"):
+        got = torch.full((rows, feats), 7.0, dtype=torch.bfloat16, device=DEV)
+        native.gemm_strided(dy.t(), x, got, config=_lib.GEMM_CONFIGS[config])
+        assert _same_bits(got, expected), config
+    got32 = torch.empty((rows, feats), dtype=torch.float32, device=DEV)
+    want32 = torch.empty((rows, feats), dtype=torch.float32, device=DEV)
+    native.gemm_strided(dy.t(), x, got32, config=_lib.GEMM_CONFIGS["shortk"])
+    native.gemm_strided(dy.t(), x, want32, config=_lib.GEMM_CONFIGS["256x256"])
+    assert torch.equal(got32.view(torch.int32), want32.view(torch.int32))
+    assert _same_bits(got32.to(torch.bfloat16), expected)
+
+
 def test_a_remainder_of_tokens_launched_on_its_own_changes_no_bit(gemm):
     """513 tokens against 32768 features: the three token rows of 256 x 256 tiles would be 384 tiles, a round and
     a half; the automatic choice launches the last token separately on the few-token kernel. Rows are
