@@ -6,9 +6,9 @@
 // per tile outside the K loop there (first loads, epilogue, workgroup turnover: 11 of 18 us for a
 // 256 x 256 tile with four K tiles), and nothing overlaps those phases. Here a workgroup keeps the
 // feature operand of 256 output columns in registers for the whole reduction (64 features x K per wave,
-// gathered once), and streams the token operand through a two-stage LDS ring, 64 tokens at a time: the loads
-// of the next two tiles are in flight while a tile is multiplied and stored, and no phase waits for a
-// workgroup to start. Same instruction, same ascending 32-wide K steps from a zero accumulator as every
+// gathered once), and streams the token operand through a ring of NS LDS stages (two; deeper rings measured the
+// same), 64 tokens at a time: the loads of the following tile are in flight while a tile is multiplied and
+// stored, and no phase waits for a workgroup to start. Same instruction, same ascending 32-wide K steps from a zero accumulator as every
 // other det_gemm kernel, so the bits are the same.
 //
 // The token operand must be K-major (x[k * ld + m], tokens contiguous, as the transposed operand of a weight
@@ -33,9 +33,11 @@ __device__ __forceinline__ void read_shortk_subtile(const char* stage, int j, in
 // KT = K / 64. Workgroup id -> (feature block, chunk of token tiles) such that the feature blocks of one chunk
 // run on one XCD at the same time: they read the same token tiles, one from the fabric and the rest from L2.
 template <int KT, bool OUT_F32, int NS>
-__global__ __launch_bounds__(256, (NS * KT > 8 ? 1 : 2)) void det_gemm_shortk_kernel(MatView W, MatView X, void* __restrict__ C,
-                                                               int64_t ldc, int M, int N, int n_blocks,
-                                                               int tiles_per_chunk, int vec_store) {
+__global__ __launch_bounds__(256, (NS * KT > 8 ? 1 : 2)) void det_gemm_shortk_kernel(MatView W, MatView X,
+                                                                                      void* __restrict__ C, int64_t ldc,
+                                                                                      int M, int N, int n_blocks,
+                                                                                      int tiles_per_chunk,
+                                                                                      int vec_store) {
   constexpr int kSteps = 2 * KT;                         // MFMA steps of the reduction
   constexpr int kStageBytes = KT * kTileK * kRowBytes;   // 64 tokens x K
   constexpr int kLoads = 2 * KT;                         // 1 KiB blocks per wave and stage
