@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256, (NS * KT > 8 ? 1 : 2)) void det_gemm_shortk_ke
   // Token tile t -> a stage: K tile kt is a K-major column (64 K rows of 128 bytes, the layout of
   // read_kmajor_fragment); a block is 8 K rows, lane -> (K row lane >> 3, chunk position lane & 7).
   const int rib = lane >> 3;
-  const int kmajor_chunk = (lane & 7) ^ (2 * ((rib >> 1) & 1));
+  const int kmajor_chunk = (lane & 7) ^ kmajor_swizzle_of_row_in_block(rib);
   const int64_t ldk = X.k_stride;
   auto issue = [&](int t, char* stage) {
     const int m0 = t * kShortKTokens;
@@ -104,7 +104,7 @@ __global__ __launch_bounds__(256, (NS * KT > 8 ? 1 : 2)) void det_gemm_shortk_ke
       const int b = wave * kLoads + j;
       const int kt = b >> 3;
       const int kblk = b & 7;
-      int at = (kmajor_chunk ^ (2 * (kblk & 3))) * kChunkElems;
+      int at = (kmajor_chunk ^ kmajor_swizzle_of_block(kblk)) * kChunkElems;
       at = at < last ? at : last;
       const bf16_bits* src = X.ptr + (int64_t)(kt * kTileK + kblk * 8 + rib) * ldk + m0 + at;
       __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + b * 1024), 16, 0, 0);

@@ -128,8 +128,20 @@ struct Stager {
 
 // Swizzle of the 16-byte chunk position inside a K row of a K-major stage (a 64-wide column of 64 K rows
 // of 128 bytes): keeps both the 16-byte stores / direct loads and the transposing fragment reads free of
-// bank conflicts.
-__device__ __forceinline__ int kmajor_swizzle(int k_row) { return 2 * (((k_row >> 1) & 1) ^ ((k_row >> 3) & 3)); }
+// bank conflicts. A transposing read takes 8 bytes per lane; of a fragment's lanes, lane group g reads K rows
+// 8 g + 4 h + a (a = 0..3) and, in a row, the 32 bytes of its MFMA tile. The bank of a lane's 8 bytes is
+// 32 (k & 1) + 4 chunk + 2 (lane & 1), so the 32 lanes the LDS serves together must differ in (k & 1, chunk): bit 2
+// of the chunk position takes bit 1 of the K row and bit 1 takes the parity of the lane group, whichever two
+// groups share a pass (0-1 / 2-3 or 0-2 / 1-3). (A swizzle that told apart only groups 0-2 / 1-3 measured one
+// conflict cycle per read: SQ_LDS_BANK_CONFLICT equal to a third of the LDS-busy cycles with a K-major weight and
+// to half of them with both operands K-major.)
+__device__ __forceinline__ int kmajor_swizzle(int k_row) {
+  return 4 * ((k_row >> 1) & 1) + 2 * (((k_row >> 3) ^ (k_row >> 4)) & 1);
+}
+// The same for the direct-to-LDS loads, which move blocks of 8 K rows (K row 8 kblk + rib of a tile): the part of
+// the swizzle that depends on the lane's K row inside a block, and the part that depends on the block.
+__device__ __forceinline__ int kmajor_swizzle_of_row_in_block(int rib) { return 4 * ((rib >> 1) & 1); }
+__device__ __forceinline__ int kmajor_swizzle_of_block(int kblk) { return 2 * ((kblk ^ (kblk >> 1)) & 1); }
 
 // The MFMA fragment of 16-row tile `j16` of a K-major column for K step `step`: ds_read_b64_tr_b16 hands lane r
 // of a 16-lane group the four K values of row r out of 4 K rows x 16 rows.
@@ -603,7 +615,7 @@ struct DmaLoader {
     chunk_elems = ((lane & 7) ^ rib) * kChunkElems;
     // K-major: lane -> (K row rib of the block, chunk position lane & 7); the K-row part
     // of the swizzle that does not depend on the block is folded in here.
-    kmajor_chunk = (lane & 7) ^ (2 * ((rib >> 1) & 1));
+    kmajor_chunk = (lane & 7) ^ kmajor_swizzle_of_row_in_block(rib);
     if (WK) {
       w_lane_off[0] = (uint32_t)(rib * ldw);
       w_lane_off[1] = 0;
@@ -620,7 +632,7 @@ struct DmaLoader {
                                                                 int b) {
     const int col = b >> 3;  // 64-wide column of the tile
     const int kblk = b & 7;  // K rows 8 kblk .. 8 kblk + 7 of the tile
-    const int chunk = kmajor_chunk ^ (2 * (kblk & 3));
+    const int chunk = kmajor_chunk ^ kmajor_swizzle_of_block(kblk);
     int at = col * 64 + chunk * kChunkElems;  // offset inside the tile along the contiguous axis
     if (first + col * 64 + 64 > rows) {       // column crosses the edge (rows % 8 == 0 here)
       const int last = rows - kChunkElems - first;

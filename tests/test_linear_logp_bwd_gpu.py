@@ -115,6 +115,10 @@ def _assert_grad_parity(oracle, c, lse, grads, *, g_lse=True):
         ((40, 3000, 264), dict(bias=True)),  # D % 64 != 0 and V % 64 != 0: staged / element loaders
         ((130, 5000, 512), dict(temperature=True)),  # T % 64 != 0: weight gradient on the element loader
         ((256, 4096, 320), dict(bias=True, temperature=True, real=4000)),
+        # from 512 tokens on (T % 8 == 0) the weight gradient reads the hidden states from a transposed copy
+        # that is staged in the grad_hidden buffer: T % 64 != 0 with D % 64 != 0, and whole tiles
+        ((520, 2048, 264), dict(bias=True)),
+        ((1024, 3000, 256), dict(bias=True, temperature=True, real=2900)),
     ],
 )
 def test_backward_parity_with_oracle(native, oracle, shape, opts):
@@ -132,17 +136,20 @@ def test_backward_parity_with_oracle(native, oracle, shape, opts):
 def test_backward_is_bitwise_deterministic_and_config_neutral(native):
     from rl_engine import _lib
 
-    c = _case(320, 3072, 256, 5200, bias=True, temperature=True, real=3000)
-    _, base = _gpu_backward(native, c)
-    for _ in range(3):
-        _, again = _gpu_backward(native, c)
-        for x, y in zip(base, again):
-            assert torch.equal(x.view(torch.uint8), y.view(torch.uint8))
-    for name, value in _lib.LOGP_CONFIGS.items():
-        for flag in (0, _lib.FORCE_STAGED):
-            _, other = _gpu_backward(native, c, config=value | flag)
-            for x, y in zip(base, other):
-                assert torch.equal(x.view(torch.uint8), y.view(torch.uint8)), (name, flag)
+    # the second case is large enough for the transposed-hidden form of the weight gradient, which the
+    # register-staged configurations do not take
+    for shape in ((320, 3072, 256), (576, 2048, 328)):
+        c = _case(*shape, 5200, bias=True, temperature=True, real=shape[1] - 72)
+        _, base = _gpu_backward(native, c)
+        for _ in range(3):
+            _, again = _gpu_backward(native, c)
+            for x, y in zip(base, again):
+                assert torch.equal(x.view(torch.uint8), y.view(torch.uint8))
+        for name, value in _lib.LOGP_CONFIGS.items():
+            for flag in (0, _lib.FORCE_STAGED):
+                _, other = _gpu_backward(native, c, config=value | flag)
+                for x, y in zip(base, other):
+                    assert torch.equal(x.view(torch.uint8), y.view(torch.uint8)), (shape, name, flag)
 
 
 def test_grad_hidden_rows_are_batch_invariant(native):
