@@ -577,10 +577,13 @@ struct DmaLoader {
   static_assert(!WK || S::TN == 4, "K-major weights need 64-feature wave columns");
   static_assert(!XK || S::BM % 128 == 0, "K-major activations need whole 64-token columns per wave group");
   static constexpr int kWBlocksPerWave = kWaveRows / 8;     // blocks of one weight column
-  // Native layout: the two waves that read a weight column split its refill. K-major operands
-  // (twice as many, transposing, fragment reads per phase) measured faster with the whole column
-  // refilled by the late wave after all of its reads.
-  static constexpr bool kSplitColumn = !WK && !XK;
+  // The two waves that read a weight column split its refill: always for the native layout, and for K-major
+  // operands on the 256-token tile (4-6 % there: lm_head weight gradient at 8192 tokens 8.32 -> 7.77 ms; that had
+  // measured slower while the transposing reads still had bank conflicts and the compiler's waits in front of them).
+  // The K-major tiles of 128 and 64 tokens run where the weight stream bounds the time, and the half of a column
+  // that the early wave refills starts one phase later: with the split they measured 16-20 % slower (12288 x 4096 at
+  // 1024 tokens, 256 x 64: 137 -> 160 us), so there the late wave refills the whole column after its reads.
+  static constexpr bool kSplitColumn = (!WK && !XK) || S::BM >= 256;
   static constexpr int kWBlocksLate = kSplitColumn ? kWBlocksPerWave / 2 : kWBlocksPerWave;
   static constexpr int kWBlocksEarly = kWBlocksPerWave - kWBlocksLate;
   static constexpr int kXBlocksPerWave = (S::BM / 16) / 4;  // every wave
@@ -888,14 +891,15 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
     wg_barrier();  // half an iteration behind the early group
     // LDS reads return in order, so once at most kXReads of them are outstanding the weight
     // fragments (issued first) are in registers and their rows may be refilled.
-    // (lgkmcnt is a 4-bit counter, so this needs at most 15 token reads per K step.)
+    // (lgkmcnt is a 4-bit counter: with the 16 reads of eight K-major token tiles the wait for 15 also covers the
+    // first of them; more reads per K step, i.e. several K tiles per stage, take the other order.)
     constexpr int kXReads = KS * S::TM * (XK ? 2 : 1);
     for (int t = 0; t < nk; ++t) {
-      if constexpr (Loader::kSplitColumn && kXReads <= 15) {
+      if constexpr (Loader::kSplitColumn && kXReads <= 16) {
         issue_late_x(stage(t), tile_k(t + NS));  // token rows the early group read one phase ago
         read_w(t);
         read_x(t, 0);
-        __builtin_amdgcn_s_waitcnt(wait_lgkmcnt(kXReads));  // my weight fragments are in registers
+        __builtin_amdgcn_s_waitcnt(wait_lgkmcnt(kXReads < 15 ? kXReads : 15));  // my weight fragments are in registers
         issue_late_w(stage(t), tile_k(t + NS));
         read_x(t, 1);
       } else {
