@@ -174,8 +174,6 @@ def main() -> int:
         # Eager host cost per call of the Python entry points (facade -> ctypes -> launch) on tiny operands:
         # `steps` calls are queued without waiting for the GPU and the wall clock is divided by their number;
         # torch.matmul on the same operands is there for scale.
-        import time
-
         from rl_engine import _C
         from rl_engine.ops.ffn import qwen3_ffn_packed_inference
         from rl_engine.ops.gemm import deterministic_gemm

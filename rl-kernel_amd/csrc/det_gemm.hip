@@ -93,9 +93,10 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
       // piece that lane g held at position c ends at lane c, position g) gives every lane the 16 consecutive
       // features 16 g .. 16 g + 15, stored as two 16-byte halves: 128 contiguous bytes per token and instruction
       // pair instead of 32 per instruction.
-      // The stores are non-temporal: the result is not read again here, and ordinary stores push operand panels
-      // that later tiles share out of the L2 (measured with both forms built side by side on one machine:
-      // gate_up at 4096 / 2048 tokens 574 -> 550 / 299 -> 284 us, the smaller results within 1 %).
+      // Ordinary stores. Non-temporal ones make a GEMM that is relaunched on the same operands 4-5 % faster (gate_up
+      // at 4096 tokens 574 -> 550 us): the result then bypasses the 256 MB memory-side cache and the weights stay in
+      // it from one launch to the next. With weights that come from HBM, as in a model with more than one layer,
+      // they measured the same or 1 % slower, and gate_up and down launched alternately 0.6 % slower; not used.
       const int n_wave = n0 + wave_n * 64;
       const bool whole_span = n_wave + 64 <= N && (reinterpret_cast<uintptr_t>(C) & 15) == 0 && (ldc & 7) == 0;
       if (whole_span) {
@@ -127,8 +128,8 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
           const int m = m_lane + jm * 16;
           if (m < M) {
             bf16_bits* dst = reinterpret_cast<bf16_bits*>(C) + (int64_t)m * ldc + n_wave + grp * 16;
-            __builtin_nontemporal_store(u32x4_t{w[0][0], w[0][1], w[1][0], w[1][1]}, reinterpret_cast<u32x4_t*>(dst));
-            __builtin_nontemporal_store(u32x4_t{w[2][0], w[2][1], w[3][0], w[3][1]}, reinterpret_cast<u32x4_t*>(dst + 8));
+            *reinterpret_cast<u32x4_t*>(dst) = u32x4_t{w[0][0], w[0][1], w[1][0], w[1][1]};
+            *reinterpret_cast<u32x4_t*>(dst + 8) = u32x4_t{w[2][0], w[2][1], w[3][0], w[3][1]};
           }
         }
         return;
@@ -173,8 +174,7 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
     // a lane holds the 16 consecutive features 16 g .. 16 g + 15 of a token as two 16-byte halves, so a store
     // instruction would write 16-byte pieces 32 bytes apart. Two lane swaps (over distance 16 between the halves,
     // then over distance 32) rotate (half, lane bit 5, lane bit 4) into (lane bit 4, half, lane bit 5): store s of
-    // lane g then holds features 32 s + 8 g .. + 7, 64 contiguous bytes per token and instruction. Non-temporal
-    // stores, as above.
+    // lane g then holds features 32 s + 8 g .. + 7, 64 contiguous bytes per token and instruction.
     const int n_wave = n0 + wave_n * 64;
     const bool whole_span = n_wave + 64 <= N && (reinterpret_cast<uintptr_t>(C) & 15) == 0 && (ldc & 7) == 0;
     if (whole_span) {
@@ -197,8 +197,8 @@ __global__ __launch_bounds__(S::kThreads) void det_gemm_kernel(MatView W, MatVie
         const int m = m_lane + jm * 16;
         if (m < M) {
           bf16_bits* dst = reinterpret_cast<bf16_bits*>(C) + (int64_t)m * ldc + n_wave + grp * 8;
-          __builtin_nontemporal_store(u32x4_t{half[0][0], half[0][1], half[0][2], half[0][3]}, reinterpret_cast<u32x4_t*>(dst));
-          __builtin_nontemporal_store(u32x4_t{half[1][0], half[1][1], half[1][2], half[1][3]}, reinterpret_cast<u32x4_t*>(dst + 32));
+          *reinterpret_cast<u32x4_t*>(dst) = u32x4_t{half[0][0], half[0][1], half[0][2], half[0][3]};
+          *reinterpret_cast<u32x4_t*>(dst + 32) = u32x4_t{half[1][0], half[1][1], half[1][2], half[1][3]};
         }
       }
       return;
