@@ -892,10 +892,13 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
     // LDS reads return in order, so once at most kXReads of them are outstanding the weight
     // fragments (issued first) are in registers and their rows may be refilled.
     // (lgkmcnt is a 4-bit counter: with the 16 reads of eight K-major token tiles the wait for 15 also covers the
-    // first of them; more reads per K step, i.e. several K tiles per stage, take the other order.)
+    // first of them; more reads per K step, i.e. several K tiles per stage, take the other order.) The order holds
+    // whether the column's refill is split or not: the early wave of the column read it one phase earlier. On the
+    // 128- and 64-token K-major tiles, which do not split, it is worth 1-7 % (12288 x 4096 at 2048 tokens, 256 x 128:
+    // 181 -> 168 us).
     constexpr int kXReads = KS * S::TM * (XK ? 2 : 1);
     for (int t = 0; t < nk; ++t) {
-      if constexpr (Loader::kSplitColumn && kXReads <= 16) {
+      if constexpr (kXReads <= 16) {
         issue_late_x(stage(t), tile_k(t + NS));  // token rows the early group read one phase ago
         read_w(t);
         read_x(t, 0);
