@@ -577,13 +577,16 @@ struct DmaLoader {
   static_assert(!WK || S::TN == 4, "K-major weights need 64-feature wave columns");
   static_assert(!XK || S::BM % 128 == 0, "K-major activations need whole 64-token columns per wave group");
   static constexpr int kWBlocksPerWave = kWaveRows / 8;     // blocks of one weight column
-  // The two waves that read a weight column split its refill: always for the native layout, and for K-major
-  // operands on the 256-token tile (4-6 % there: lm_head weight gradient at 8192 tokens 8.32 -> 7.77 ms; that had
-  // measured slower while the transposing reads still had bank conflicts and the compiler's waits in front of them).
-  // The K-major tiles of 128 and 64 tokens run where the weight stream bounds the time, and the half of a column
-  // that the early wave refills starts one phase later: with the split they measured 16-20 % slower (12288 x 4096 at
-  // 1024 tokens, 256 x 64: 137 -> 160 us), so there the late wave refills the whole column after its reads.
-  static constexpr bool kSplitColumn = (!WK && !XK) || S::BM >= 256;
+  // Who refills a weight column. On the 256-token tiles, which are bound by the matrix pipe, its two waves split the
+  // refill (native loop: MFMA utilisation 77 -> 82 %; K-major loops 4-6 %, lm_head weight gradient at 8192 tokens
+  // 8.32 -> 7.77 ms, which had measured slower while the transposing reads still had bank conflicts and the compiler's
+  // waits in front of them). The tiles of 128 and 64 tokens run where the weight stream bounds the time, and the half
+  // of a column that the early wave refills starts one phase later: there the late wave refills the whole column as
+  // soon as its weight fragments are in registers. Measured with weights from HBM, split -> whole column: the deep-stage
+  // 64 x 64 / 128 x 64 / 128 x 128 tiles 6-13 % faster (down at 256 / 1024 tokens 57.6 -> 51.4 / 116 -> 101 us), native
+  // 256 x 128 2-6 % faster, K-major 256 x 128 / 256 x 64 16-20 % faster; only the native 256 x 64 tile (three stages, one
+  // token block per wave) is 3-8 % faster with the split and keeps it.
+  static constexpr bool kSplitColumn = S::BM >= 256 || (!WK && !XK && S::BN == 256 && S::BM == 64);
   static constexpr int kWBlocksLate = kSplitColumn ? kWBlocksPerWave / 2 : kWBlocksPerWave;
   static constexpr int kWBlocksEarly = kWBlocksPerWave - kWBlocksLate;
   static constexpr int kXBlocksPerWave = (S::BM / 16) / 4;  // every wave
