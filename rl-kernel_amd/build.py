@@ -1,4 +1,4 @@
-"""Build librlk_gfx950.so (the C-ABI HIP library) in-tree with hipcc.
+"""Build librlk_gfx950.so (the C-ABI HIP library) and the load-path probe (a diagnostic executable) in-tree with hipcc.
 
 Usage: python rl-kernel_amd/build.py            (or __graft_entry__.build())
 """
@@ -15,6 +15,8 @@ PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "librlk_gfx950.so"
 OBJ_DIR = PKG_DIR / "build"  # object files (git-ignored)
+PROBE_SRC = CSRC / "probe" / "load_path_probe.hip"  # a stand-alone diagnostic, not part of the library
+PROBE_PATH = PKG_DIR / "load_path_probe"
 SOURCES = ["det_gemm.hip", "det_gemm_stream.hip", "det_gemm_shortk.hip", "det_gemm_tree.hip", "det_gemm_seq.hip", "linear_logp.hip",
     "linear_logp_bwd.hip", "logits_logp.hip", "swiglu.hip", "grpo.hip", "rlk_api.hip"]
 
@@ -77,6 +79,11 @@ def build(verbose: bool = True, only: list[str] | None = None) -> Path:
     if verbose:
         print("[rlk build]", " ".join(link), flush=True)
     outs.append(_run(link))
+    if only is None or PROBE_SRC.name in only:
+        probe = [hipcc, *[f for f in compile_flags if f != "-fPIC"], "-o", str(PROBE_PATH), str(PROBE_SRC)]
+        if verbose:
+            print("[rlk build]", " ".join(probe), flush=True)
+        outs.append(_run(probe))
     if verbose:
         for out in outs:
             if out:

@@ -1,0 +1,227 @@
+// Load-path probe for MI355X (gfx950): what the memory system delivers to the CUs, measured with kernels that
+// only load. A diagnostic, not part of librlk_gfx950.so: it prices the load side of the tile kernels
+// (det_gemm_tile.h) so that their measured times can be compared with what the hardware allows.
+//
+//   1. ceilings: bytes per second out of the L2, the memory-side cache and HBM with every CU loading
+//   2. rate of one workgroup against the bytes it keeps in flight (few workgroups: nothing else is busy)
+//   3. the load side of a small-tile GEMM without its arithmetic: npanels weight panels, each read at the same
+//      pace by the workgroups of its token tiles (all on one XCD), plus the token rows, which stay in the L2
+//
+// Loads are the direct-to-LDS DMA form the tile kernels use (or ordinary vector loads, "vgpr"). Build:
+//   hipcc --offload-arch=gfx950 -O3 -o load_path_probe load_path_probe.hip     (rl-kernel_amd/build.py does it)
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* global_ptr_t;
+
+#define CK(x)                                                                 \
+  do {                                                                        \
+    hipError_t e_ = (x);                                                      \
+    if (e_ != hipSuccess) {                                                   \
+      printf("HIP error %s at line %d\n", hipGetErrorString(e_), __LINE__);   \
+      exit(1);                                                                \
+    }                                                                         \
+  } while (0)
+
+static void require(bool ok, const char* what) {
+  if (!ok) {
+    printf("refused: %s\n", what);
+    exit(1);
+  }
+}
+
+constexpr int kWaitAllVm = 0x0f70;  // s_waitcnt vmcnt(0); low four bits = loads allowed to stay in flight
+
+// ---- 1 and 2: streams ------------------------------------------------------------------------------------
+// Workgroup w reads stream w % nstreams, `steps` steps of NW * U KiB, wrapping inside the stream; each wave
+// issues U loads of 1 KiB per step and waits until the previous step's loads have landed (2U in flight).
+template <int MODE, int NW, int U>
+__global__ __launch_bounds__(NW * 64) void stream_kernel(const char* base, size_t stream_bytes, int nstreams,
+                                                          int steps, unsigned* sink) {
+  extern __shared__ __align__(1024) char lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wg = blockIdx.x;
+  const size_t step_bytes = (size_t)NW * U * 1024;
+  const size_t steps_in_stream = stream_bytes / step_bytes;
+  const char* stream = base + (size_t)(wg % nstreams) * stream_bytes;
+  size_t pos = ((size_t)(wg / nstreams) * 7) % steps_in_stream;  // readers of one stream start apart
+  unsigned acc = 0;
+  if constexpr (MODE == 0) {
+    char* mine = lds + wave * (2 * U * 1024);
+    for (int s = 0; s < steps; ++s) {
+      const char* src = stream + pos * step_bytes + (size_t)wave * U * 1024 + lane * 16;
+      char* dst = mine + (s & 1) * (U * 1024);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(src + u * 1024), (lds_ptr_t)(dst + u * 1024), 16, 0, 0);
+      __builtin_amdgcn_s_waitcnt(kWaitAllVm | U);
+      if (++pos == steps_in_stream) pos = 0;
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitAllVm);
+    __syncthreads();
+    acc = *(unsigned*)(lds + threadIdx.x * 4);
+  } else {
+    uint4 v[U];
+    for (int s = 0; s < steps; ++s) {
+      const char* src = stream + pos * step_bytes + (size_t)wave * U * 1024 + lane * 16;
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = *(const uint4*)(src + u * 1024);
+#pragma unroll
+      for (int u = 0; u < U; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+      if (++pos == steps_in_stream) pos = 0;
+    }
+  }
+  if (acc == 0x12345678u) sink[0] = acc;  // never true for the 0x01 fill; keeps the loads alive
+}
+
+static size_t g_buffer_bytes = 0;
+
+template <int MODE, int NW, int U>
+static void run_streams(const char* name, const char* buf, size_t stream_bytes, int nstreams, int nwg, int steps,
+                        unsigned* sink) {
+  static_assert(U <= 8 && NW * 2 * U * 1024 <= 128 * 1024, "LDS ring of a workgroup");
+  require((size_t)nstreams * stream_bytes <= g_buffer_bytes, "streams exceed the buffer");
+  require(stream_bytes % ((size_t)NW * U * 1024) == 0 && stream_bytes >= (size_t)NW * U * 1024, "stream size");
+  const size_t lds = MODE == 0 ? (size_t)NW * 2 * U * 1024 : 0;
+  CK(hipFuncSetAttribute((const void*)stream_kernel<MODE, NW, U>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipEvent_t a, b;
+  CK(hipEventCreate(&a));
+  CK(hipEventCreate(&b));
+  for (int i = 0; i < 2; ++i) stream_kernel<MODE, NW, U><<<nwg, NW * 64, lds>>>(buf, stream_bytes, nstreams, steps, sink);
+  CK(hipEventRecord(a));
+  const int reps = 5;
+  for (int i = 0; i < reps; ++i) stream_kernel<MODE, NW, U><<<nwg, NW * 64, lds>>>(buf, stream_bytes, nstreams, steps, sink);
+  CK(hipEventRecord(b));
+  CK(hipEventSynchronize(b));
+  float ms;
+  CK(hipEventElapsedTime(&ms, a, b));
+  ms /= reps;
+  const double bytes = (double)nwg * steps * NW * U * 1024;
+  printf("%-40s %s %3d KB in flight per workgroup, %4d workgroups, %4d streams x %7.2f MB: %7.1f us  %6.2f TB/s  %6.1f GB/s per workgroup\n",
+         name, MODE == 0 ? "dma " : "vgpr", NW * 2 * U, nwg, nstreams, stream_bytes / 1e6, ms * 1e3,
+         bytes / ms * 1e-9, bytes / ms * 1e-6 / nwg);
+  fflush(stdout);
+}
+
+// ---- 3: the load side of a small-tile GEMM ---------------------------------------------------------------
+// Workgroup w loads weight panel w % npanels and token tile w / npanels, 32 KiB of each per step, and waits for
+// the previous step (128 KiB in flight per workgroup, more than the tile kernels keep). Consecutive workgroup
+// ids go round the eight XCDs, so with npanels a multiple of 8 the readers of a panel share an L2.
+// PREFETCH (four token tiles only): each reader also touches its quarter of the panel's step LEAD steps ahead,
+// one dword per 128-byte line, into a spare 256 bytes of LDS - a load with no register destination.
+template <int PREFETCH, int LEAD>
+__global__ __launch_bounds__(512) void panel_kernel(const char* weights, const char* tokens, size_t panel_bytes,
+                                                    int npanels, int steps, unsigned* sink) {
+  extern __shared__ __align__(1024) char lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int panel = blockIdx.x % npanels, ttile = blockIdx.x / npanels;
+  const char* w = weights + (size_t)panel * panel_bytes;
+  const char* x = tokens + (size_t)ttile * panel_bytes;
+  char* mine = lds + wave * 16384;
+  for (int s = 0; s < steps; ++s) {
+    const char* ws = w + (size_t)s * 32768 + wave * 4096 + lane * 16;
+    const char* xs = x + (size_t)s * 32768 + wave * 4096 + lane * 16;
+    char* dst = mine + (s & 1) * 8192;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(ws + u * 1024), (lds_ptr_t)(dst + u * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(xs + u * 1024), (lds_ptr_t)(dst + 4096 + u * 1024), 16, 0, 0);
+    }
+    if (PREFETCH && wave == 0) {
+      if (s + LEAD < steps) {
+        const char* p = w + (size_t)(s + LEAD) * 32768 + ttile * 8192 + lane * 128;
+        __builtin_amdgcn_global_load_lds((global_ptr_t)p, (lds_ptr_t)(lds + 131072), 4, 0, 0);
+      }
+      __builtin_amdgcn_s_waitcnt(kWaitAllVm | 9);
+    } else {
+      __builtin_amdgcn_s_waitcnt(kWaitAllVm | 8);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(kWaitAllVm);
+  __syncthreads();
+  const unsigned acc = *(unsigned*)(lds + threadIdx.x * 4);
+  if (acc == 0x12345678u) sink[0] = acc;
+}
+
+template <int PREFETCH, int LEAD>
+static void run_panels(const char* name, const char* buf, int npanels, int token_tiles, size_t panel_bytes,
+                       int ncopies, unsigned* sink) {
+  const int steps = (int)(panel_bytes / 32768);
+  const size_t copy_bytes = (size_t)npanels * panel_bytes;
+  require(panel_bytes % 32768 == 0 && npanels % 8 == 0, "panel size / count");
+  require(!PREFETCH || token_tiles == 4, "the quarter touch needs four readers per panel");
+  require((size_t)ncopies * copy_bytes + (size_t)token_tiles * panel_bytes <= g_buffer_bytes, "panels exceed the buffer");
+  const char* tokens = buf + (size_t)ncopies * copy_bytes;
+  const int lds = 131072 + 256, nwg = npanels * token_tiles;
+  CK(hipFuncSetAttribute((const void*)panel_kernel<PREFETCH, LEAD>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+  hipEvent_t a, b;
+  CK(hipEventCreate(&a));
+  CK(hipEventCreate(&b));
+  int c = 0;
+  for (int i = 0; i < 5; ++i, c = (c + 1) % ncopies)
+    panel_kernel<PREFETCH, LEAD><<<nwg, 512, lds>>>(buf + (size_t)c * copy_bytes, tokens, panel_bytes, npanels, steps, sink);
+  CK(hipEventRecord(a));
+  const int reps = 40;
+  for (int i = 0; i < reps; ++i, c = (c + 1) % ncopies)
+    panel_kernel<PREFETCH, LEAD><<<nwg, 512, lds>>>(buf + (size_t)c * copy_bytes, tokens, panel_bytes, npanels, steps, sink);
+  CK(hipEventRecord(b));
+  CK(hipEventSynchronize(b));
+  float ms;
+  CK(hipEventElapsedTime(&ms, a, b));
+  ms /= reps;
+  printf("%-58s %3d panels x %d token tiles, weights %s: %6.1f us per launch\n", name, npanels, token_tiles,
+         ncopies == 1 ? "relaunched (memory-side cache)" : "rotating (from HBM)          ", ms * 1e3);
+  fflush(stdout);
+}
+
+int main() {
+  g_buffer_bytes = (size_t)4 << 30;
+  char* buf;
+  unsigned* sink;
+  CK(hipMalloc(&buf, g_buffer_bytes));
+  CK(hipMalloc(&sink, 4));
+  CK(hipMemset(buf, 1, g_buffer_bytes));
+  CK(hipDeviceSynchronize());
+
+  printf("== 1. ceilings, every CU loading\n");
+  run_streams<0, 8, 8>("L2: all workgroups cycle over 1 MB", buf, 1 << 20, 1, 256, 400, sink);
+  run_streams<1, 8, 8>("L2: all workgroups cycle over 1 MB", buf, 1 << 20, 1, 256, 400, sink);
+  run_streams<0, 8, 8>("memory-side cache: 128 MB cycled", buf, 1 << 19, 256, 256, 400, sink);
+  run_streams<1, 8, 8>("memory-side cache: 128 MB cycled", buf, 1 << 19, 256, 256, 400, sink);
+  run_streams<0, 8, 8>("HBM: 4 GB once, 16 MB per workgroup", buf, 16 << 20, 256, 256, 256, sink);
+  run_streams<1, 8, 8>("HBM: 4 GB once, 16 MB per workgroup", buf, 16 << 20, 256, 256, 256, sink);
+  run_streams<1, 4, 8>("HBM: 4 GB once, 2 MB per workgroup", buf, 2 << 20, 2048, 2048, 64, sink);
+
+  printf("== 2. one workgroup's rate against its bytes in flight (each streams its own 16 MB from HBM)\n");
+  for (int nwg : {32, 256}) {
+    run_streams<0, 1, 1>("HBM", buf, 16 << 20, nwg, nwg, 2048, sink);
+    run_streams<0, 1, 4>("HBM", buf, 16 << 20, nwg, nwg, 2048, sink);
+    run_streams<0, 2, 4>("HBM", buf, 16 << 20, nwg, nwg, 2048, sink);
+    run_streams<0, 4, 4>("HBM", buf, 16 << 20, nwg, nwg, 1024, sink);
+    run_streams<0, 8, 4>("HBM", buf, 16 << 20, nwg, nwg, 512, sink);
+    run_streams<0, 8, 8>("HBM", buf, 16 << 20, nwg, nwg, 256, sink);
+  }
+  for (int nwg : {8, 256}) {
+    printf("   (each workgroup cycles over its own 64 KB: L2 hits)\n");
+    run_streams<0, 1, 1>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
+    run_streams<0, 1, 4>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
+    run_streams<0, 2, 4>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
+    run_streams<0, 4, 4>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
+    run_streams<0, 8, 8>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
+  }
+
+  printf("== 3. load side of the small-tile GEMMs of the down projection (4096 features, K = 12288), no arithmetic\n");
+  for (int ncopies : {1, 14}) {
+    // 256 tokens, 64 x 64 tiles: 64 panels of 64 features (1.5 MB), four token tiles of 64 tokens (1.5 MB each)
+    run_panels<0, 0>("256 tokens, 64x64 tiles", buf, 64, 4, 3 << 19, ncopies, sink);
+    run_panels<1, 2>("256 tokens, 64x64 tiles, quarter touch 2 steps ahead", buf, 64, 4, 3 << 19, ncopies, sink);
+    run_panels<1, 6>("256 tokens, 64x64 tiles, quarter touch 6 steps ahead", buf, 64, 4, 3 << 19, ncopies, sink);
+    // 1024 tokens, 128 x 128 tiles: 32 panels of 128 features (3 MB), eight token tiles of 128 tokens (3 MB each)
+    run_panels<0, 0>("1024 tokens, 128x128 tiles", buf, 32, 8, 3 << 20, ncopies, sink);
+  }
+  return 0;
+}
