@@ -338,6 +338,13 @@ static hipError_t launch_deep(const MatView& W, const MatView& X, void* C, int64
 template <class S>
 static hipError_t launch_staged_kmajor(const MatView& W, const MatView& X, void* C, int64_t ldc, int M, int N, int K,
                                        bool out_f32, hipStream_t stream) {
+  // Whole stages of two K tiles: the direct-to-LDS ping-pong loop with a ring of as many stages as 128 KiB (144 for
+  // the 128 x 64 tile) hold.
+  constexpr int kDmaKs = 2;
+  constexpr int kDmaNs = S::kStageBytes <= 16 * 1024 ? 4 : S::kStageBytes <= 24 * 1024 ? 3 : 2;
+  if (K % (kTileK * kDmaKs) == 0 && K >= kTileK * kDmaKs * kDmaNs)
+    return out_f32 ? launch_tile<S, kLoopPingPongKMajor, true, kDmaKs, kDmaNs>(W, X, C, ldc, M, N, K, stream)
+                   : launch_tile<S, kLoopPingPongKMajor, false, kDmaKs, kDmaNs>(W, X, C, ldc, M, N, K, stream);
   constexpr int kKs = 128 * 1024 / (2 * S::kStageBytes) >= 4 ? 4 : 2;
   if (K % kTileK != 0)
     return out_f32 ? launch_tile<S, kLoopStagedKMajorTail, true, kKs, 2>(W, X, C, ldc, M, N, K, stream)
@@ -508,13 +515,14 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
         int config, bn, bm;
         double quality;
       };
-      // The 64- and 128-feature tiles (register-staged K-major weight, native activations only) give a long
+      // The 64- and 128-feature tiles (K-major weight, native activations only) give a long
       // reduction against few output tiles, e.g. grad_hidden of the LogP backward up to about a thousand
       // tokens (N = 4096, K = 151936), a workgroup per CU: every workgroup then streams a narrow slice of the
-      // weight instead of a 256-column one (1.9 -> 0.9 ms at 256 tokens, 1.8 -> 1.3 ms at 512).
+      // weight instead of a 256-column one (1.9 -> 0.8 ms at 256 tokens, 1.8 -> 1.03 ms at 512, 1.65 -> 1.45 ms
+      // at 1024). Their qualities are those of the direct-to-LDS loop (128 divides K).
       const Shape shapes[] = {{RLK_GEMM_CFG_256x256, 256, 256, 1.00}, {RLK_GEMM_CFG_256x128, 256, 128, 0.70},
-                              {RLK_GEMM_CFG_256x64, 256, 64, 0.56},   {RLK_GEMM_CFG_128x128, 128, 128, 0.52},
-                              {RLK_GEMM_CFG_128x64, 128, 64, 0.36},   {RLK_GEMM_CFG_64x64, 64, 64, 0.25}};
+                              {RLK_GEMM_CFG_256x64, 256, 64, 0.56},   {RLK_GEMM_CFG_128x128, 128, 128, 0.62},
+                              {RLK_GEMM_CFG_128x64, 128, 64, 0.40},   {RLK_GEMM_CFG_64x64, 64, 64, 0.25}};
       double best = 1e300;
       for (const Shape& c : shapes) {
         if (c.config == RLK_GEMM_CFG_256x64 && x_kmajor) continue;

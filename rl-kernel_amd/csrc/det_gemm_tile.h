@@ -574,9 +574,13 @@ template <class S, bool WK = false, bool XK = false, class Map = PlainRowMap<S>>
 struct DmaLoader {
   static_assert(!(WK && Map::kGated), "the gated row map is for the native weight layout");
   static constexpr int kWaveRows = 16 * S::TN;
-  static_assert(!WK || S::TN == 4, "K-major weights need 64-feature wave columns");
+  static_assert(!WK || S::BN % 64 == 0, "K-major weights are staged in 64-feature columns");
   static_assert(!XK || S::BM % 128 == 0, "K-major activations need whole 64-token columns per wave group");
   static constexpr int kWBlocksPerWave = kWaveRows / 8;     // blocks of one weight column
+  // A K-major weight of a tile whose waves cover fewer than 64 features each (TN < 4): the waves of several
+  // wave columns read the same 64-feature stage column, so a block has no single pair of owners and may be
+  // refilled only when every wave has read it, i.e. behind the barrier that ends the late group's read phase.
+  static constexpr bool kSharedWColumn = WK && S::TN < 4;
   // Who refills a weight column. On the 256-token tiles, which are bound by the matrix pipe, its two waves split the
   // refill (native loop: MFMA utilisation 77 -> 82 %; K-major loops 4-6 %, lm_head weight gradient at 8192 tokens
   // 8.32 -> 7.77 ms, which had measured slower while the transposing reads still had bank conflicts and the compiler's
@@ -587,6 +591,7 @@ struct DmaLoader {
   // 256 x 128 2-6 % faster, K-major 256 x 128 / 256 x 64 16-20 % faster; only the native 256 x 64 tile (three stages, one
   // token block per wave) is 3-8 % faster with the split and keeps it.
   static constexpr bool kSplitColumn = S::BM >= 256 || (!WK && !XK && S::BN == 256 && S::BM == 64);
+  static_assert(!(kSharedWColumn && kSplitColumn), "a shared stage column is refilled by the late group alone");
   static constexpr int kWBlocksLate = kSplitColumn ? kWBlocksPerWave / 2 : kWBlocksPerWave;
   static constexpr int kWBlocksEarly = kWBlocksPerWave - kWBlocksLate;
   static constexpr int kXBlocksPerWave = (S::BM / 16) / 4;  // every wave
@@ -789,7 +794,8 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
     return read_kmajor_fragment(col, j16, step, l16, grp);
   };
   auto read_w_kmajor = [&](const char* st, int jn, int step) -> u32x4_t {
-    return read_kmajor(st + wave_n * (64 * kRowBytes), jn, step);
+    const int t16 = wave_n * S::TN + jn;  // 16-feature tile of the weight tile: column t16 / 4, tile t16 % 4 of it
+    return read_kmajor(st + (t16 >> 2) * (64 * kRowBytes), t16 & 3, step);
   };
   auto read_x_kmajor = [&](const char* st, int jm, int step) -> u32x4_t {
     const int col = wave_m * (S::TM / 4) + (jm >> 2);
@@ -901,7 +907,10 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
     // 181 -> 168 us).
     constexpr int kXReads = KS * S::TM * (XK ? 2 : 1);
     for (int t = 0; t < nk; ++t) {
-      if constexpr (kXReads <= 16) {
+      if constexpr (Loader::kSharedWColumn) {
+        issue_late_x(stage(t), tile_k(t + NS));  // token rows the early group read one phase ago
+        read_tile(t);
+      } else if constexpr (kXReads <= 16) {
         issue_late_x(stage(t), tile_k(t + NS));  // token rows the early group read one phase ago
         read_w(t);
         read_x(t, 0);
@@ -915,8 +924,16 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
         issue_late_x(stage(t), tile_k(t + NS));
       }
       __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // all my fragments are in registers
-      __builtin_amdgcn_s_waitcnt(wait_vmcnt((NS - 1) * KS * Loader::kLateLoads));  // my part of tile t+1 has landed
-      wg_barrier();
+      if constexpr (Loader::kSharedWColumn) {
+        // Behind tile t + 1 this wave has started tiles t + 2 .. t + NS - 1 and the token rows of tile t + NS;
+        // the weight blocks of tile t + NS follow the barrier, when every wave has read tile t.
+        __builtin_amdgcn_s_waitcnt(wait_vmcnt((NS - 2) * KS * Loader::kLateLoads + KS * Loader::kXBlocksPerWave));
+        wg_barrier();
+        issue_late_w(stage(t), tile_k(t + NS));
+      } else {
+        __builtin_amdgcn_s_waitcnt(wait_vmcnt((NS - 1) * KS * Loader::kLateLoads));  // my part of tile t+1 has landed
+        wg_barrier();
+      }
       compute();
       wg_barrier();
     }
@@ -943,7 +960,7 @@ __device__ __forceinline__ void tile_mainloop_pingpong(const MatView& W, const M
 template <class S, bool WK, bool XK>
 __device__ __forceinline__ void tile_tail_step(const MatView& W, const MatView& X, int n0, int m0, int k0, int K,
                                                char* lds, f32x4_t (&acc)[S::TN][S::TM]) {
-  static_assert(!WK || S::TN == 4, "K-major weights need 64-feature wave columns");
+  static_assert(!WK || S::BN % 64 == 0, "K-major weights are staged in 64-feature columns");
   static_assert(!XK || S::BM % 128 == 0, "K-major activations need whole 64-token columns per wave group");
   int tid = threadIdx.x;
   asm volatile("" : "+v"(tid));
@@ -988,7 +1005,8 @@ __device__ __forceinline__ void tile_tail_step(const MatView& W, const MatView& 
 #pragma unroll
     for (int jn = 0; jn < S::TN; ++jn) {
       if constexpr (WK) {
-        wf[jn] = read_kmajor_fragment(lds + wave_n * (64 * kRowBytes), jn, s, l16, grp);
+        const int t16 = wave_n * S::TN + jn;
+        wf[jn] = read_kmajor_fragment(lds + (t16 >> 2) * (64 * kRowBytes), t16 & 3, s, l16, grp);
       } else {
         wf[jn] = *reinterpret_cast<const u32x4_t*>(lds + w_row_base + jn * 16 * kRowBytes + (frag_lo ^ (s << 6)));
       }

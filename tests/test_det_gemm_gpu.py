@@ -336,7 +336,8 @@ def test_operand_layouts_give_the_same_bits(gemm, native, shape):
 
 
 @pytest.mark.parametrize("shape", [(512, 1024, 4096), (300, 1000, 192), (1000, 2056, 320), (64, 8, 64), (7, 1024, 1024), (2048, 4096, 1024),
-                                   (520, 1024, 200), (264, 520, 1000), (16, 128, 72)])  # the last three: K % 64 != 0, a zero-filled tail tile
+                                   (520, 1024, 200), (264, 520, 1000), (16, 128, 72),  # these three: K % 64 != 0, a zero-filled tail tile
+                                   (200, 1000, 1152), (256, 2056, 640), (72, 200, 640)])  # K % 128 == 0 with feature and token edges: the small tiles' direct-to-LDS K-major loop
 def test_kmajor_weight_fast_path_gives_the_same_bits(gemm, native, shape):
     """B[K,N] with N contiguous (the `a @ b`, prepared-weight and input-gradient
     form) and token-contiguous activations are read through transposing LDS loads. Each must
@@ -348,7 +349,8 @@ def test_kmajor_weight_fast_path_gives_the_same_bits(gemm, native, shape):
     bt = inputs.randn_bf16(54, n, k, 0.02).to(DEV)  # [N,K]
     b = bt.t().contiguous()  # [K,N]
     expected = gemm.mfma_gemm(a, bt.t(), config="16x16")
-    # (128x128, 128x64 and 64x64 with a K-major weight: the register-staged K-major loop)
+    # (128x128, 128x64 and 64x64 with a K-major weight: the direct-to-LDS loop with a shared stage column when
+    # 128 divides K, else the register-staged K-major loop)
     for name in ("auto", "256x256", "256x128", "256x64", "128x128", "128x64", "64x64"):
         for _ in range(2):
             assert _same_bits(gemm.mfma_gemm(a, b, config=name), expected), name
