@@ -373,6 +373,26 @@ def test_kmajor_weight_fast_path_gives_the_same_bits(gemm, native, shape):
     assert _same_bits(acc_kn.to(torch.bfloat16), expected)
 
 
+@pytest.mark.parametrize("tokens", (256, 200, 520))
+def test_input_gradient_of_the_lm_head_at_full_reduction_length(gemm, oracle, tokens):
+    """dX = dZ[T, V] @ W[V, D] at V = 151936, D = 4096: 2374 K tiles against few outputs, the shape the small
+    K-major tiles serve (direct-to-LDS loop with a shared stage column: 64 x 64 at up to 256 tokens, 128 x 64 up
+    to 512). Every tile shape must give the bits of the 256 x 256 K-major loop, and sampled rows and columns
+    (tile edges included) must meet the oracle's bound."""
+    v, d = 151936, 4096
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(7100 + tokens)
+    w = (torch.randn((v, d), generator=gen, device=DEV) * 0.02).to(torch.bfloat16)  # [K, N]: K-major weight
+    dz = (torch.randn((tokens, v), generator=gen, device=DEV) * 0.01).to(torch.bfloat16)
+    expected = gemm.mfma_gemm(dz, w, config="256x256")
+    for name in ("auto", "64x64", "128x64", "128x128", "256x64"):
+        assert _same_bits(gemm.mfma_gemm(dz, w, config=name), expected), name
+    rows = sorted({0, 63, 64, tokens // 2, tokens - 1})
+    cols = sorted({0, 15, 16, 63, 64, 127, 128, 255, 256, 2047, d - 1})
+    sub = expected[rows][:, cols]
+    _assert_parity(oracle, sub, dz[rows], w[:, cols].t().contiguous(), f"input gradient T={tokens}")
+
+
 @pytest.mark.parametrize("tokens", (1, 7, 63, 64, 65, 100, 257, 1000, 4095))
 def test_weight_gradient_at_any_token_count_keeps_the_bits(gemm, native, oracle, tokens):
     """dW = dY^T @ X reduces over the tokens with both operands K-major. A token count that 64 does not divide
