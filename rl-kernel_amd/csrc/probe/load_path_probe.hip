@@ -6,6 +6,7 @@
 //   2. rate of one workgroup against the bytes it keeps in flight (few workgroups: nothing else is busy)
 //   3. the load side of a small-tile GEMM without its arithmetic: npanels weight panels, each read at the same
 //      pace by the workgroups of its token tiles (all on one XCD), plus the token rows, which stay in the L2
+//   4. L2-resident matrix rows read 128 bytes at a time, by the distance between the rows
 //
 // Loads are the direct-to-LDS DMA form the tile kernels use (or ordinary vector loads, "vgpr"). Build:
 //   hipcc --offload-arch=gfx950 -O3 -o load_path_probe load_path_probe.hip     (rl-kernel_amd/build.py does it)
@@ -178,6 +179,57 @@ static void run_panels(const char* name, const char* buf, int npanels, int token
   fflush(stdout);
 }
 
+// ---- 4: rows of a matrix, 128 bytes at a time ------------------------------------------------------------
+// What a tile kernel's loads look like: a workgroup reads 256 rows x 128 bytes per step (wave w, load u covers
+// rows 32 w + 8 u .. + 7, a lane takes 16 bytes of row lane / 8), rows `row_stride` bytes apart, and moves 128
+// bytes along the rows per step, wrapping after `row_steps`. The workgroups of an XCD read the same 256 rows
+// (L2 hits); the question is whether the distance between rows (pages, DRAM rows, channels) limits a CU.
+__global__ __launch_bounds__(512) void rows_kernel(const char* base, size_t row_stride, int row_steps, int steps,
+                                                   unsigned* sink) {
+  extern __shared__ __align__(1024) char lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const char* mine = base + (size_t)(blockIdx.x % 8) * 256 * row_stride +
+                     (size_t)(32 * wave + (lane >> 3)) * row_stride + (lane & 7) * 16;
+  char* dst = lds + wave * 8192;
+  int pos = (blockIdx.x / 8) % row_steps;
+  for (int s = 0; s < steps; ++s) {
+    const char* src = mine + (size_t)pos * 128;
+    char* d = dst + (s & 1) * 4096;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(src + (size_t)(8 * u) * row_stride), (lds_ptr_t)(d + u * 1024), 16, 0, 0);
+    __builtin_amdgcn_s_waitcnt(kWaitAllVm | 4);
+    if (++pos == row_steps) pos = 0;
+  }
+  __builtin_amdgcn_s_waitcnt(kWaitAllVm);
+  __syncthreads();
+  const unsigned acc = *(unsigned*)(lds + threadIdx.x * 4);
+  if (acc == 0x12345678u) sink[0] = acc;
+}
+
+static void run_rows(const char* name, const char* buf, size_t row_stride, int row_steps, int nwg, unsigned* sink) {
+  require((size_t)(8 * 256) * row_stride <= g_buffer_bytes, "rows exceed the buffer");
+  require((size_t)row_steps * 128 <= row_stride && row_steps >= 1, "row length");
+  const int steps = 2048, lds = 65536;
+  CK(hipFuncSetAttribute((const void*)rows_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+  hipEvent_t a, b;
+  CK(hipEventCreate(&a));
+  CK(hipEventCreate(&b));
+  for (int i = 0; i < 2; ++i) rows_kernel<<<nwg, 512, lds>>>(buf, row_stride, row_steps, steps, sink);
+  CK(hipEventRecord(a));
+  const int reps = 5;
+  for (int i = 0; i < reps; ++i) rows_kernel<<<nwg, 512, lds>>>(buf, row_stride, row_steps, steps, sink);
+  CK(hipEventRecord(b));
+  CK(hipEventSynchronize(b));
+  float ms;
+  CK(hipEventElapsedTime(&ms, a, b));
+  ms /= reps;
+  const double bytes = (double)nwg * steps * 32768;
+  printf("%-40s rows %8zu B apart, %2d steps along a row, %3d workgroups: %6.2f TB/s  %6.1f GB/s per workgroup\n", name,
+         row_stride, row_steps, nwg, bytes / ms * 1e-9, bytes / ms * 1e-6 / nwg);
+  fflush(stdout);
+}
+
 int main() {
   g_buffer_bytes = (size_t)4 << 30;
   char* buf;
@@ -222,6 +274,13 @@ int main() {
     run_panels<1, 6>("256 tokens, 64x64 tiles, quarter touch 6 steps ahead", buf, 64, 4, 3 << 19, ncopies, sink);
     // 1024 tokens, 128 x 128 tiles: 32 panels of 128 features (3 MB), eight token tiles of 128 tokens (3 MB each)
     run_panels<0, 0>("1024 tokens, 128x128 tiles", buf, 32, 8, 3 << 20, ncopies, sink);
+  }
+  printf("== 4. 256 rows x 128 bytes per step out of the L2, by the distance between rows\n");
+  for (int nwg : {8, 256}) {
+    run_rows("rows back to back (8 KB each)", buf, 8192, 64, nwg, sink);
+    run_rows("rows of K = 12288 bf16", buf, 24576, 64, nwg, sink);
+    run_rows("rows of V = 151936 bf16", buf, 303872, 64, nwg, sink);
+    run_rows("rows 1 MB apart", buf, 1 << 20, 64, nwg, sink);
   }
   return 0;
 }
