@@ -148,6 +148,65 @@ __global__ __launch_bounds__(512) void panel_kernel(const char* weights, const c
   if (acc == 0x12345678u) sink[0] = acc;
 }
 
+// The same with the addresses of the real operands: the weight [4096, 12288] and the token rows [T, 12288] are
+// row-major bf16 (rows 24576 bytes apart), a panel is R consecutive rows, a step covers 32 KiB of it (KT K tiles of
+// 128 bytes per row, R * KT = 256) and a load instruction moves 8 rows x 128 bytes, as in the tile kernels.
+template <int R>
+__global__ __launch_bounds__(512) void panel_rows_kernel(const char* weights, const char* tokens, int npanels, int steps,
+                                                         unsigned* sink) {
+  extern __shared__ __align__(1024) char lds[];
+  constexpr int kRowBytes = 24576, kRowBlocks = R / 8, kKt = 256 / R;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int panel = blockIdx.x % npanels, ttile = blockIdx.x / npanels;
+  const char* w = weights + (size_t)panel * R * kRowBytes + (size_t)(lane >> 3) * kRowBytes + (lane & 7) * 16;
+  const char* x = tokens + (size_t)ttile * R * kRowBytes + (size_t)(lane >> 3) * kRowBytes + (lane & 7) * 16;
+  char* mine = lds + wave * 16384;
+  for (int s = 0; s < steps; ++s) {
+    char* dst = mine + (s & 1) * 8192;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = wave * 4 + u;  // block j of the step: rows 8 (j % kRowBlocks) .., K tile j / kRowBlocks
+      const size_t off = (size_t)(8 * (j % kRowBlocks)) * kRowBytes + (size_t)(s * kKt + j / kRowBlocks) * 128;
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(w + off), (lds_ptr_t)(dst + u * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(x + off), (lds_ptr_t)(dst + 4096 + u * 1024), 16, 0, 0);
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitAllVm | 8);
+  }
+  __builtin_amdgcn_s_waitcnt(kWaitAllVm);
+  __syncthreads();
+  const unsigned acc = *(unsigned*)(lds + threadIdx.x * 4);
+  if (acc == 0x12345678u) sink[0] = acc;
+}
+
+template <int R>
+static void run_panel_rows(const char* name, const char* buf, int token_tiles, int ncopies, unsigned* sink) {
+  constexpr size_t kRowBytes = 24576;
+  const int npanels = 4096 / R, steps = (int)(kRowBytes / ((256 / R) * 128));
+  const size_t copy_bytes = 4096 * kRowBytes, token_bytes = (size_t)token_tiles * R * kRowBytes;
+  require((size_t)ncopies * copy_bytes + token_bytes <= g_buffer_bytes, "operands exceed the buffer");
+  const char* tokens = buf + (size_t)ncopies * copy_bytes;
+  const int lds = 131072, nwg = npanels * token_tiles;
+  CK(hipFuncSetAttribute((const void*)panel_rows_kernel<R>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+  hipEvent_t a, b;
+  CK(hipEventCreate(&a));
+  CK(hipEventCreate(&b));
+  int c = 0;
+  for (int i = 0; i < 5; ++i, c = (c + 1) % ncopies)
+    panel_rows_kernel<R><<<nwg, 512, lds>>>(buf + (size_t)c * copy_bytes, tokens, npanels, steps, sink);
+  CK(hipEventRecord(a));
+  const int reps = 40;
+  for (int i = 0; i < reps; ++i, c = (c + 1) % ncopies)
+    panel_rows_kernel<R><<<nwg, 512, lds>>>(buf + (size_t)c * copy_bytes, tokens, npanels, steps, sink);
+  CK(hipEventRecord(b));
+  CK(hipEventSynchronize(b));
+  float ms;
+  CK(hipEventElapsedTime(&ms, a, b));
+  ms /= reps;
+  printf("%-58s %3d panels x %d token tiles, weights %s: %6.1f us per launch\n", name, npanels, token_tiles,
+         ncopies == 1 ? "relaunched (memory-side cache)" : "rotating (from HBM)          ", ms * 1e3);
+  fflush(stdout);
+}
+
 template <int PREFETCH, int LEAD>
 static void run_panels(const char* name, const char* buf, int npanels, int token_tiles, size_t panel_bytes,
                        int ncopies, unsigned* sink) {
@@ -274,6 +333,9 @@ int main() {
     run_panels<1, 6>("256 tokens, 64x64 tiles, quarter touch 6 steps ahead", buf, 64, 4, 3 << 19, ncopies, sink);
     // 1024 tokens, 128 x 128 tiles: 32 panels of 128 features (3 MB), eight token tiles of 128 tokens (3 MB each)
     run_panels<0, 0>("1024 tokens, 128x128 tiles", buf, 32, 8, 3 << 20, ncopies, sink);
+    // and with the row-major addresses of the operands themselves
+    run_panel_rows<64>("256 tokens, 64x64 tiles, row-major operands", buf, 4, ncopies, sink);
+    run_panel_rows<128>("1024 tokens, 128x128 tiles, row-major operands", buf, 8, ncopies, sink);
   }
   printf("== 4. 256 rows x 128 bytes per step out of the L2, by the distance between rows\n");
   for (int nwg : {8, 256}) {
