@@ -7,6 +7,7 @@
 //   3. the load side of a small-tile GEMM without its arithmetic: npanels weight panels, each read at the same
 //      pace by the workgroups of its token tiles (all on one XCD), plus the token rows, which stay in the L2
 //   4. L2-resident matrix rows read 128 bytes at a time, by the distance between the rows
+//   5. the load side of the 256 x 256 tile GEMM at its headline shape
 //
 // Loads are the direct-to-LDS DMA form the tile kernels use (or ordinary vector loads, "vgpr"). Build:
 //   hipcc --offload-arch=gfx950 -O3 -o load_path_probe load_path_probe.hip     (rl-kernel_amd/build.py does it)
@@ -289,6 +290,61 @@ static void run_rows(const char* name, const char* buf, size_t row_stride, int r
   fflush(stdout);
 }
 
+// ---- 5: the load side of the 256 x 256 tile GEMM at its headline shape ------------------------------------
+// gate_up at 4096 tokens (W [24576, 4096], X [4096, 4096], bf16, rows of 8 KiB): 1536 workgroups, each 64 steps
+// of (256 weight rows + 256 token rows) x 128 bytes with the previous step awaited before the next is issued
+// (one K tile of lead, as in the kernel), and the kernel's raster (XCD-compact ids, groups of eight token tiles).
+__global__ __launch_bounds__(512) void big_tile_kernel(const char* weights, const char* tokens, int tiles_m, int tiles_n,
+                                                       unsigned* sink) {
+  extern __shared__ __align__(1024) char lds[];
+  constexpr int kRowBytes = 8192;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int per_xcd = tiles_m * tiles_n / 8;
+  const int id = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  const int group_m = 8, per_group = group_m * tiles_n;
+  const int group = id / per_group, within = id - group * per_group;
+  const int tile_m = group * group_m + within % group_m, tile_n = within / group_m;
+  const char* w = weights + (size_t)tile_n * 256 * kRowBytes + (size_t)(lane >> 3) * kRowBytes + (lane & 7) * 16;
+  const char* x = tokens + (size_t)tile_m * 256 * kRowBytes + (size_t)(lane >> 3) * kRowBytes + (lane & 7) * 16;
+  char* mine = lds + wave * 16384;
+  for (int s = 0; s < 64; ++s) {
+    char* dst = mine + (s & 1) * 8192;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const size_t off = (size_t)(8 * (wave * 4 + u)) * kRowBytes + (size_t)s * 128;
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(w + off), (lds_ptr_t)(dst + u * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(x + off), (lds_ptr_t)(dst + 4096 + u * 1024), 16, 0, 0);
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitAllVm | 8);
+  }
+  __builtin_amdgcn_s_waitcnt(kWaitAllVm);
+  __syncthreads();
+  const unsigned acc = *(unsigned*)(lds + threadIdx.x * 4);
+  if (acc == 0x12345678u) sink[0] = acc;
+}
+
+static void run_big_tile(const char* buf, unsigned* sink) {
+  const int tiles_m = 16, tiles_n = 96, lds = 131072;
+  const size_t wbytes = (size_t)24576 * 8192, xbytes = (size_t)4096 * 8192;
+  require(wbytes + xbytes <= g_buffer_bytes, "operands exceed the buffer");
+  CK(hipFuncSetAttribute((const void*)big_tile_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+  hipEvent_t a, b;
+  CK(hipEventCreate(&a));
+  CK(hipEventCreate(&b));
+  for (int i = 0; i < 5; ++i) big_tile_kernel<<<tiles_m * tiles_n, 512, lds>>>(buf, buf + wbytes, tiles_m, tiles_n, sink);
+  CK(hipEventRecord(a));
+  const int reps = 20;
+  for (int i = 0; i < reps; ++i) big_tile_kernel<<<tiles_m * tiles_n, 512, lds>>>(buf, buf + wbytes, tiles_m, tiles_n, sink);
+  CK(hipEventRecord(b));
+  CK(hipEventSynchronize(b));
+  float ms;
+  CK(hipEventElapsedTime(&ms, a, b));
+  ms /= reps;
+  printf("gate_up at 4096 tokens, 256x256 tiles, loads only: %6.1f us per launch (%.1f TB/s out of the L2s)\n", ms * 1e3,
+         1536.0 * 64 * 65536 / ms * 1e-9);
+  fflush(stdout);
+}
+
 int main() {
   g_buffer_bytes = (size_t)4 << 30;
   char* buf;
@@ -344,5 +400,7 @@ int main() {
     run_rows("rows of V = 151936 bf16", buf, 303872, 64, nwg, sink);
     run_rows("rows 1 MB apart", buf, 1 << 20, 64, nwg, sink);
   }
+  printf("== 5. load side of the 256 x 256 tile GEMM at the headline shape, no arithmetic\n");
+  run_big_tile(buf, sink);
   return 0;
 }
