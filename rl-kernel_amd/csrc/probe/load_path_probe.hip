@@ -8,6 +8,7 @@
 //      pace by the workgroups of its token tiles (all on one XCD), plus the token rows, which stay in the L2
 //   4. L2-resident matrix rows read 128 bytes at a time, by the distance between the rows
 //   5. the load side of the 256 x 256 tile GEMM at its headline shape
+//   6. the other side: the matrix pipe alone, the same MFMA sequence out of registers, at the power cap
 //
 // Loads are the direct-to-LDS DMA form the tile kernels use (or ordinary vector loads, "vgpr"). Build:
 //   hipcc --offload-arch=gfx950 -O3 -o load_path_probe load_path_probe.hip     (rl-kernel_amd/build.py does it)
@@ -345,6 +346,91 @@ static void run_big_tile(const char* buf, unsigned* sink) {
   fflush(stdout);
 }
 
+// ---- 6: the matrix pipe alone ----------------------------------------------------------------------------
+// The MFMA sequence of the 256 x 256 tile kernel out of registers: per wave and K tile 64 v_mfma_f32_16x16x32_bf16
+// (4 weight x 8 token fragments, two K steps), eight waves per CU, no loads, no LDS. One launch is the matrix work
+// of gate_up at 4096 tokens. With random bf16 operand values (weights scaled by 0.02, as in the benchmark) and
+// with zeros: what the part sustains at its power cap when nothing but the matrix pipe runs.
+typedef __attribute__((ext_vector_type(8))) __bf16 probe_bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float probe_f32x4_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t probe_u32x4_t;
+
+__global__ __launch_bounds__(512) void mfma_only_kernel(const probe_u32x4_t* frags, int ktiles, float* sink) {
+  const int lane = threadIdx.x & 63;
+  probe_u32x4_t w[2][4], x[2][8];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[s][j] = frags[(s * 12 + j) * 64 + lane];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[s][j] = frags[(s * 12 + 4 + j) * 64 + lane];
+  }
+  probe_f32x4_t acc[4][8];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 8; ++b) acc[a][b] = probe_f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < ktiles; ++t) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 8; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(probe_bf16x8_t, w[s][a]),
+                                                               __builtin_bit_cast(probe_bf16x8_t, x[s][b]), acc[a][b], 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(w[0][j]), "+v"(w[1][j]));  // the loop is not collapsed
+  }
+  float r = 0.f;
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 8; ++b) r += acc[a][b][0] + acc[a][b][1] + acc[a][b][2] + acc[a][b][3];
+  if (r == 123.456f) sink[0] = r;
+}
+
+static uint16_t probe_bf16_of(float f) {
+  uint32_t u;
+  __builtin_memcpy(&u, &f, 4);
+  return (uint16_t)((u + 0x7fff + ((u >> 16) & 1)) >> 16);
+}
+
+static void run_mfma_only(char* buf, unsigned* sink) {
+  constexpr int kFrags = 24 * 64;  // 24 fragments of 64 lanes x 16 bytes
+  static uint16_t host[kFrags * 8];
+  for (int mode = 0; mode < 2; ++mode) {
+    srand(7);
+    for (int i = 0; i < kFrags * 8; ++i) {
+      float g = 0.f;  // a sum of 12 uniforms: about normal
+      for (int q = 0; q < 12; ++q) g += (float)(rand() % 65536) / 65536.f;
+      g -= 6.f;
+      const int frag = (i / 8 / 64) % 12;
+      host[i] = mode == 0 ? probe_bf16_of(frag < 4 ? 0.02f * g : g) : 0;
+    }
+    CK(hipMemcpy(buf, host, sizeof(host), hipMemcpyHostToDevice));
+    const int ktiles = 64 * 6;  // 256 workgroups x 6 tiles x 64 K tiles = the 1536 tiles of gate_up at 4096 tokens
+    hipEvent_t a, b;
+    CK(hipEventCreate(&a));
+    CK(hipEventCreate(&b));
+    for (int i = 0; i < 100; ++i)  // the clocks settle
+      mfma_only_kernel<<<256, 512>>>(reinterpret_cast<const probe_u32x4_t*>(buf), ktiles, reinterpret_cast<float*>(sink));
+    CK(hipEventRecord(a));
+    const int reps = 200;
+    for (int i = 0; i < reps; ++i)
+      mfma_only_kernel<<<256, 512>>>(reinterpret_cast<const probe_u32x4_t*>(buf), ktiles, reinterpret_cast<float*>(sink));
+    CK(hipEventRecord(b));
+    CK(hipEventSynchronize(b));
+    float ms;
+    CK(hipEventElapsedTime(&ms, a, b));
+    ms /= reps;
+    const double flops = 256.0 * 8 * ktiles * 64 * (2.0 * 16 * 16 * 32);
+    printf("matrix pipe only, %s operands: %6.1f us per launch of %.1f GFLOP = %6.1f TFLOP/s (%.1f %% of 2.5 PFLOP/s)\n",
+           mode == 0 ? "random" : "zero  ", ms * 1e3, flops * 1e-9, flops / ms * 1e-9, flops / ms * 1e-9 / 25.0);
+    fflush(stdout);
+  }
+}
+
 int main() {
   g_buffer_bytes = (size_t)4 << 30;
   char* buf;
@@ -402,5 +488,7 @@ int main() {
   }
   printf("== 5. load side of the 256 x 256 tile GEMM at the headline shape, no arithmetic\n");
   run_big_tile(buf, sink);
+  printf("== 6. the matrix pipe alone: the MFMA sequence of the 256 x 256 tile kernel out of registers\n");
+  run_mfma_only(buf, sink);
   return 0;
 }
