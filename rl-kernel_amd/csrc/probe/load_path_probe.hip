@@ -9,6 +9,7 @@
 //   4. L2-resident matrix rows read 128 bytes at a time, by the distance between the rows
 //   5. the load side of the 256 x 256 tile GEMM at its headline shape
 //   6. the other side: the matrix pipe alone, the same MFMA sequence out of registers, at the power cap
+//   7. that sequence with the kernel's LDS reads, L2 loads and barriers added, and the shader clock each variant sees
 //
 // Loads are the direct-to-LDS DMA form the tile kernels use (or ordinary vector loads, "vgpr"). Build:
 //   hipcc --offload-arch=gfx950 -O3 -o load_path_probe load_path_probe.hip     (rl-kernel_amd/build.py does it)
@@ -431,12 +432,137 @@ static void run_mfma_only(char* buf, unsigned* sink) {
   }
 }
 
+// ---- 7: what the data movement of the tile kernel costs the matrix pipe ------------------------------------
+// The MFMA sequence of section 6 with, one after the other, the kernel's LDS fragment reads (24 ds_read_b128 per
+// wave and K tile at the kernel's addresses), its direct-to-LDS loads (8 per wave and K tile = 64 KiB per workgroup,
+// from 4 MiB that stay in the L2) and two barriers per K tile; every wave reads, loads and multiplies (no roles).
+// Workgroup 0 also reports the shader clock it saw (clock64 against the 100 MHz wall clock): on zero operands the
+// clock stays at its maximum and the cost is cycles, on random operands the power cap turns bytes into clock.
+// MODE bit 0: fragment reads, bit 1: loads, bit 2: barriers.
+template <int MODE>
+__global__ __launch_bounds__(512) void mfma_with_traffic_kernel(const char* src, int ktiles, float* sink) {
+  extern __shared__ __align__(1024) char lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wave_n = wave & 3, wave_m = wave >> 2;
+  const int l16 = lane & 15, grp = lane >> 4;
+  for (int i = tid; i < 131072 / 16; i += 512)
+    reinterpret_cast<probe_u32x4_t*>(lds)[i] = reinterpret_cast<const probe_u32x4_t*>(src)[i];
+  __syncthreads();
+  const int frag_lo = (grp ^ (l16 & 7)) << 4;
+  const int w_row = (wave_n * 64 + l16) * 128, x_row = 256 * 128 + (wave_m * 128 + l16) * 128;
+  probe_u32x4_t w[2][4], x[2][8];
+  auto read_frags = [&](const char* st) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        w[s][j] = *reinterpret_cast<const probe_u32x4_t*>(st + w_row + j * 16 * 128 + (frag_lo ^ (s << 6)));
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        x[s][j] = *reinterpret_cast<const probe_u32x4_t*>(st + x_row + j * 16 * 128 + (frag_lo ^ (s << 6)));
+    }
+  };
+  read_frags(lds);
+  const long long c0 = clock64(), r0 = wall_clock64();
+  probe_f32x4_t acc[4][8];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 8; ++b) acc[a][b] = probe_f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const char* gsrc = src + (size_t)(blockIdx.x % 32) * 131072 + wave * 8192 + lane * 16;  // 4 MiB per 32 workgroups
+  for (int t = 0; t < ktiles; ++t) {
+    char* st = lds + (t & 1) * 65536;
+    if (MODE & 2) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(gsrc + (t & 1) * 65536 + u * 1024),
+                                         (lds_ptr_t)(st + wave * 8192 + u * 1024), 16, 0, 0);
+    }
+    if (MODE & 1) read_frags(lds + ((t + 1) & 1) * 65536);
+    if (MODE & 4) __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 8; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(probe_bf16x8_t, w[s][a]),
+                                                               __builtin_bit_cast(probe_bf16x8_t, x[s][b]), acc[a][b], 0, 0, 0);
+    if (MODE & 4) __builtin_amdgcn_s_barrier();
+    if (!(MODE & 1)) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(w[0][j]), "+v"(w[1][j]));
+    }
+    if (MODE & 2) __builtin_amdgcn_s_waitcnt(kWaitAllVm | 8);
+  }
+  __builtin_amdgcn_s_waitcnt(kWaitAllVm);
+  float r = 0.f;
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 8; ++b) r += acc[a][b][0] + acc[a][b][1] + acc[a][b][2] + acc[a][b][3];
+  if (r == 123.456f) sink[0] = r;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    const long long c1 = clock64(), r1 = wall_clock64();
+    reinterpret_cast<long long*>(sink)[1] = c1 - c0;
+    reinterpret_cast<long long*>(sink)[2] = r1 - r0;
+  }
+}
+
+template <int MODE>
+static void run_mfma_with_traffic(const char* name, const char* buf, float* sink) {
+  CK(hipFuncSetAttribute((const void*)mfma_with_traffic_kernel<MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, 131072));
+  const int ktiles = 64 * 6;
+  hipEvent_t a, b;
+  CK(hipEventCreate(&a));
+  CK(hipEventCreate(&b));
+  for (int i = 0; i < 100; ++i) mfma_with_traffic_kernel<MODE><<<256, 512, 131072>>>(buf, ktiles, sink);
+  CK(hipEventRecord(a));
+  const int reps = 200;
+  for (int i = 0; i < reps; ++i) mfma_with_traffic_kernel<MODE><<<256, 512, 131072>>>(buf, ktiles, sink);
+  CK(hipEventRecord(b));
+  CK(hipEventSynchronize(b));
+  float ms;
+  CK(hipEventElapsedTime(&ms, a, b));
+  ms /= reps;
+  long long rec[4];
+  CK(hipMemcpy(rec, sink, 32, hipMemcpyDeviceToHost));
+  const double flops = 256.0 * 8 * ktiles * 64 * (2.0 * 16 * 16 * 32);
+  printf("%-50s %6.1f us  %6.1f TFLOP/s  shader clock %.2f GHz\n", name, ms * 1e3, flops / ms * 1e-9,
+         (double)rec[1] / (double)rec[2] * 0.1);
+  fflush(stdout);
+}
+
+static void run_traffic_cost(char* buf, char* sink_bytes) {
+  constexpr size_t kBytes = (size_t)8 << 20;  // 4 MiB are read; stages of 64 KiB: weight rows first (scaled by 0.02)
+  static uint16_t host[kBytes / 2];
+  float* sink = reinterpret_cast<float*>(sink_bytes);
+  for (int mode = 0; mode < 2; ++mode) {
+    srand(7);
+    for (size_t i = 0; i < kBytes / 2; ++i) {
+      float g = 0.f;
+      for (int q = 0; q < 12; ++q) g += (float)(rand() % 65536) / 65536.f;
+      g -= 6.f;
+      host[i] = mode == 0 ? probe_bf16_of(((i * 2) % 65536) < 32768 ? 0.02f * g : g) : 0;
+    }
+    CK(hipMemcpy(buf, host, kBytes, hipMemcpyHostToDevice));
+    printf("   %s operands\n", mode == 0 ? "random" : "zero");
+    run_mfma_with_traffic<0>("matrix pipe only", buf, sink);
+    run_mfma_with_traffic<1>("+ LDS fragment reads", buf, sink);
+    run_mfma_with_traffic<3>("+ fragment reads + direct-to-LDS loads from L2", buf, sink);
+    run_mfma_with_traffic<7>("+ reads + loads + two barriers per K tile", buf, sink);
+    run_mfma_with_traffic<2>("matrix pipe + direct-to-LDS loads only", buf, sink);
+  }
+}
+
 int main() {
   g_buffer_bytes = (size_t)4 << 30;
   char* buf;
   unsigned* sink;
   CK(hipMalloc(&buf, g_buffer_bytes));
   CK(hipMalloc(&sink, 4));
+  char* scratch;
+  CK(hipMalloc(&scratch, 32));
   CK(hipMemset(buf, 1, g_buffer_bytes));
   CK(hipDeviceSynchronize());
 
@@ -490,5 +616,7 @@ int main() {
   run_big_tile(buf, sink);
   printf("== 6. the matrix pipe alone: the MFMA sequence of the 256 x 256 tile kernel out of registers\n");
   run_mfma_only(buf, sink);
+  printf("== 7. the same sequence with the kernel's LDS reads, L2 loads and barriers added one after the other\n");
+  run_traffic_cost(buf, scratch);
   return 0;
 }
