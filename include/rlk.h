@@ -54,7 +54,8 @@ typedef enum rlk_gemm_config {
   RLK_GEMM_CFG_256x256_SOLO = 15, /* 256 x 256 tile on four waves (one per SIMD, 128 x 128 each) */
   RLK_GEMM_CFG_192x256 = 16,      /* 192 features x 256 tokens (N / 192 tiles where N / 256 leaves a round half empty) */
   RLK_GEMM_CFG_SHORTK = 17,       /* K <= 256, K-major token operand: features stationary in registers, tokens streamed */
-  RLK_GEMM_CFG_COUNT = 18,
+  RLK_GEMM_CFG_192x128 = 18,      /* 192 features x 128 tokens, three stages (N / 192 x M / 128 tiles that fill one round) */
+  RLK_GEMM_CFG_COUNT = 19,
   /* OR-ed into a configuration: use the register-staged main loop even where the
    * direct-to-LDS ping-pong loop applies. Bit-neutral; exists so tests can
    * compare the two loops. */

@@ -293,7 +293,7 @@ static hipError_t launch_loop(const MatView& W, const MatView& X, void* C, int64
 // deep-stage variants; the K-major loops measured no gain from a third stage and keep two.
 template <class S>
 constexpr int pingpong_stages() {
-  return (S::BN == 256 && S::BM <= 128) ? 3 : 2;
+  return (S::BN >= 192 && S::BM <= 128) ? 3 : 2;
 }
 
 // kmajor_loop: 0, or the K-major ping-pong variant the operand layouts call for.
@@ -357,6 +357,7 @@ static hipError_t launch_staged_kmajor(const MatView& W, const MatView& X, void*
 using Shape256x256 = TileShape<256, 256, 4, 2>;
 using Shape256x256Solo = TileShape<256, 256, 2, 2>;
 using Shape192x256 = TileShape<192, 256, 4, 2>;  // 192 features x 256 tokens: three MFMA tiles per wave along N
+using Shape192x128 = TileShape<192, 128, 4, 2>;  // 192 features x 128 tokens
 using Shape256x128 = TileShape<256, 128, 4, 2>;
 using Shape256x64 = TileShape<256, 64, 4, 2>;
 using Shape128x128 = TileShape<128, 128, 4, 2>;
@@ -408,9 +409,12 @@ int pick_det_gemm_config(int M, int N, int K) {
   // last feature tile is partly empty and the shape counts as 0.85: it still wins where it turns a round and a
   // fraction into less (N = 5120 at 4096 tokens 293 -> 256 us, N = 10240 at 2048 tokens 190 -> 162 us, N = 2560 at
   // 8192 tokens 347 -> 308 us) and loses the tie against 256 x 128 at N = 4096, 2048 tokens (177 against 166 us).
+  // 192 x 128 (three stages) does the same one size down: N / 192 x M / 128 tiles fill a round that 256 x 128 leaves a
+  // quarter empty (weights from HBM: gate_up at 256 tokens 65.0 -> 62.2 us, N = 12288 at 384 tokens 58.4 -> 53.2,
+  // N = 6144 at 768 tokens 55.1 -> 49.1, N = 5120 at 1024 tokens 72.7 -> 63.5).
   static const Candidate kCandidates[] = {
       {RLK_GEMM_CFG_256x256, 256, 256, 1.00}, {RLK_GEMM_CFG_192x256, 192, 256, 0.89},
-      {RLK_GEMM_CFG_256x128, 256, 128, 0.65},
+      {RLK_GEMM_CFG_256x128, 256, 128, 0.65}, {RLK_GEMM_CFG_192x128, 192, 128, 0.56},
       {RLK_GEMM_CFG_256x64, 256, 64, 0.50},
       {RLK_GEMM_CFG_128x128, 128, 128, 0.65}, {RLK_GEMM_CFG_128x64, 128, 64, 0.45},
       {RLK_GEMM_CFG_64x64, 64, 64, 0.42},
@@ -418,8 +422,9 @@ int pick_det_gemm_config(int M, int N, int K) {
   int best = RLK_GEMM_CFG_64x64;
   double best_time = 1e300;
   for (const Candidate& c : kCandidates) {
-    if (c.config == RLK_GEMM_CFG_192x256 && K % kTileK != 0) continue;
-    const double quality = (c.config == RLK_GEMM_CFG_192x256 && N % 192 != 0) ? 0.85 : c.quality;
+    const bool wide192 = c.config == RLK_GEMM_CFG_192x256 || c.config == RLK_GEMM_CFG_192x128;
+    if (wide192 && K % kTileK != 0) continue;
+    const double quality = (wide192 && N % 192 != 0) ? (c.config == RLK_GEMM_CFG_192x256 ? 0.85 : 0.53) : c.quality;
     const int64_t tiles = tile_count(M, N, c.bm, c.bn);
     const int64_t full = tiles / kCus;
     const double part = (double)(tiles - full * kCus) / kCus;
@@ -589,6 +594,11 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
     if (vec && allow_pingpong && K % kTileK == 0)
       return launch_loop<Shape256x256Solo, kLoopSolo>(W, X, C, ldc, M, N, K, out_f32, stream);
     config = RLK_GEMM_CFG_256x256;
+  }
+  if (config == RLK_GEMM_CFG_192x128) {
+    if (vec && allow_pingpong && K % kTileK == 0)
+      return launch_loop<Shape192x128, kLoopPingPong, pingpong_stages<Shape192x128>()>(W, X, C, ldc, M, N, K, out_f32, stream);
+    config = RLK_GEMM_CFG_256x128;
   }
   if (config == RLK_GEMM_CFG_192x256) {
     if (vec && allow_pingpong && K % kTileK == 0)

@@ -40,6 +40,7 @@ GEMM_CONFIGS = {
     "256x256_solo": 15,
     "192x256": 16,
     "shortk": 17,
+    "192x128": 18,
 }
 # OR-ed into a GEMM or LogP configuration: register-staged main loop (bit-neutral).
 FORCE_STAGED = 0x100
