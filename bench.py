@@ -7,7 +7,10 @@ H[4096,12288] x W[4096,12288]^T, inputs resident in HBM. The JSON line also carr
 
 * ``roofline``     - the dominant kernel (the 256x256-tile MFMA kernel on gate_up)
                      against the MI355X dense bf16 MFMA peak, timed with HIP events
-                     on the launch stream;
+                     on the launch stream; ``roofline.matrix_pipe_alone`` adds, for orientation,
+                     what the same MFMA sequence sustains on this machine out of registers with
+                     nothing else running (random and zero operands; ``rl-kernel_amd/load_path_probe 6``,
+                     a child process started before this one touches the GPU);
 * ``cpu_baseline`` - the CPU oracle (``oracle/reference_math.det_gemm_ref``) timed on
                      this box's host cores on the same step;
 * ``shapes``       - every token count of the configuration (T = 1, 16, 64, 256, 1024, 4096)
@@ -65,6 +68,26 @@ def _measured_traffic() -> dict:
     except (OSError, ValueError):
         pass
     return out
+
+
+def _matrix_pipe_alone() -> dict | None:
+    """What the matrix pipe sustains at the power cap when nothing else runs: the MFMA sequence of the 256 x 256 tile
+    kernel out of registers, on random and on zero operands (section 6 of rl-kernel_amd/load_path_probe, a program of
+    its own, run as a child process before this process touches the GPU). None when the program is missing or fails."""
+    import re
+    import subprocess
+
+    probe = ROOT / "rl-kernel_amd" / "load_path_probe"
+    if not probe.exists():
+        return None
+    try:
+        done = subprocess.run([str(probe), "6"], stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True, timeout=120)
+    except (OSError, subprocess.SubprocessError):
+        return None
+    found = {}
+    for kind, value in re.findall(r"matrix pipe only, (random|zero)\s+operands:.*?=\s*([0-9.]+) TFLOP/s", done.stdout):
+        found[f"{kind}_operands_tflops"] = float(value)
+    return found if done.returncode == 0 and len(found) == 2 else None
 
 
 def _parse():
@@ -128,6 +151,9 @@ def main() -> int:
             file=sys.stderr,
         )
         return 2
+
+    # a child process; it has to start before this process initialises the GPU
+    matrix_pipe_alone = _matrix_pipe_alone() if args.only == "" else None
 
     import torch
 
@@ -391,6 +417,10 @@ def main() -> int:
         "traffic_measured_on_commit": traffic["commit"],
     }
     roofline.update(_launch_percentiles(gate_up, args.steps, 5))
+    if matrix_pipe_alone is not None:
+        # orientation: the matrix pipe with nothing else running, same MFMA sequence, at the power cap of this machine
+        roofline["matrix_pipe_alone"] = dict(
+            matrix_pipe_alone, frac_of_random_operands_rate=round(achieved / matrix_pipe_alone["random_operands_tflops"], 4))
 
     result = {
         "metric": "bf16 det-GEMM TFLOP/s at Qwen3-8B FFN shapes (gate_up + down, T=4096)",

@@ -13,6 +13,7 @@
 //
 // Loads are the direct-to-LDS DMA form the tile kernels use (or ordinary vector loads, "vgpr"). Build:
 //   hipcc --offload-arch=gfx950 -O3 -o load_path_probe load_path_probe.hip     (rl-kernel_amd/build.py does it)
+// Run without arguments for every section, or with one section number.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -555,7 +556,10 @@ static void run_traffic_cost(char* buf, char* sink_bytes) {
   }
 }
 
-int main() {
+// Without arguments every section runs; with a section number (1 .. 7) only that one.
+int main(int argc, char** argv) {
+  const int only = argc > 1 ? atoi(argv[1]) : 0;
+  auto want = [&](int section) { return only == 0 || only == section; };
   g_buffer_bytes = (size_t)4 << 30;
   char* buf;
   unsigned* sink;
@@ -566,57 +570,69 @@ int main() {
   CK(hipMemset(buf, 1, g_buffer_bytes));
   CK(hipDeviceSynchronize());
 
-  printf("== 1. ceilings, every CU loading\n");
-  run_streams<0, 8, 8>("L2: all workgroups cycle over 1 MB", buf, 1 << 20, 1, 256, 400, sink);
-  run_streams<1, 8, 8>("L2: all workgroups cycle over 1 MB", buf, 1 << 20, 1, 256, 400, sink);
-  run_streams<0, 8, 8>("memory-side cache: 128 MB cycled", buf, 1 << 19, 256, 256, 400, sink);
-  run_streams<1, 8, 8>("memory-side cache: 128 MB cycled", buf, 1 << 19, 256, 256, 400, sink);
-  run_streams<0, 8, 8>("HBM: 4 GB once, 16 MB per workgroup", buf, 16 << 20, 256, 256, 256, sink);
-  run_streams<1, 8, 8>("HBM: 4 GB once, 16 MB per workgroup", buf, 16 << 20, 256, 256, 256, sink);
-  run_streams<1, 4, 8>("HBM: 4 GB once, 2 MB per workgroup", buf, 2 << 20, 2048, 2048, 64, sink);
-
-  printf("== 2. one workgroup's rate against its bytes in flight (each streams its own 16 MB from HBM)\n");
-  for (int nwg : {32, 256}) {
-    run_streams<0, 1, 1>("HBM", buf, 16 << 20, nwg, nwg, 2048, sink);
-    run_streams<0, 1, 4>("HBM", buf, 16 << 20, nwg, nwg, 2048, sink);
-    run_streams<0, 2, 4>("HBM", buf, 16 << 20, nwg, nwg, 2048, sink);
-    run_streams<0, 4, 4>("HBM", buf, 16 << 20, nwg, nwg, 1024, sink);
-    run_streams<0, 8, 4>("HBM", buf, 16 << 20, nwg, nwg, 512, sink);
-    run_streams<0, 8, 8>("HBM", buf, 16 << 20, nwg, nwg, 256, sink);
+  if (want(1)) {
+    printf("== 1. ceilings, every CU loading\n");
+    run_streams<0, 8, 8>("L2: all workgroups cycle over 1 MB", buf, 1 << 20, 1, 256, 400, sink);
+    run_streams<1, 8, 8>("L2: all workgroups cycle over 1 MB", buf, 1 << 20, 1, 256, 400, sink);
+    run_streams<0, 8, 8>("memory-side cache: 128 MB cycled", buf, 1 << 19, 256, 256, 400, sink);
+    run_streams<1, 8, 8>("memory-side cache: 128 MB cycled", buf, 1 << 19, 256, 256, 400, sink);
+    run_streams<0, 8, 8>("HBM: 4 GB once, 16 MB per workgroup", buf, 16 << 20, 256, 256, 256, sink);
+    run_streams<1, 8, 8>("HBM: 4 GB once, 16 MB per workgroup", buf, 16 << 20, 256, 256, 256, sink);
+    run_streams<1, 4, 8>("HBM: 4 GB once, 2 MB per workgroup", buf, 2 << 20, 2048, 2048, 64, sink);
   }
-  for (int nwg : {8, 256}) {
-    printf("   (each workgroup cycles over its own 64 KB: L2 hits)\n");
-    run_streams<0, 1, 1>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
-    run_streams<0, 1, 4>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
-    run_streams<0, 2, 4>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
-    run_streams<0, 4, 4>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
-    run_streams<0, 8, 8>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
+  if (want(2)) {
+    printf("== 2. one workgroup's rate against its bytes in flight (each streams its own 16 MB from HBM)\n");
+    for (int nwg : {32, 256}) {
+      run_streams<0, 1, 1>("HBM", buf, 16 << 20, nwg, nwg, 2048, sink);
+      run_streams<0, 1, 4>("HBM", buf, 16 << 20, nwg, nwg, 2048, sink);
+      run_streams<0, 2, 4>("HBM", buf, 16 << 20, nwg, nwg, 2048, sink);
+      run_streams<0, 4, 4>("HBM", buf, 16 << 20, nwg, nwg, 1024, sink);
+      run_streams<0, 8, 4>("HBM", buf, 16 << 20, nwg, nwg, 512, sink);
+      run_streams<0, 8, 8>("HBM", buf, 16 << 20, nwg, nwg, 256, sink);
+    }
+    for (int nwg : {8, 256}) {
+      printf("   (each workgroup cycles over its own 64 KB: L2 hits)\n");
+      run_streams<0, 1, 1>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
+      run_streams<0, 1, 4>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
+      run_streams<0, 2, 4>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
+      run_streams<0, 4, 4>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
+      run_streams<0, 8, 8>("L2", buf, 64 << 10, nwg, nwg, 4096, sink);
+    }
   }
-
-  printf("== 3. load side of the small-tile GEMMs of the down projection (4096 features, K = 12288), no arithmetic\n");
-  for (int ncopies : {1, 14}) {
-    // 256 tokens, 64 x 64 tiles: 64 panels of 64 features (1.5 MB), four token tiles of 64 tokens (1.5 MB each)
-    run_panels<0, 0>("256 tokens, 64x64 tiles", buf, 64, 4, 3 << 19, ncopies, sink);
-    run_panels<1, 2>("256 tokens, 64x64 tiles, quarter touch 2 steps ahead", buf, 64, 4, 3 << 19, ncopies, sink);
-    run_panels<1, 6>("256 tokens, 64x64 tiles, quarter touch 6 steps ahead", buf, 64, 4, 3 << 19, ncopies, sink);
-    // 1024 tokens, 128 x 128 tiles: 32 panels of 128 features (3 MB), eight token tiles of 128 tokens (3 MB each)
-    run_panels<0, 0>("1024 tokens, 128x128 tiles", buf, 32, 8, 3 << 20, ncopies, sink);
-    // and with the row-major addresses of the operands themselves
-    run_panel_rows<64>("256 tokens, 64x64 tiles, row-major operands", buf, 4, ncopies, sink);
-    run_panel_rows<128>("1024 tokens, 128x128 tiles, row-major operands", buf, 8, ncopies, sink);
+  if (want(3)) {
+    printf("== 3. load side of the small-tile GEMMs of the down projection (4096 features, K = 12288), no arithmetic\n");
+    for (int ncopies : {1, 14}) {
+      // 256 tokens, 64 x 64 tiles: 64 panels of 64 features (1.5 MB), four token tiles of 64 tokens (1.5 MB each)
+      run_panels<0, 0>("256 tokens, 64x64 tiles", buf, 64, 4, 3 << 19, ncopies, sink);
+      run_panels<1, 2>("256 tokens, 64x64 tiles, quarter touch 2 steps ahead", buf, 64, 4, 3 << 19, ncopies, sink);
+      run_panels<1, 6>("256 tokens, 64x64 tiles, quarter touch 6 steps ahead", buf, 64, 4, 3 << 19, ncopies, sink);
+      // 1024 tokens, 128 x 128 tiles: 32 panels of 128 features (3 MB), eight token tiles of 128 tokens (3 MB each)
+      run_panels<0, 0>("1024 tokens, 128x128 tiles", buf, 32, 8, 3 << 20, ncopies, sink);
+      // and with the row-major addresses of the operands themselves
+      run_panel_rows<64>("256 tokens, 64x64 tiles, row-major operands", buf, 4, ncopies, sink);
+      run_panel_rows<128>("1024 tokens, 128x128 tiles, row-major operands", buf, 8, ncopies, sink);
+    }
   }
-  printf("== 4. 256 rows x 128 bytes per step out of the L2, by the distance between rows\n");
-  for (int nwg : {8, 256}) {
-    run_rows("rows back to back (8 KB each)", buf, 8192, 64, nwg, sink);
-    run_rows("rows of K = 12288 bf16", buf, 24576, 64, nwg, sink);
-    run_rows("rows of V = 151936 bf16", buf, 303872, 64, nwg, sink);
-    run_rows("rows 1 MB apart", buf, 1 << 20, 64, nwg, sink);
+  if (want(4)) {
+    printf("== 4. 256 rows x 128 bytes per step out of the L2, by the distance between rows\n");
+    for (int nwg : {8, 256}) {
+      run_rows("rows back to back (8 KB each)", buf, 8192, 64, nwg, sink);
+      run_rows("rows of K = 12288 bf16", buf, 24576, 64, nwg, sink);
+      run_rows("rows of V = 151936 bf16", buf, 303872, 64, nwg, sink);
+      run_rows("rows 1 MB apart", buf, 1 << 20, 64, nwg, sink);
+    }
   }
-  printf("== 5. load side of the 256 x 256 tile GEMM at the headline shape, no arithmetic\n");
-  run_big_tile(buf, sink);
-  printf("== 6. the matrix pipe alone: the MFMA sequence of the 256 x 256 tile kernel out of registers\n");
-  run_mfma_only(buf, sink);
-  printf("== 7. the same sequence with the kernel's LDS reads, L2 loads and barriers added one after the other\n");
-  run_traffic_cost(buf, scratch);
+  if (want(5)) {
+    printf("== 5. load side of the 256 x 256 tile GEMM at the headline shape, no arithmetic\n");
+    run_big_tile(buf, sink);
+  }
+  if (want(6)) {
+    printf("== 6. the matrix pipe alone: the MFMA sequence of the 256 x 256 tile kernel out of registers\n");
+    run_mfma_only(buf, sink);
+  }
+  if (want(7)) {
+    printf("== 7. the same sequence with the kernel's LDS reads, L2 loads and barriers added one after the other\n");
+    run_traffic_cost(buf, scratch);
+  }
   return 0;
 }
