@@ -80,6 +80,9 @@ def _matrix_pipe_alone() -> dict | None:
     probe = ROOT / "rl-kernel_amd" / "load_path_probe"
     if not probe.exists():
         return None
+    # under a profiler the child would be traced as well, and the profiler has already initialised the GPU
+    if "rocprof" in os.environ.get("LD_PRELOAD", "").lower() or any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ):
+        return None
     try:
         done = subprocess.run([str(probe), "6"], stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True, timeout=120)
     except (OSError, subprocess.SubprocessError):
