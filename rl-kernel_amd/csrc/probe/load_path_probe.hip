@@ -10,6 +10,7 @@
 //   5. the load side of the 256 x 256 tile GEMM at its headline shape
 //   6. the other side: the matrix pipe alone, the same MFMA sequence out of registers, at the power cap
 //   7. that sequence with the kernel's LDS reads, L2 loads and barriers added, and the shader clock each variant sees
+//   8. a K-major weight streamed as column slabs by one workgroup per slab (decode against a prepared weight)
 //
 // Loads are the direct-to-LDS DMA form the tile kernels use (or ordinary vector loads, "vgpr"). Build:
 //   hipcc --offload-arch=gfx950 -O3 -o load_path_probe load_path_probe.hip     (rl-kernel_amd/build.py does it)
@@ -556,7 +557,62 @@ static void run_traffic_cost(char* buf, char* sink_bytes) {
   }
 }
 
-// Without arguments every section runs; with a section number (1 .. 7) only that one.
+// ---- 8: column slabs of a K-major weight ------------------------------------------------------------------
+// Decode against a prepared weight B[K = 12288][N = 4096] (rows of 8 KiB): with no split-K a workgroup owns its
+// features for the whole reduction, i.e. it streams a column slab of `slab_bytes` per K row (128 bytes = 64 features:
+// 64 workgroups; 64 bytes: 128; 32 bytes: 256), 32 KiB per step, the previous step awaited. Copies of the weight
+// rotate, so it comes from HBM, or one copy is relaunched (memory-side cache).
+__global__ __launch_bounds__(512) void column_slab_kernel(const char* w, int slab_bytes, int nslabs, int krows, unsigned* sink) {
+  extern __shared__ __align__(1024) char lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const size_t row_bytes = (size_t)slab_bytes * nslabs;
+  const int lanes_per_row = slab_bytes / 16;      // 8, 4, 2
+  const int rows_per_instr = 64 / lanes_per_row;  // 8, 16, 32
+  const int rows_per_step = 8 * 4 * rows_per_instr;
+  const char* mine = w + (size_t)blockIdx.x * slab_bytes + (size_t)(lane / lanes_per_row) * row_bytes + (lane % lanes_per_row) * 16;
+  char* dst = lds + wave * 8192;
+  const int steps = krows / rows_per_step;
+  for (int s = 0; s < steps; ++s) {
+    const char* src = mine + (size_t)(s * rows_per_step + wave * 4 * rows_per_instr) * row_bytes;
+    char* d = dst + (s & 1) * 4096;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(src + (size_t)(u * rows_per_instr) * row_bytes), (lds_ptr_t)(d + u * 1024), 16, 0, 0);
+    __builtin_amdgcn_s_waitcnt(kWaitAllVm | 4);
+  }
+  __builtin_amdgcn_s_waitcnt(kWaitAllVm);
+  __syncthreads();
+  const unsigned acc = *(unsigned*)(lds + threadIdx.x * 4);
+  if (acc == 0x12345678u) sink[0] = acc;
+}
+
+static void run_column_slabs(const char* buf, int slab_bytes, int ncopies, unsigned* sink) {
+  const int krows = 12288, row_bytes = 8192, nslabs = row_bytes / slab_bytes, lds = 65536;
+  const size_t copy_bytes = (size_t)krows * row_bytes;
+  require(slab_bytes == 128 || slab_bytes == 64 || slab_bytes == 32, "slab width");
+  require((size_t)ncopies * copy_bytes <= g_buffer_bytes, "copies exceed the buffer");
+  CK(hipFuncSetAttribute((const void*)column_slab_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+  hipEvent_t a, b;
+  CK(hipEventCreate(&a));
+  CK(hipEventCreate(&b));
+  int c = 0;
+  for (int i = 0; i < 5; ++i, c = (c + 1) % ncopies)
+    column_slab_kernel<<<nslabs, 512, lds>>>(buf + (size_t)c * copy_bytes, slab_bytes, nslabs, krows, sink);
+  CK(hipEventRecord(a));
+  const int reps = 40;
+  for (int i = 0; i < reps; ++i, c = (c + 1) % ncopies)
+    column_slab_kernel<<<nslabs, 512, lds>>>(buf + (size_t)c * copy_bytes, slab_bytes, nslabs, krows, sink);
+  CK(hipEventRecord(b));
+  CK(hipEventSynchronize(b));
+  float ms;
+  CK(hipEventElapsedTime(&ms, a, b));
+  ms /= reps;
+  printf("slabs of %3d bytes per K row, %3d workgroups, weight %s: %6.1f us  %5.2f TB/s\n", slab_bytes, nslabs,
+         ncopies == 1 ? "relaunched (memory-side cache)" : "rotating (from HBM)          ", ms * 1e3, copy_bytes / ms * 1e-9);
+  fflush(stdout);
+}
+
+// Without arguments every section runs; with a section number (1 .. 8) only that one.
 int main(int argc, char** argv) {
   const int only = argc > 1 ? atoi(argv[1]) : 0;
   auto want = [&](int section) { return only == 0 || only == section; };
@@ -633,6 +689,11 @@ int main(int argc, char** argv) {
   if (want(7)) {
     printf("== 7. the same sequence with the kernel's LDS reads, L2 loads and barriers added one after the other\n");
     run_traffic_cost(buf, scratch);
+  }
+  if (want(8)) {
+    printf("== 8. a K-major weight [12288][4096] streamed as column slabs, one workgroup per slab (decode against a prepared weight)\n");
+    for (int ncopies : {1, 14})
+      for (int slab : {128, 64, 32}) run_column_slabs(buf, slab, ncopies, sink);
   }
   return 0;
 }
