@@ -7,11 +7,10 @@ H[4096,12288] x W[4096,12288]^T, inputs resident in HBM. The JSON line also carr
 
 * ``roofline``     - the dominant kernel (the 256x256-tile MFMA kernel on gate_up)
                      against the MI355X dense bf16 MFMA peak, timed with HIP events
-                     on the launch stream; ``roofline.matrix_pipe_alone`` adds, for orientation,
-                     what the same MFMA sequence sustains on this machine out of registers with
-                     nothing else running (random and zero operands; ``rl-kernel_amd/load_path_probe 6``,
-                     a child process started before this one touches the GPU);
-* ``cpu_baseline`` - the CPU oracle (``oracle/reference_math.det_gemm_ref``) timed on
+                     on the launch stream; ``roofline.matrix_pipe_alone`` quotes, for orientation,
+                     what the same MFMA sequence sustained out of registers with nothing else
+                     running on machines of this pool (recorded constants, not measured here);
+* ``cpu_baseline`` - the CPU oracle (``oracle/reference_math.det_gemm_ref_torch``) timed on
                      this box's host cores on the same step;
 * ``shapes``       - every token count of the configuration (T = 1, 16, 64, 256, 1024, 4096)
                      with its own MFMA or HBM fraction; up to 1024 tokens also over copies of
@@ -70,27 +69,15 @@ def _measured_traffic() -> dict:
     return out
 
 
-def _matrix_pipe_alone() -> dict | None:
-    """What the matrix pipe sustains at the power cap when nothing else runs: the MFMA sequence of the 256 x 256 tile
-    kernel out of registers, on random and on zero operands (section 6 of rl-kernel_amd/load_path_probe, a program of
-    its own, run as a child process before this process touches the GPU). None when the program is missing or fails."""
-    import re
-    import subprocess
-
-    probe = ROOT / "rl-kernel_amd" / "load_path_probe"
-    if not probe.exists():
-        return None
-    # under a profiler the child would be traced as well, and the profiler has already initialised the GPU
-    if "rocprof" in os.environ.get("LD_PRELOAD", "").lower() or any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ):
-        return None
-    try:
-        done = subprocess.run([str(probe), "6"], stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True, timeout=120)
-    except (OSError, subprocess.SubprocessError):
-        return None
-    found = {}
-    for kind, value in re.findall(r"matrix pipe only, (random|zero)\s+operands:.*?=\s*([0-9.]+) TFLOP/s", done.stdout):
-        found[f"{kind}_operands_tflops"] = float(value)
-    return found if done.returncode == 0 and len(found) == 2 else None
+# What the matrix pipe sustains at the power cap when nothing else runs: the MFMA sequence of the 256 x 256 tile
+# kernel out of registers (no loads, no LDS), measured once with a stand-alone probe on machines of this pool
+# (profiles/load_path_probe_mi355x.md, section 6). Constants, not measured by this run: the spread is the spread
+# between machines.
+MATRIX_PIPE_ALONE = {
+    "random_operands_tflops": [1970.0, 2130.0],
+    "zero_operands_tflops": [2440.0, 2450.0],
+    "source": "profiles/load_path_probe_mi355x.md section 6",
+}
 
 
 def _parse():
@@ -154,9 +141,6 @@ def main() -> int:
             file=sys.stderr,
         )
         return 2
-
-    # a child process; it has to start before this process initialises the GPU
-    matrix_pipe_alone = _matrix_pipe_alone() if args.only == "" else None
 
     import torch
 
@@ -420,10 +404,10 @@ def main() -> int:
         "traffic_measured_on_commit": traffic["commit"],
     }
     roofline.update(_launch_percentiles(gate_up, args.steps, 5))
-    if matrix_pipe_alone is not None:
-        # orientation: the matrix pipe with nothing else running, same MFMA sequence, at the power cap of this machine
-        roofline["matrix_pipe_alone"] = dict(
-            matrix_pipe_alone, frac_of_random_operands_rate=round(achieved / matrix_pipe_alone["random_operands_tflops"], 4))
+    # orientation: the matrix pipe with nothing else running, same MFMA sequence, at the power cap (recorded range)
+    lo, hi = MATRIX_PIPE_ALONE["random_operands_tflops"]
+    roofline["matrix_pipe_alone"] = dict(
+        MATRIX_PIPE_ALONE, frac_of_random_operands_rate=[round(achieved / hi, 4), round(achieved / lo, 4)])
 
     result = {
         "metric": "bf16 det-GEMM TFLOP/s at Qwen3-8B FFN shapes (gate_up + down, T=4096)",
@@ -705,50 +689,58 @@ def main() -> int:
             "tokens_per_s": round(T / ms_ffn * 1e3, 1),
         }
 
-    # ---- CPU baseline: the oracle on the same step, on this box's host cores
+    # ---- CPU baseline: the oracle's torch forms (the reference's own CPU expressions) on the same step, on this
+    # box's host cores
     if not args.no_cpu:
         import numpy as np
 
-        import inputs
         from oracle import reference_math as oracle
 
-        try:
-            from threadpoolctl import threadpool_info
-
-            blas_threads = max([p.get("num_threads", 1) for p in threadpool_info() if p.get("user_api") == "blas"] or [1])
-        except Exception:
-            blas_threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-        xb, hb = inputs.bits(x), inputs.bits(h)
-        wgb, wdb = inputs.bits(w_gu), inputs.bits(w_d)
+        torch.set_num_threads(int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+        threads = torch.get_num_threads()
+        cpu_model = oracle.cpu_model_string()
+        xc, hc, wgc, wdc = x.cpu(), h.cpu(), w_gu.cpu(), w_d.cpu()
+        oracle.det_gemm_ref_torch(xc[:256], wgc)  # warm-up: thread pool, allocator
         times = []
         while len(times) < 3 or sum(times) < 10.0:  # about 10 s of host work, at least three runs
             t0 = time.perf_counter()
-            oracle.det_gemm_ref(xb, wgb)
-            oracle.det_gemm_ref(hb, wdb)
+            oracle.det_gemm_ref_torch(xc, wgc)
+            oracle.det_gemm_ref_torch(hc, wdc)
             times.append(time.perf_counter() - t0)
             if sum(times) > 30:
                 break
         cpu_s = float(np.median(times))
+        t0 = time.perf_counter()
+        oracle.native_gemm_torch(xc, wgc)
+        oracle.native_gemm_torch(hc, wdc)
+        native_s = time.perf_counter() - t0
         result["cpu_baseline"] = {
             "value": round((flops_gu + flops_d) / cpu_s * 1e-12, 4),
             "unit": "TFLOP/s",
-            "cores": int(blas_threads),
+            "cores": int(threads),
             "kind": "port",
+            "cpu_model": cpu_model,
+            "torch_num_threads": int(threads),
+            "torch_version": torch.__version__,
             "sample": f"the full step (gate_up + down at T=4096, {(flops_gu + flops_d) / 1e9:.0f} GFLOP), "
-            f"median of {len(times)} runs of oracle.det_gemm_ref (fp32 upcast, numpy sgemm, one bf16 rounding), {cpu_s:.2f} s each",
+            f"median of {len(times)} runs of oracle.det_gemm_ref_torch ((a.float() @ b.float()).to(bf16)), {cpu_s:.2f} s each",
+            "native_bf16_matmul": {"value": round((flops_gu + flops_d) / native_s * 1e-12, 4), "unit": "TFLOP/s",
+                                   "sample": f"one run of torch.matmul on the bf16 tensors (NativeGemmOp), {native_s:.2f} s"},
         }
+        del xc, hc, wgc, wdc
         if not args.no_logp:
-            ts = 8192  # the whole workload once: several seconds of host work on 16 threads
-            hb2, wb2 = inputs.bits(hid[:ts]), inputs.bits(w_lm)
+            ts = 8192  # the whole workload once: several seconds of host work
             t0 = time.perf_counter()
-            oracle.linear_logp_chunked(hb2, wb2, tgt[:ts].cpu().numpy(), chunk_elems=ts * 2048)
+            oracle.linear_logp_chunked_torch(hid[:ts].cpu(), w_lm.cpu(), tgt[:ts].cpu(), chunk_elems=ts * 2048)
             cpu_lp = time.perf_counter() - t0
             result["linear_logp"]["cpu_baseline"] = {
                 "value": round(ts / cpu_lp, 1),
                 "unit": "tokens/s",
-                "cores": int(blas_threads),
+                "cores": int(threads),
                 "kind": "port",
-                "sample": f"all {ts} tokens once, oracle.linear_logp_chunked (2048-row vocabulary chunks), {cpu_lp:.2f} s",
+                "cpu_model": cpu_model,
+                "torch_num_threads": int(threads),
+                "sample": f"all {ts} tokens once, oracle.linear_logp_chunked_torch (2048-row vocabulary chunks), {cpu_lp:.2f} s",
             }
 
     print(json.dumps(result))

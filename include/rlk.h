@@ -184,9 +184,13 @@ size_t rlk_linear_logp_workspace_bytes(int T, int V);
  *   lse     [T] fp32 out (may be NULL)
  *   real_vocab_end: local column bound of the real vocabulary (columns >= it are
  *                   padding and contribute -inf / 0); pass V for "no padding".
- * A target outside [vocab_start, vocab_start + real_vocab_end) contributes a target
- * logit of 0 (range checking is the caller's job, as in the reference's Python
- * layer, linear_logp.py:664-672). The full [T, V] logits are never written.
+ * A target outside [vocab_start, vocab_start + real_vocab_end) names no column of this
+ * call: that row's logp is NaN (its lse is unaffected), so a caller that does not check
+ * the range on the host beforehand (the reference's Python layer does, with a device
+ * read-back, linear_logp.py:664-672) still sees the mistake in the result; likewise a
+ * temperature that is not a positive number makes the row's logp and lse NaN.
+ * rlk_linear_logp_fwd_shard, whose targets may belong to another shard, writes a target
+ * logit of 0 for them instead. The full [T, V] logits are never written.
  *
  * Stands in for rl_engine._C.fused_linear_logp_sm90 (csrc/bindings/ops.cpp:514-526;
  * csrc/cuda/logprob/fused_linear_logp_sm90.cu:2040-2176), for
@@ -284,6 +288,9 @@ size_t rlk_linear_logp_bwd_workspace_bytes(int T, int V, int with_bias);
  * 256-token blocks, blocks added ascending. The clamp
  * logp = min(., 0) of the forward is not differentiated (gradient 1), as in the reference.
  * workspace must be 256-byte aligned.
+ * grad_hidden is also scratch during the call: from 512 tokens on (T % 8 == 0, gh_row_stride == D,
+ * 16-byte aligned) it first holds the transposed hidden states that the weight-gradient GEMM reads,
+ * and receives its result last. It must not alias hidden, weight, or any other argument.
  *
  * Stands in for _DetTritonLinearLogpAutograd.backward and _det_reference_dlogits
  * (rl_engine/backends/shared/triton/logprob/linear_logp.py:522-570, 600-628) and for

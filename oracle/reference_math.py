@@ -41,6 +41,9 @@ Pinning (which check fixes which function; see tests/test_oracle.py):
   tests/ops/loss/test_grpo_loss.py:112-119) and closed forms (old == logp gives
   ratio 1, ref == logp gives k3 0, clip saturation).
 
+* ``det_gemm_ref_torch`` / ``native_gemm_torch`` / ``linear_logp_chunked_torch`` (the torch forms the CPU baseline
+  times): against the numpy forms on seeded inputs (tests/test_oracle.py).
+
 No function here is "parity unpinned".
 """
 
@@ -232,6 +235,64 @@ def bf16_ulp_distance(x_bits: np.ndarray, y_bits: np.ndarray) -> np.ndarray:
         return np.where(b & 0x8000, -(b & 0x7FFF), b & 0x7FFF)
 
     return np.abs(ordered(np.asarray(x_bits)) - ordered(np.asarray(y_bits)))
+
+
+# ---------------------------------------------------------------------------
+# The same two paths written with torch on the CPU, the way the reference itself writes them. They exist for
+# the CPU baseline (timed on the host cores next to the GPU) and are pinned against the numpy forms above.
+# ---------------------------------------------------------------------------
+
+
+def cpu_model_string() -> str:
+    """The host CPU's model name (first ``model name`` line of /proc/cpuinfo), or ``"unknown"``."""
+    try:
+        for line in Path("/proc/cpuinfo").read_text().splitlines():
+            if line.lower().startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def det_gemm_ref_torch(a, bt):
+    """``(a.float() @ b.float()).to(torch.bfloat16)`` on CPU bf16 tensors ``a[M,K]``, ``bt[N,K]`` (the native linear
+    weight, b = bt.t()): NativeMatmulOp, rl_engine/reference/embedding/matmul.py:22-28."""
+    import torch
+
+    return (a.float() @ bt.float().t()).to(torch.bfloat16)
+
+
+def native_gemm_torch(a, bt):
+    """``torch.matmul(a, b)`` on the bf16 tensors themselves: NativeGemmOp, rl_engine/reference/gemm/det_gemm.py:15-23.
+    Its summation order (and whether partial sums are rounded to bf16) is the CPU BLAS's own."""
+    import torch
+
+    return torch.matmul(a, bt.t())
+
+
+def linear_logp_chunked_torch(h, w, target, *, chunk_elems: int = 1 << 24):
+    """_chunked_local_linear_logp_stats (rl_engine/reference/logprob/linear_logp.py:259-308) in torch on CPU tensors:
+    the recurrence of ``linear_logp_chunked`` above, operands upcast to fp32 (:31-36). Returns ``(logp, lse)``."""
+    import torch
+
+    h32, n, v = h.float(), h.shape[0], w.shape[0]
+    target = target.long().reshape(-1)
+    local_max = torch.full((n,), float("-inf"))
+    local_sum = torch.zeros((n,))
+    target_logit = torch.zeros((n,))
+    rows = torch.arange(n)
+    chunk = max(1, min(v, chunk_elems // max(n, 1)))
+    for v0 in range(0, v, chunk):
+        v1 = min(v0 + chunk, v)
+        logits = h32 @ w[v0:v1].float().t()
+        new_max = torch.maximum(local_max, logits.max(dim=-1).values)
+        local_sum = local_sum * torch.exp(local_max - new_max) + torch.exp(logits - new_max[:, None]).sum(dim=-1)
+        local_max = new_max
+        owns = (target >= v0) & (target < v1)
+        safe = (target - v0).clamp(0, v1 - v0 - 1)
+        target_logit = torch.where(owns, logits[rows, safe], target_logit)
+    lse = local_max + torch.log(local_sum)
+    return target_logit - lse, lse
 
 
 # ---------------------------------------------------------------------------

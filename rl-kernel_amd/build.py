@@ -1,4 +1,4 @@
-"""Build librlk_gfx950.so (the C-ABI HIP library) and the load-path probe (a diagnostic executable) in-tree with hipcc.
+"""Build librlk_gfx950.so (the C-ABI HIP library) in-tree with hipcc.
 
 Usage: python rl-kernel_amd/build.py            (or __graft_entry__.build())
 """
@@ -15,8 +15,6 @@ PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "librlk_gfx950.so"
 OBJ_DIR = PKG_DIR / "build"  # object files (git-ignored)
-PROBE_SRC = CSRC / "probe" / "load_path_probe.hip"  # a stand-alone diagnostic, not part of the library
-PROBE_PATH = PKG_DIR / "load_path_probe"
 SOURCES = ["det_gemm.hip", "det_gemm_stream.hip", "det_gemm_shortk.hip", "det_gemm_tree.hip", "det_gemm_seq.hip", "linear_logp.hip",
     "linear_logp_bwd.hip", "logits_logp.hip", "swiglu.hip", "grpo.hip", "rlk_api.hip"]
 
@@ -56,16 +54,20 @@ def _run(cmd: list[str]) -> str:
 def build(verbose: bool = True, only: list[str] | None = None) -> Path:
     """Compile every HIP source for gfx950 (one hipcc per source, side by side) and link them into
     one shared library. `only` names the sources to recompile; the objects of the others are reused
-    when they exist (a developer's shortcut, the default recompiles everything)."""
+    when they exist and are newer than every header under csrc/ and include/ (a developer's
+    shortcut, the default recompiles everything)."""
     from concurrent.futures import ThreadPoolExecutor
 
     hipcc = find_hipcc()
     OBJ_DIR.mkdir(exist_ok=True)
     compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    headers = [*CSRC.glob("*.h"), *(PKG_DIR.parent / "include").glob("*.h")]
+    newest_header = max((h.stat().st_mtime for h in headers), default=0.0)
     jobs = []
     for src in SOURCES:
         obj = OBJ_DIR / (src + ".o")
-        if only is not None and src not in only and obj.exists():
+        fresh = obj.exists() and obj.stat().st_mtime > max(newest_header, (CSRC / src).stat().st_mtime)
+        if only is not None and src not in only and fresh:
             continue
         jobs.append([hipcc, *compile_flags, "-c", "-o", str(obj), str(CSRC / src)])
     if verbose:
@@ -79,11 +81,6 @@ def build(verbose: bool = True, only: list[str] | None = None) -> Path:
     if verbose:
         print("[rlk build]", " ".join(link), flush=True)
     outs.append(_run(link))
-    if only is None or PROBE_SRC.name in only:
-        probe = [hipcc, *[f for f in compile_flags if f != "-fPIC"], "-o", str(PROBE_PATH), str(PROBE_SRC)]
-        if verbose:
-            print("[rlk build]", " ".join(probe), flush=True)
-        outs.append(_run(probe))
     if verbose:
         for out in outs:
             if out:

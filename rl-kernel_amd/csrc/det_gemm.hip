@@ -375,8 +375,83 @@ static int64_t tile_count(int M, int N, int bm, int bn) {
   return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
 }
 
+int device_cu_count() {
+  static std::atomic<int> cached[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  const bool tracked = dev >= 0 && dev < kMaxDevices;
+  if (tracked) {
+    const int have = cached[dev].load(std::memory_order_relaxed);
+    if (have > 0) return have;
+  }
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, dev) != hipSuccess || prop.multiProcessorCount <= 0) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  if (tracked) cached[dev].store(prop.multiProcessorCount, std::memory_order_relaxed);
+  return prop.multiProcessorCount;
+}
+
+// Every tile shape the automatic choice weighs, in one table. `native` is the relative throughput of the shape on a
+// full chip with both operands in the native (reduction-contiguous) layout, `w_kmajor` the same with a K-major weight
+// (0: the shape has no such loop); `x_kmajor` says whether the shape also takes a K-major activation operand. The
+// estimated time of a launch is rounds_of_workgroups(tiles) x tile area / quality; larger tiles win ties.
+//
+// Native column, fitted to sweeps over the Qwen3-8B projection shapes at 384 ... 6144 tokens: 192 x 256 (three
+// quarters of the large tile at 0.89 of its throughput) fills the rounds that N / 256 leaves half empty - gate_up at
+// 1024 tokens is 512 tiles = two full rounds instead of 384 = one and a half (169 -> 152 us), qkv at 3072 tokens
+// 150 -> 128 us. Where 192 does not divide N its last feature tile is partly empty and the shape counts as
+// `ragged192`: it still wins where it turns a round and a fraction into less (N = 5120 at 4096 tokens 293 -> 256 us,
+// N = 10240 at 2048 tokens 190 -> 162 us) and loses the tie against 256 x 128 at N = 4096, 2048 tokens. 192 x 128
+// (three stages) does the same one size down (weights from HBM: gate_up at 256 tokens 65.0 -> 62.2 us, N = 6144 at 768
+// tokens 55.1 -> 49.1 us).
+// K-major-weight column (`dY @ W`, `a @ b`, prepared weights): the 64- and 128-feature tiles give a long reduction
+// against few output tiles - grad_hidden of the LogP backward up to about a thousand tokens (N = 4096, K = 151936) - a
+// workgroup per CU, each streaming a narrow slice of the weight instead of a 256-column one (1.9 -> 0.8 ms at 256
+// tokens, 1.8 -> 1.03 ms at 512, 1.65 -> 1.45 ms at 1024); their qualities are those of the direct-to-LDS loop.
+struct TileCandidate {
+  int config, bn, bm;
+  double native, ragged192, w_kmajor;
+  bool x_kmajor;
+};
+static const TileCandidate kTileCandidates[] = {
+    {RLK_GEMM_CFG_256x256, 256, 256, 1.00, 0.00, 1.00, true},  {RLK_GEMM_CFG_192x256, 192, 256, 0.89, 0.85, 0.00, false},
+    {RLK_GEMM_CFG_256x128, 256, 128, 0.65, 0.00, 0.70, true},  {RLK_GEMM_CFG_192x128, 192, 128, 0.56, 0.53, 0.00, false},
+    {RLK_GEMM_CFG_256x64, 256, 64, 0.50, 0.00, 0.56, false},   {RLK_GEMM_CFG_128x128, 128, 128, 0.65, 0.00, 0.62, false},
+    {RLK_GEMM_CFG_128x64, 128, 64, 0.45, 0.00, 0.40, false},   {RLK_GEMM_CFG_64x64, 64, 64, 0.42, 0.00, 0.25, false},
+};
+
+// The cheapest candidate by the estimate above. `w_kmajor` / `x_kmajor`: the operand layouts of the call.
+static int pick_tile_candidate(int M, int N, int K, bool w_kmajor, bool x_kmajor) {
+  const int cus = device_cu_count();
+  int best = RLK_GEMM_CFG_64x64;
+  double best_time = 1e300;
+  for (const TileCandidate& c : kTileCandidates) {
+    double quality;
+    if (w_kmajor || x_kmajor) {
+      if (c.w_kmajor == 0.0 || (x_kmajor && !c.x_kmajor)) continue;
+      if (c.bn <= 128 && !w_kmajor) continue;  // the small K-major tiles exist for a K-major weight only
+      quality = c.w_kmajor;
+    } else {
+      const bool wide192 = c.ragged192 != 0.0;
+      if (wide192 && K % kTileK != 0) continue;
+      quality = (wide192 && N % 192 != 0) ? c.ragged192 : c.native;
+    }
+    const double t = rounds_of_workgroups(tile_count(M, N, c.bm, c.bn), cus) * (double)(c.bn * c.bm) / quality;
+    if (t < best_time * 0.999) {
+      best_time = t;
+      best = c.config;
+    }
+  }
+  return best;
+}
+
 int pick_det_gemm_config(int M, int N, int K) {
-  constexpr int kCus = 256;
+  const int cus = device_cu_count();
   // Decode (weights fitted while they rotate through 1.3 GB, i.e. come from HBM as in a model with
   // many layers, not from the 256 MB memory-side cache): up to 16 tokens the streaming kernel with
   // two workgroups per CU is the fastest or equal for every Qwen3-8B projection (gate_up 52 -> 38 us,
@@ -384,58 +459,17 @@ int pick_det_gemm_config(int M, int N, int K) {
   // resident). Up to 32 / 64 tokens it holds while there are at most 1.5 / 1 panels per CU: a
   // 64-token tile kernel would run on N / 64 CUs only.
   if (M <= 16) return (K >= 1024 && K % kTileK == 0) ? RLK_GEMM_CFG_STREAM16 : RLK_GEMM_CFG_16x16;
-  if (K >= 1024 && K % kTileK == 0 && ((M <= 32 && N <= 24 * kCus) || (M <= 64 && N <= 16 * kCus)))
+  if (K >= 1024 && K % kTileK == 0 && ((M <= 32 && N <= 24 * cus) || (M <= 64 && N <= 16 * cus)))
     return RLK_GEMM_CFG_STREAM64;
   // Problems that give the chip at most one small tile per CU: the deep-stage variants
   // (one workgroup per CU, several K tiles per barrier pair) beat the same tile run several
   // workgroups per CU. Smallest tile first: it spreads the weight stream over most CUs.
-  if (K % (kTileK * kDeep64) == 0 && tile_count(M, N, 64, 64) <= kCus) return RLK_GEMM_CFG_64x64_DEEP;
+  if (K % (kTileK * kDeep64) == 0 && tile_count(M, N, 64, 64) <= cus) return RLK_GEMM_CFG_64x64_DEEP;
   if (K % (kTileK * kDeep128) == 0) {
-    if (tile_count(M, N, 64, 128) <= kCus) return RLK_GEMM_CFG_128x64_DEEP;
-    if (tile_count(M, N, 128, 128) <= kCus) return RLK_GEMM_CFG_128x128_DEEP;
+    if (tile_count(M, N, 64, 128) <= cus) return RLK_GEMM_CFG_128x64_DEEP;
+    if (tile_count(M, N, 128, 128) <= cus) return RLK_GEMM_CFG_128x128_DEEP;
   }
-  // Estimated time = (rounds of 256 workgroups) x (tile area / relative throughput of the
-  // shape when the chip is full), fitted to sweeps over the Qwen3-8B projection shapes at
-  // 384 ... 6144 tokens. A last, partly filled round is nearly free beyond its own share: the
-  // chip is power limited, and a round that keeps fewer CUs busy runs at a higher clock, so
-  // the 256 x 256 tile wins unless its tiles cover well under one round. Larger tiles win ties.
-  struct Candidate {
-    int config, bn, bm;
-    double quality;
-  };
-  // 192 x 256 (three quarters of the large tile at 0.89 of its throughput) fills the rounds that
-  // N / 256 leaves half empty: gate_up at 1024 tokens is 512 tiles = two full rounds instead of
-  // 384 = one and a half (169 -> 152 us), qkv at 3072 tokens 150 -> 128 us. Where 192 does not divide N the
-  // last feature tile is partly empty and the shape counts as 0.85: it still wins where it turns a round and a
-  // fraction into less (N = 5120 at 4096 tokens 293 -> 256 us, N = 10240 at 2048 tokens 190 -> 162 us, N = 2560 at
-  // 8192 tokens 347 -> 308 us) and loses the tie against 256 x 128 at N = 4096, 2048 tokens (177 against 166 us).
-  // 192 x 128 (three stages) does the same one size down: N / 192 x M / 128 tiles fill a round that 256 x 128 leaves a
-  // quarter empty (weights from HBM: gate_up at 256 tokens 65.0 -> 62.2 us, N = 12288 at 384 tokens 58.4 -> 53.2,
-  // N = 6144 at 768 tokens 55.1 -> 49.1, N = 5120 at 1024 tokens 72.7 -> 63.5).
-  static const Candidate kCandidates[] = {
-      {RLK_GEMM_CFG_256x256, 256, 256, 1.00}, {RLK_GEMM_CFG_192x256, 192, 256, 0.89},
-      {RLK_GEMM_CFG_256x128, 256, 128, 0.65}, {RLK_GEMM_CFG_192x128, 192, 128, 0.56},
-      {RLK_GEMM_CFG_256x64, 256, 64, 0.50},
-      {RLK_GEMM_CFG_128x128, 128, 128, 0.65}, {RLK_GEMM_CFG_128x64, 128, 64, 0.45},
-      {RLK_GEMM_CFG_64x64, 64, 64, 0.42},
-  };
-  int best = RLK_GEMM_CFG_64x64;
-  double best_time = 1e300;
-  for (const Candidate& c : kCandidates) {
-    const bool wide192 = c.config == RLK_GEMM_CFG_192x256 || c.config == RLK_GEMM_CFG_192x128;
-    if (wide192 && K % kTileK != 0) continue;
-    const double quality = (wide192 && N % 192 != 0) ? (c.config == RLK_GEMM_CFG_192x256 ? 0.85 : 0.53) : c.quality;
-    const int64_t tiles = tile_count(M, N, c.bm, c.bn);
-    const int64_t full = tiles / kCus;
-    const double part = (double)(tiles - full * kCus) / kCus;
-    const double rounds = (double)full + (part > 0.0 ? (part > 0.9 ? part : 0.9) : 0.0);
-    const double t = rounds * (double)(c.bn * c.bm) / quality;
-    if (t < best_time * 0.999) {
-      best_time = t;
-      best = c.config;
-    }
-  }
-  return best;
+  return pick_tile_candidate(M, N, K, false, false);
 }
 
 // A K-major view (element [row, k] at ptr[k * k_stride + row], rows contiguous: B[K,N] as the
@@ -453,9 +487,10 @@ static bool view_is_kmajor_fast(const MatView& v) {
 // whether that pays: the round the remainder opens, priced at 11 + 21 K / 1024 us for a 256 x 256 tile
 // (measured on gate_up across K), against the few-token launch, which streams the weight once.
 static bool remainder_launch_pays(int M, int N, int K, int rest, bool fast_few_tokens, bool w_kmajor) {
+  const int64_t cus = device_cu_count();
   const int64_t feature_tiles = (N + 255) / 256;
-  const int64_t rounds_all = (feature_tiles * ((M + 255) / 256) + 255) / 256;
-  const int64_t rounds_main = (feature_tiles * (M / 256) + 255) / 256;
+  const int64_t rounds_all = (feature_tiles * ((M + 255) / 256) + cus - 1) / cus;
+  const int64_t rounds_main = (feature_tiles * (M / 256) + cus - 1) / cus;
   if (rounds_all == rounds_main) return false;  // the remainder's tiles fit beside the last round
   const double round_us = 11.0 + 21.0 * K / 1024.0;
   double rest_us;
@@ -510,38 +545,9 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
     const int loop = w_kmajor ? (x_kmajor ? kLoopPingPongBothKMajor : kLoopPingPongKMajor) : kLoopPingPongXKMajor;
     // Only the shapes with 64-feature wave columns have the transposing loop, and a K-major
     // activation needs at least 128 tokens per tile.
-    if (config == RLK_GEMM_CFG_AUTO) {
-      // The same estimate as pick_det_gemm_config over the three shapes that have the loop: rounds of
-      // 256 workgroups (a partly filled one costs at least 0.9) x tile area / relative throughput. With
-      // few token tiles against a long reduction (grad_hidden of the LogP backward at 1024 tokens:
-      // N = 4096, K = 151936) the 64-token tile doubles the workgroups (2.15 -> 2.0 ms: every
-      // workgroup of a feature tile still streams the whole 78 MB weight panel).
-      struct Shape {
-        int config, bn, bm;
-        double quality;
-      };
-      // The 64- and 128-feature tiles (K-major weight, native activations only) give a long
-      // reduction against few output tiles, e.g. grad_hidden of the LogP backward up to about a thousand
-      // tokens (N = 4096, K = 151936), a workgroup per CU: every workgroup then streams a narrow slice of the
-      // weight instead of a 256-column one (1.9 -> 0.8 ms at 256 tokens, 1.8 -> 1.03 ms at 512, 1.65 -> 1.45 ms
-      // at 1024). Their qualities are those of the direct-to-LDS loop (128 divides K).
-      const Shape shapes[] = {{RLK_GEMM_CFG_256x256, 256, 256, 1.00}, {RLK_GEMM_CFG_256x128, 256, 128, 0.70},
-                              {RLK_GEMM_CFG_256x64, 256, 64, 0.56},   {RLK_GEMM_CFG_128x128, 128, 128, 0.62},
-                              {RLK_GEMM_CFG_128x64, 128, 64, 0.40},   {RLK_GEMM_CFG_64x64, 64, 64, 0.25}};
-      double best = 1e300;
-      for (const Shape& c : shapes) {
-        if (c.config == RLK_GEMM_CFG_256x64 && x_kmajor) continue;
-        if (c.bn <= 128 && (x_kmajor || !w_kmajor)) continue;
-        const int64_t tiles = tile_count(M, N, c.bm, c.bn);
-        const int64_t full = tiles / 256;
-        const double part = (double)(tiles - full * 256) / 256.0;
-        const double t = ((double)full + (part > 0.0 ? (part > 0.9 ? part : 0.9) : 0.0)) * ((double)c.bn * c.bm) / c.quality;
-        if (t < best * 0.999) {
-          best = t;
-          config = c.config;
-        }
-      }
-    }
+    // With few token tiles against a long reduction (grad_hidden of the LogP backward at 1024 tokens: N = 4096,
+    // K = 151936) a smaller token tile doubles the workgroups, every one of which still streams its whole weight panel.
+    if (config == RLK_GEMM_CFG_AUTO) config = pick_tile_candidate(M, N, K, w_kmajor, x_kmajor);
     switch (config) {
       case RLK_GEMM_CFG_256x256:
         return launch_shape<Shape256x256>(W, X, C, ldc, M, N, K, false, loop, true, out_f32, stream);

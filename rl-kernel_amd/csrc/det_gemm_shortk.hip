@@ -229,7 +229,7 @@ bool det_gemm_shortk_supported(const MatView& W, const MatView& X, int M, int N,
 static int shortk_tiles_per_chunk(int M, int N, int per_cu) {
   const int n_blocks = (N + kShortKFeatures - 1) / kShortKFeatures;
   const int m_tiles = (M + kShortKTokens - 1) / kShortKTokens;
-  int chunks = (per_cu * 256 + n_blocks - 1) / n_blocks;
+  int chunks = (per_cu * device_cu_count() + n_blocks - 1) / n_blocks;
   chunks = (chunks + kShortKXcds - 1) / kShortKXcds * kShortKXcds;
   const int tiles = (m_tiles + chunks - 1) / chunks;
   return tiles < 1 ? 1 : tiles;

@@ -284,7 +284,10 @@ __global__ __launch_bounds__(kMergeThreads) void linear_logp_merge_kernel(const 
                                                                           float* __restrict__ logp,
                                                                           float* __restrict__ lse,
                                                                           float* __restrict__ target_logit, int T,
-                                                                          int n_split, bool clamp) {
+                                                                          int n_split, bool clamp,
+                                                                          const int64_t* __restrict__ target,
+                                                                          int64_t target_lo, int64_t target_hi,
+                                                                          const float* __restrict__ temperature) {
   __shared__ float red[kMergeLanes][kMergeTokens];
   __shared__ float terms[kMergeChunk][kMergeTokens];
   const int tk = threadIdx.x % kMergeTokens;
@@ -335,17 +338,29 @@ __global__ __launch_bounds__(kMergeThreads) void linear_logp_merge_kernel(const 
     __syncthreads();
   }
   if (sp == 0 && live) {
-    const float l = big + logf(sum);
+    float l = big + logf(sum);
+    // A temperature that is not a positive number scales nothing meaningful: both results of the row are NaN.
+    const bool bad_temperature = temperature != nullptr && !(temperature[m] > 0.f);
+    // A target id outside [target_lo, target_hi) names no column this call reduces over: the row's log-prob is
+    // NaN instead of a number made of a zero target logit (lse is that of the row all the same).
+    const bool bad_target = target != nullptr && (target[m] < target_lo || target[m] >= target_hi);
+    if (bad_temperature) l = __builtin_nanf("");
     if (lse) lse[m] = l;
-    if (logp) logp[m] = clamp ? fminf(zt - l, 0.f) : zt - l;
+    if (logp) {
+      float value = clamp ? fminf(zt - l, 0.f) : zt - l;
+      if (bad_temperature || bad_target) value = __builtin_nanf("");  // fminf would drop a NaN operand
+      logp[m] = value;
+    }
     if (target_logit) target_logit[m] = zt;
   }
 }
 
 hipError_t linear_logp_merge_launch(const float* part, float* logp, float* lse, float* target_logit, int T,
-                                    int n_split, bool clamp, hipStream_t stream) {
+                                    int n_split, bool clamp, hipStream_t stream, const int64_t* target,
+                                    int64_t target_lo, int64_t target_hi, const float* temperature) {
   hipLaunchKernelGGL(linear_logp_merge_kernel, dim3((T + kMergeTokens - 1) / kMergeTokens), dim3(kMergeThreads), 0,
-                     stream, part, logp, lse, target_logit, T, n_split, clamp);
+                     stream, part, logp, lse, target_logit, T, n_split, clamp, target, target_lo, target_hi,
+                     temperature);
   return hipGetLastError();
 }
 
@@ -407,7 +422,7 @@ static hipError_t launch_streamgroup_range(LogpArgs a, float* spart, int split_f
 // is not part of the contract.
 template <class S>
 static hipError_t launch_streamgroup(LogpArgs a, bool balance, hipStream_t stream) {
-  constexpr int kCus = 256;
+  const int kCus = device_cu_count();
   float* spart = a.part + (size_t)3 * a.n_split * a.T;  // behind the per-split partials
   const int tiles_m = (a.T + S::BM - 1) / S::BM;
   const int per_split = tiles_m * (kLogpStreams / 4);
@@ -510,7 +525,11 @@ hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t*
       return hipErrorInvalidValue;
   }
   if (err != hipSuccess) return err;
-  return linear_logp_merge_launch(workspace, logp, lse, target_logit, T, a.n_split, true, stream);
+  // The whole-vocabulary entries (those that write logp) mark rows whose target lies outside the real vocabulary;
+  // a shard's target logit is legitimately 0 for a target another shard owns.
+  return linear_logp_merge_launch(workspace, logp, lse, target_logit, T, a.n_split, true, stream,
+                                  logp != nullptr ? target : nullptr, vocab_start, vocab_start + vocab_limit,
+                                  temperature);
 }
 
 }  // namespace rlk

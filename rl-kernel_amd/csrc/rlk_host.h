@@ -31,6 +31,19 @@ inline hipError_t allow_dynamic_lds(const void* kernel, int bytes, PerDeviceOnce
   return err;
 }
 
+// Compute units of the current device (hipDeviceProp_t::multiProcessorCount, read once per device; 256 on an
+// MI355X, which is also the answer when no device can be asked).
+int device_cu_count();
+
+// What a launch of `tiles` equal workgroups costs in rounds of one workgroup per compute unit: the whole rounds plus
+// a last, partly filled one priced at max(0.9, its share) - the chip is power limited and a round that keeps fewer
+// compute units busy runs at a higher clock, so its cost is little more than its share, but never free.
+inline double rounds_of_workgroups(int64_t tiles, int cus) {
+  const int64_t full = tiles / cus;
+  const double part = (double)(tiles - full * cus) / cus;
+  return (double)full + (part > 0.0 ? (part > 0.9 ? part : 0.9) : 0.0);
+}
+
 int pick_det_gemm_config(int M, int N, int K);
 
 // W[N,K] is the operand whose rows are output features, X[M,K] the one whose
@@ -89,9 +102,12 @@ hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t*
 
 // Ascending merge of (max, sum, target logit) partials laid out [3][n_split][T] into
 // lse = M + log(S), logp = target - lse (clamped at 0 when `clamp`) and the merged target
-// logit itself (0 for a target no partial owns); each output may be null.
+// logit itself (0 for a target no partial owns); each output may be null. With `target` given, a row whose
+// target id lies outside [target_lo, target_hi) gets logp = NaN; with `temperature` given, a row whose
+// temperature is not a positive number gets logp = lse = NaN.
 hipError_t linear_logp_merge_launch(const float* part, float* logp, float* lse, float* target_logit, int T,
-                                    int n_split, bool clamp, hipStream_t stream);
+                                    int n_split, bool clamp, hipStream_t stream, const int64_t* target = nullptr,
+                                    int64_t target_lo = 0, int64_t target_hi = 0, const float* temperature = nullptr);
 
 // Per-row, per-tile (max, sum of exp relative to it[, target logit]) of materialised logits
 // of element type `dtype` (rlk_dtype); element (row, tile) of each output sits at

@@ -271,12 +271,11 @@ hipError_t det_gemm_swiglu_launch(const MatView& W, const MatView& X, void* Y, i
     if (streams_gated(M, K)) return det_gemm_stream_gated_launch(W, X, Y, ldy, M, I, K, stream);
     const int64_t t256 = (int64_t)((M + 255) / 256) * ((I + 127) / 128);
     const int64_t t128 = (int64_t)((M + 127) / 128) * ((I + 127) / 128);
-    // Rounds of 256 workgroups x tokens per tile / relative throughput, as in pick_det_gemm_config:
+    // Rounds of workgroups x tokens per tile / relative throughput, as in pick_det_gemm_config:
     // a partly filled last round costs little more than its share, so the large tile wins early.
-    auto cost = [](int64_t tiles, double tokens, double quality) {
-      const int64_t full = tiles / 256;
-      const double part = (double)(tiles - full * 256) / 256.0;
-      return ((double)full + (part > 0.0 ? (part > 0.9 ? part : 0.9) : 0.0)) * tokens / quality;
+    const int cus = device_cu_count();
+    auto cost = [cus](int64_t tiles, double tokens, double quality) {
+      return rounds_of_workgroups(tiles, cus) * tokens / quality;
     };
     if (M > 128 && cost(t256, 256.0, 1.0) <= cost(t128, 128.0, 0.65))
       return launch_gated<GatedShape256>(W, X, Y, ldy, M, I, K, stream);

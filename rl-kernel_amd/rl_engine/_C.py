@@ -19,7 +19,32 @@ _BF16 = torch.bfloat16
 
 
 def _stream_handle(device: torch.device) -> int:
-    return int(torch.cuda.current_stream(device).cuda_stream)
+    """The raw handle of ``device``'s current stream (what ``torch.cuda.current_stream(device).cuda_stream`` holds,
+    without building the stream object: this runs on every call)."""
+    return torch._C._cuda_getCurrentRawStream(device.index)
+
+
+class _NoSwitch:
+    """A context manager that does nothing: the device is already current."""
+
+    __slots__ = ()
+
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on(device: torch.device):
+    """``torch.cuda.device(device)`` for the launch, or nothing at all when that device is current already (the
+    usual case; entering and leaving the guard costs several microseconds per call)."""
+    if device.index == torch._C._cuda_getDevice():
+        return _NO_SWITCH
+    return torch.cuda.device(device)
 
 
 def _check_in(t: torch.Tensor, name: str) -> None:
@@ -45,7 +70,7 @@ def _raw_gemm(
 ) -> None:
     """One call of rlk_det_gemm_bf16 on the current stream of ``a``'s device."""
     lib = _lib.load()
-    with torch.cuda.device(a.device):
+    with _on(a.device):
         status = lib.rlk_det_gemm_bf16(
             a.data_ptr(),
             a_row_stride,
@@ -81,6 +106,40 @@ def gemm_strided(
     return out
 
 
+_gemm_entry = None  # rlk_det_gemm_bf16, looked up once
+
+
+def linear_plain(a: torch.Tensor, weight: torch.Tensor) -> Optional[torch.Tensor]:
+    """``a[M,K] @ weight[N,K].T`` into a fresh bf16 ``[M,N]`` for the everyday operands - two non-empty 2-D bf16
+    tensors on one GPU with matching K and contiguous rows - or ``None`` for anything else (including everything
+    that has to raise: the long way words the errors). The same call of rlk_det_gemm_bf16 that
+    :func:`gemm_strided` makes for ``(a, weight.t())``, without the rule tables and the transposed view."""
+    global _gemm_entry
+    sa, sw = a.stride(), weight.stride()
+    if len(sa) != 2 or len(sw) != 2 or sa[1] != 1 or sw[1] != 1 or sa[0] < 0 or sw[0] < 0:
+        return None
+    if a.dtype is not _BF16 or weight.dtype is not _BF16:
+        return None
+    device = a.device
+    if device.type != "cuda" or weight.device != device:
+        return None
+    m, k = a.shape
+    n, kw = weight.shape
+    if k != kw or m == 0 or n == 0 or k == 0:
+        return None
+    if _gemm_entry is None:
+        _gemm_entry = _lib.load().rlk_det_gemm_bf16
+    out = torch.empty((m, n), dtype=_BF16, device=device)
+    with _on(device):
+        status = _gemm_entry(
+            a.data_ptr(), sa[0], 1, weight.data_ptr(), 1, sw[0], out.data_ptr(), n, m, n, k, 0, 0,
+            torch._C._cuda_getCurrentRawStream(device.index),
+        )  # fmt: skip
+    if status:
+        _lib.check(status, "rlk_det_gemm_bf16 failed")
+    return out
+
+
 def gemm_tree_strided(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor, config: int = 0) -> torch.Tensor:
     """``out[M,N] = a[M,K] @ b[K,N]`` under the k-tree contract, arbitrary non-negative strides.
 
@@ -92,7 +151,7 @@ def gemm_tree_strided(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor, confi
     if m == 0 or n == 0:
         return out
     lib = _lib.load()
-    with torch.cuda.device(a.device):
+    with _on(a.device):
         status = lib.rlk_det_gemm_tree_bf16_config(
             a.data_ptr(),
             a.stride(0),
@@ -178,7 +237,7 @@ def det_gemm_seq(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype = torc
     out = torch.empty((m, n), dtype=out_dtype, device=a.device)
     if m == 0 or n == 0:
         return out
-    with torch.cuda.device(a.device):
+    with _on(a.device):
         status = _lib.load().rlk_det_gemm_seq(
             a.data_ptr(), _SEQ_DTYPES[a.dtype], a.stride(0), a.stride(1), b.data_ptr(), _SEQ_DTYPES[b.dtype],
             b.stride(0), b.stride(1), out.data_ptr(), _SEQ_DTYPES[out_dtype], n, m, n, k, _stream_handle(a.device),
@@ -335,7 +394,7 @@ def _linear_logp_forward(
             first.data_ptr(), lse.data_ptr(),
         )  # fmt: skip
         tail = (workspace.data_ptr(), ws_bytes, n, d, v, int(vocab_start_index), real_vocab, config, _stream_handle(hidden.device))
-        with torch.cuda.device(hidden.device):
+        with _on(hidden.device):
             if want_logits:  # the logits come out of the same pass: entry + "_logits"
                 entry = entry + "_logits"
                 status = getattr(lib, entry)(*head, logits.data_ptr(), logits.stride(0), *tail)
@@ -482,7 +541,7 @@ def fused_linear_logp_bwd(
         if grad_bias is not None:
             grad_bias.zero_()
         return [grad_hidden, grad_weight, grad_bias]
-    with torch.cuda.device(hidden.device):
+    with _on(hidden.device):
         status = lib.rlk_linear_logp_bwd(
             hidden.data_ptr(),
             hidden.stride(0),
@@ -595,7 +654,7 @@ def hip_deterministic_logp_tile_stats(
         if temperature.numel() != rows:
             raise RuntimeError("temperature must have one value per row")
         temp = temperature.reshape(-1).to(device=logits.device, dtype=torch.float32).contiguous()
-    with torch.cuda.device(logits.device):
+    with _on(logits.device):
         status = _lib.load().rlk_logits_tile_stats(
             src.data_ptr(), code, src.stride(0), temp.data_ptr() if temp is not None else None, rows, local_vocab,
             int(vocab_start), int(real_vocab), int(num_tiles), tile_max.data_ptr(), tile_sum.data_ptr(),
@@ -638,7 +697,7 @@ def hip_deterministic_logp_from_logits(
     lib = _lib.load()
     ws_bytes = int(lib.rlk_logp_from_logits_workspace_bytes(rows, int(num_tiles)))
     workspace = torch.empty((ws_bytes // 4,), dtype=torch.float32, device=logits.device)
-    with torch.cuda.device(logits.device):
+    with _on(logits.device):
         status = lib.rlk_logp_from_logits(
             src.data_ptr(), code, src.stride(0), target_i64.data_ptr(), temp.data_ptr() if temp is not None else None,
             rows, local_vocab, int(vocab_start), int(real_vocab), int(num_tiles), logp.data_ptr(), lse.data_ptr(),
@@ -693,7 +752,7 @@ def hip_deterministic_logp_backward(
         if temperature.numel() != rows:
             raise RuntimeError("temperature must have one value per row")
         temp = temperature.reshape(-1).to(device=src.device, dtype=torch.float32).contiguous()
-    with torch.cuda.device(src.device):
+    with _on(src.device):
         status = _lib.load().rlk_logits_logp_backward(
             src.data_ptr(), code, src.stride(0), lse.data_ptr(), coef_logp.data_ptr(),
             coef_lse.data_ptr() if has_lse_grad else None, target_local.data_ptr(),
@@ -740,7 +799,7 @@ def swiglu_forward(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     y = torch.empty_like(gate)
     rows, cols = _rows_cols(gate)
     if gate.numel():
-        with torch.cuda.device(gate.device):
+        with _on(gate.device):
             status = _lib.load().rlk_swiglu_fwd(
                 gate.data_ptr(), cols, up.data_ptr(), cols, y.data_ptr(), cols, rows, cols,
                 _act_dtype_code(gate), _stream_handle(gate.device),
@@ -763,7 +822,7 @@ def swiglu_backward(dy: torch.Tensor, gate: torch.Tensor, up: torch.Tensor) -> L
     d_gate, d_up = torch.empty_like(gate), torch.empty_like(up)
     rows, cols = _rows_cols(gate)
     if gate.numel():
-        with torch.cuda.device(gate.device):
+        with _on(gate.device):
             status = _lib.load().rlk_swiglu_bwd(
                 dy.data_ptr(), cols, gate.data_ptr(), cols, up.data_ptr(), cols, d_gate.data_ptr(), cols,
                 d_up.data_ptr(), cols, rows, cols, _act_dtype_code(gate), _stream_handle(gate.device),
@@ -784,7 +843,7 @@ def swiglu_packed_forward(gate_up: torch.Tensor) -> torch.Tensor:
     y = torch.empty((rows, width), dtype=gate_up.dtype, device=gate_up.device)
     if y.numel():
         base = gate_up.data_ptr()
-        with torch.cuda.device(gate_up.device):
+        with _on(gate_up.device):
             status = _lib.load().rlk_swiglu_fwd(
                 base, 2 * width, base + gate_up.element_size() * width, 2 * width, y.data_ptr(), width, rows, width,
                 _act_dtype_code(gate_up), _stream_handle(gate_up.device),
@@ -810,7 +869,7 @@ def swiglu_packed_backward(dy: torch.Tensor, gate_up: torch.Tensor) -> List[torc
     d_up = torch.empty_like(d_gate)
     if d_gate.numel():
         base = gate_up.data_ptr()
-        with torch.cuda.device(gate_up.device):
+        with _on(gate_up.device):
             status = _lib.load().rlk_swiglu_bwd(
                 dy.data_ptr(), width, base, 2 * width, base + gate_up.element_size() * width, 2 * width,
                 d_gate.data_ptr(), width, d_up.data_ptr(), width, rows, width, _act_dtype_code(gate_up),
@@ -848,7 +907,7 @@ def det_gemm_swiglu(a: torch.Tensor, weight: torch.Tensor, out: Optional[torch.T
     lib = _lib.load()
     ws_bytes = int(lib.rlk_det_gemm_swiglu_workspace_bytes(a_c.data_ptr(), a_c.stride(0), w_c.data_ptr(), w_c.stride(0), m, inter, k))
     workspace = torch.empty((ws_bytes // 2,), dtype=_BF16, device=a.device) if ws_bytes else None
-    with torch.cuda.device(a.device):
+    with _on(a.device):
         status = lib.rlk_det_gemm_swiglu_bf16(
             a_c.data_ptr(), a_c.stride(0), w_c.data_ptr(), w_c.stride(0), out.data_ptr(), out.stride(0),
             workspace.data_ptr() if workspace is not None else None, ws_bytes, m, inter, k, _stream_handle(a.device),
@@ -895,7 +954,7 @@ def grpo_ratio_kl_loss(
     out3 = torch.empty((3,), dtype=torch.float32, device=logp.device)
     ws_bytes = int(lib.rlk_grpo_workspace_bytes(rollouts))
     workspace = torch.empty((max(ws_bytes, 4) // 4,), dtype=torch.float32, device=logp.device)
-    with torch.cuda.device(logp.device):
+    with _on(logp.device):
         status = lib.rlk_grpo_ratio_kl_loss(
             logp_c.data_ptr(),
             old_c.data_ptr(),

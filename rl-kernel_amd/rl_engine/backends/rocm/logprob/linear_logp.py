@@ -33,6 +33,7 @@ def _prepare(
     weight: torch.Tensor,
     target_ids: torch.Tensor,
     temperature: Optional[torch.Tensor],
+    validate: bool,
 ):
     if hidden.device.type != "cuda":
         raise RuntimeError(f"deterministic HIP linear_logp requires a GPU tensor, got device '{hidden.device}'.")
@@ -42,9 +43,13 @@ def _prepare(
         raise ValueError(f"hidden dim {hidden.size(-1)} must match lm_head_weight dim {weight.size(-1)}")
     if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
         raise TypeError("deterministic HIP linear_logp requires BF16 hidden and lm_head_weight")
-    hidden_2d = hidden.reshape(-1, hidden.size(-1)).contiguous()
-    weight_c = weight.contiguous()
-    target_1d = target_ids.reshape(-1).to(device=hidden_2d.device, dtype=torch.long).contiguous()
+    # the usual call hands over what the kernel takes; only other layouts pay for a reshape or a copy
+    hidden_2d = hidden if hidden.dim() == 2 and hidden.is_contiguous() else hidden.reshape(-1, hidden.size(-1)).contiguous()
+    weight_c = weight if weight.is_contiguous() else weight.contiguous()
+    if target_ids.dim() == 1 and target_ids.dtype == torch.long and target_ids.device == hidden_2d.device and target_ids.is_contiguous():
+        target_1d = target_ids
+    else:
+        target_1d = target_ids.reshape(-1).to(device=hidden_2d.device, dtype=torch.long).contiguous()
     if target_1d.numel() != hidden_2d.size(0):
         raise ValueError("target_ids must have one id per hidden row")
     temp_arg = None
@@ -54,7 +59,7 @@ def _prepare(
             temp_arg = temp_arg.expand(hidden_2d.size(0)).contiguous()
         else:
             temp_arg = temp_arg.contiguous()
-        if temp_arg.numel() != hidden_2d.size(0) or bool((temp_arg <= 0).any().item()):
+        if temp_arg.numel() != hidden_2d.size(0) or (validate and bool((temp_arg <= 0).any().item())):
             raise ValueError("temperature must be positive and scalar or per-token")
     return hidden_2d, weight_c, target_1d, temp_arg
 
@@ -135,6 +140,7 @@ def hip_deterministic_linear_logp(
     real_vocab_size: int = -1,
     vocab_start_index: int = 0,
     config: str | int = 0,
+    validate: bool = False,
 ):
     """Strict entry: returns fp32 ``(logp, lse)`` (plus logits on request); differentiable
     with respect to ``hidden``, ``lm_head_weight`` and ``bias``.
@@ -143,13 +149,21 @@ def hip_deterministic_linear_logp(
     ``target_ids`` and ``temperature`` receive bitwise-identical results for a
     row whatever batch it arrives in. ``real_vocab_size`` masks padded vocabulary
     lanes out of the LSE; ``-1`` disables masking.
+
+    Values of ``target_ids`` and ``temperature``: the reference's strict entry reads them back from the device
+    before it launches and raises ``ValueError`` for an id outside the real vocabulary or a temperature that is
+    not positive (rl_engine/backends/shared/triton/logprob/linear_logp.py:516-517, 666-672). That read-back is a
+    host synchronisation on every call, so here it is opt-in: ``validate=True`` does exactly that; by default
+    nothing is read back (the call can be captured in a HIP graph) and the kernel marks such a row instead -
+    ``logp`` is NaN for an id outside ``[vocab_start_index, vocab_start_index + real_vocab_size)``, ``logp`` and
+    ``lse`` are NaN for a temperature that is not a positive number.
     """
-    hidden_2d, weight, target_1d, temp_arg = _prepare(hidden, lm_head_weight, target_ids, temperature)
+    hidden_2d, weight, target_1d, temp_arg = _prepare(hidden, lm_head_weight, target_ids, temperature, bool(validate))
     lead_shape = hidden.shape[:-1]
     real_vocab = weight.size(0) if int(real_vocab_size) < 0 else int(real_vocab_size)
     if not 0 < real_vocab <= weight.size(0):
         raise ValueError(f"real_vocab_size must be in [1, {weight.size(0)}], got {real_vocab_size}")
-    if target_1d.numel():
+    if validate and target_1d.numel():
         lo = int(vocab_start_index)
         bad = (target_1d < lo) | (target_1d >= lo + real_vocab)
         if bool(bad.any().item()):
@@ -177,8 +191,10 @@ def hip_deterministic_linear_logp(
         vocab_start_index=int(vocab_start_index),
         config=int(config),
     )
-    logp = outputs[0].reshape(lead_shape)
-    lse = outputs[1].reshape(lead_shape)
+    if hidden.dim() == 2:
+        logp, lse = outputs[0], outputs[1]
+    else:
+        logp, lse = outputs[0].reshape(lead_shape), outputs[1].reshape(lead_shape)
     if return_logits:
         return logp, lse, outputs[2].reshape(*lead_shape, weight.size(0))
     return logp, lse

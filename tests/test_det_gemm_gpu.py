@@ -671,6 +671,40 @@ def test_weight_transpose_cache_refresh(gemm):
     assert gemm.refresh_cached_weight_transposes([w]) == 0
 
 
+def test_prepare_writes_only_its_own_output(gemm):
+    # a second prepare of a weight that was updated in place leaves the first buffer alone (it may be a snapshot)
+    w = inputs.randn_bf16(124, 24, 32, 0.1).to(DEV)
+    old_t = gemm.prepare_det_gemm_linear_weight(w)
+    old_bits = old_t.clone()
+    w.mul_(3)
+    new_t = gemm.prepare_det_gemm_linear_weight(w)
+    assert torch.equal(old_t, old_bits) and torch.equal(new_t, w.t()) and not torch.equal(new_t, old_t)
+    # weights loaded layer by layer through one staging tensor: the allocator hands out the same address and
+    # shape again, and the earlier layers' prepared weights must keep their values
+    layers, prepared = [], []
+    for seed in (125, 126, 127):
+        staging = inputs.randn_bf16(seed, 48, 64, 0.1).to(DEV)
+        layers.append(staging.clone().t().contiguous())
+        prepared.append(gemm.prepare_det_gemm_linear_weight(staging))
+        del staging  # freed: the next layer's staging tensor usually reuses the block
+    for want, got in zip(layers, prepared):
+        assert torch.equal(want, got)
+    # the same through one tensor object that is overwritten in place between layers
+    staging = torch.empty((48, 64), dtype=torch.bfloat16, device=DEV)
+    layers, prepared = [], []
+    for seed in (128, 129):
+        staging.copy_(inputs.randn_bf16(seed, 48, 64, 0.1).to(DEV))
+        layers.append(staging.clone().t().contiguous())
+        prepared.append(gemm.prepare_det_gemm_linear_weight(staging))
+    for want, got in zip(layers, prepared):
+        assert torch.equal(want, got)
+    # a source that died is forgotten: a new tensor at its address has no prepared copies
+    del staging
+    fresh = torch.zeros((48, 64), dtype=torch.bfloat16, device=DEV)
+    assert gemm.refresh_cached_weight_transposes([fresh]) == 0
+    assert torch.equal(prepared[1], layers[1])
+
+
 @pytest.mark.parametrize("rows", (16, 48, 300))
 def test_hip_graph_capture_replays_bit_identically(gemm, rows):
     # 16 and 48 rows: the streaming kernel (one and three token tiles); 300: a tile kernel

@@ -198,6 +198,30 @@ def test_facade_validation_matches_the_reference_error_types():
         facade.prepare_det_gemm_linear_weight(a[0])
 
 
+def test_prepared_weight_registry_identifies_sources_by_storage():
+    import gc
+
+    from rl_engine.backends.rocm.gemm import det_gemm as facade
+
+    w = torch.zeros((6, 4), dtype=torch.bfloat16)
+    buf_a, buf_b = torch.zeros((4, 6), dtype=torch.bfloat16), torch.zeros((4, 6), dtype=torch.bfloat16)
+    facade._remember_prepared(w, buf_a)
+    facade._remember_prepared(w.data, buf_b)  # another tensor object over the same storage: the same source
+    facade._remember_prepared(w, buf_a)  # registered once
+    live = facade._live_prepared(w)
+    assert len(live) == 2 and live[0] is buf_a and live[1] is buf_b
+    assert facade._live_prepared(w[:3]) == [] and facade._live_prepared(w.view(4, 6)) == []  # other views: other sources
+    del buf_b, live
+    gc.collect()
+    assert [b is buf_a for b in facade._live_prepared(w)] == [True]  # a dropped buffer is forgotten
+    entries = len(facade._PREPARED_TRANSPOSES)
+    del w
+    gc.collect()
+    assert len(facade._PREPARED_TRANSPOSES) == entries - 1  # the entry dies with the source's storage
+    w2 = torch.zeros((6, 4), dtype=torch.bfloat16)  # likely the same address; a different source all the same
+    assert facade._live_prepared(w2) == []
+
+
 def test_linear_logp_python_validation():
     from rl_engine.ops.logprob import LinearLogpOp, deterministic_linear_logp
 

@@ -152,6 +152,22 @@ def test_backward_is_bitwise_deterministic_and_config_neutral(native):
                     assert torch.equal(x.view(torch.uint8), y.view(torch.uint8)), (shape, name, flag)
 
 
+@pytest.mark.parametrize("tokens", (1040, 2100))
+def test_bias_gradient_is_config_neutral_above_1024_tokens(native, tokens):
+    # above 1024 tokens the bias partial rows are per 64-token tile, and a forced 16-token tile is remapped to 64:
+    # grad_bias (and the other two gradients) must keep the bits of the automatic choice under every configuration
+    from rl_engine import _lib
+
+    c = _case(tokens, 1536, 128, 5250 + tokens, bias=True, temperature=True, real=1500)
+    _, base = _gpu_backward(native, c)
+    for name, value in _lib.LOGP_CONFIGS.items():
+        for flag in (0, _lib.FORCE_STAGED):
+            _, other = _gpu_backward(native, c, config=value | flag)
+            for x, y in zip(base, other):
+                assert torch.equal(x.view(torch.uint8), y.view(torch.uint8)), (tokens, name, flag)
+    assert not bool(base[2][1500:].any()) and bool(torch.isfinite(base[2]).all())
+
+
 def test_grad_hidden_rows_are_batch_invariant(native):
     c = _case(384, 4096, 256, 5300, temperature=True)
     _, (gh_full, _, _) = _gpu_backward(native, c)

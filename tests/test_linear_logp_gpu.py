@@ -221,12 +221,23 @@ def test_uniform_logits_and_target_checks(logp_mod):
     logp, lse = logp_mod.deterministic_linear_logp(h, w, t)
     assert torch.allclose(logp, torch.full_like(logp, -float(np.log(v))), atol=1e-5)
     assert torch.allclose(lse, torch.full_like(lse, float(np.log(v))), atol=1e-5)
+    # values are checked on the host (a read-back, as the reference's strict entry does) only on request ...
+    bad_t = torch.tensor([0, 1, 5000, 2], device=DEV)
+    bad_temp = torch.tensor([1.0, 0.0, 1.0, -2.0])
     with pytest.raises(ValueError, match="real vocabulary"):
-        logp_mod.deterministic_linear_logp(h, w, torch.tensor([0, 1, 5000, 2], device=DEV))
+        logp_mod.deterministic_linear_logp(h, w, bad_t, validate=True)
+    with pytest.raises(ValueError, match="temperature"):
+        logp_mod.deterministic_linear_logp(h, w, t, temperature=bad_temp, validate=True)
+    # ... by default the kernel marks the offending rows, and only those, with NaN
+    marked, lse_marked = logp_mod.deterministic_linear_logp(h, w, bad_t)
+    assert bool(torch.isnan(marked[2])) and _same_bits(marked[[0, 1]], logp[[0, 1]]) and _same_bits(lse_marked, lse)
+    marked, _ = logp_mod.deterministic_linear_logp(h, w, torch.tensor([-1, 1, 4990, 2], device=DEV), real_vocab_size=4990)
+    assert torch.isnan(marked).tolist() == [True, False, True, False]
+    marked, lse_marked = logp_mod.deterministic_linear_logp(h, w, t, temperature=bad_temp)
+    assert torch.isnan(marked).tolist() == [False, True, False, True] and torch.isnan(lse_marked).tolist() == [False, True, False, True]
+    assert _same_bits(marked[[0, 2]], logp[[0, 2]])
     with pytest.raises(ValueError, match="real_vocab_size"):
         logp_mod.deterministic_linear_logp(h, w, t, real_vocab_size=v + 1)
-    with pytest.raises(ValueError, match="temperature"):
-        logp_mod.deterministic_linear_logp(h, w, t, temperature=torch.tensor([1.0, 0.0, 1.0, 1.0]))
     with pytest.raises(ValueError, match="one id per hidden row"):
         logp_mod.deterministic_linear_logp(h, w, t[:3])
     hg = h.clone().requires_grad_(True)

@@ -651,3 +651,42 @@ def test_swiglu_values_is_the_unrounded_form_of_the_bf16_functions(oracle):
     dg, du = oracle.swiglu_values(np.zeros(2), np.full(2, 3.0), np.full(2, 2.0))
     assert dg.tolist() == [3.0, 3.0] and du.tolist() == [0.0, 0.0]
     assert oracle.swiglu_values(np.full(1, 40.0), np.full(1, 0.5))[0] == 20.0
+
+
+# ---------------------------------------------------------------------------
+# torch forms (what the CPU baseline times)
+# ---------------------------------------------------------------------------
+
+
+def test_torch_forms_agree_with_the_numpy_forms(oracle):
+    import torch
+
+    rng = np.random.default_rng(77)
+    a_bits = oracle.randn_bf16(rng, (33, 192))
+    bt_bits = oracle.randn_bf16(rng, (70, 192), 0.05)
+    a = torch.from_numpy(a_bits.view(np.int16)).view(torch.bfloat16)
+    bt = torch.from_numpy(bt_bits.view(np.int16)).view(torch.bfloat16)
+    want = oracle.det_gemm_ref(a_bits, bt_bits)
+    got = oracle.det_gemm_ref_torch(a, bt).view(torch.int16).numpy().view(np.uint16)
+    # two fp32 BLAS orders, one rounding each: identical except where the fp32 sums straddle a rounding boundary
+    assert (oracle.bf16_ulp_distance(got, want) <= 1).all()
+    assert (got == want).mean() > 0.98
+    exact = oracle.det_gemm_f64(a_bits, bt_bits)
+    native = oracle.native_gemm_torch(a, bt).float().numpy().astype(np.float64)
+    scale = np.abs(oracle.bf16_to_f32(a_bits).astype(np.float64)) @ np.abs(oracle.bf16_to_f32(bt_bits).astype(np.float64)).T
+    assert (np.abs(native - exact) <= 2.0**-7 * scale).all()  # bf16 matmul: at most bf16-level error of the term sum
+    # an order-sensitive transposition check: a @ bt.T is not bt @ a.T
+    assert got.shape == (33, 70)
+
+    h_bits = oracle.randn_bf16(rng, (9, 64))
+    w_bits = oracle.randn_bf16(rng, (301, 64), 0.3)
+    target = rng.integers(0, 301, size=9)
+    h = torch.from_numpy(h_bits.view(np.int16)).view(torch.bfloat16)
+    w = torch.from_numpy(w_bits.view(np.int16)).view(torch.bfloat16)
+    logp_t, lse_t = oracle.linear_logp_chunked_torch(h, w, torch.from_numpy(target), chunk_elems=9 * 50)
+    logp_n, lse_n, *_ = oracle.linear_logp_chunked(h_bits, w_bits, target, chunk_elems=9 * 50)
+    np.testing.assert_allclose(logp_t.numpy(), logp_n, atol=2e-6, rtol=0)
+    np.testing.assert_allclose(lse_t.numpy(), lse_n, atol=2e-6, rtol=0)
+    f64_logp, _ = oracle.linear_logp_f64(h_bits, w_bits, target)
+    np.testing.assert_allclose(logp_t.numpy(), f64_logp, atol=1e-5, rtol=0)
+    assert oracle.cpu_model_string()
