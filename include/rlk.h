@@ -312,8 +312,9 @@ typedef enum rlk_dtype { RLK_DTYPE_BF16 = 0, RLK_DTYPE_FP16 = 1, RLK_DTYPE_FP32 
  * one fp32 fused multiply-add per k, k ascending, one accumulator per element, nothing rounded below fp32.
  * a_dtype / b_dtype / c_dtype are RLK_DTYPE_BF16 or RLK_DTYPE_FP32 (bf16 operands are widened exactly; a
  * bf16 output is the fp32 result rounded once). Strides in elements as in rlk_det_gemm_bf16, any
- * non-negative values. Rows are batch invariant. Vector-ALU kernel (about 80 TFLOP/s): the fp32-result
- * path of the strict GEMM, not a replacement for rlk_det_gemm_bf16.
+ * non-negative values. Rows are batch invariant. Runs on the fp32 matrix pipe, one reduction-length-one
+ * MFMA per k (that instruction is a fused multiply-add on fp32 operands as well), at 120-135 TFLOP/s: the
+ * fp32-result path of the strict GEMM, not a replacement for rlk_det_gemm_bf16.
  *
  * Stands in for _triton_gemm_fp32 / _det_gemm_fp32_kernel
  * (rl_engine/backends/shared/triton/gemm/det_gemm.py:680-749), i.e. DetGemmOp.forward_fp32 and

@@ -316,7 +316,9 @@ def test_tree_backend_routes_the_whole_facade(gemm, oracle, monkeypatch):
     assert gemm.det_gemm_backend() == "hip_mfma"
 
 
-@pytest.mark.parametrize("shape", [(1, 1, 1), (5, 9, 31), (64, 128, 32), (65, 129, 33), (70, 200, 1000), (130, 40, 4096), (3, 300, 97)])
+@pytest.mark.parametrize("shape", [(1, 1, 1), (5, 9, 31), (64, 128, 32), (65, 129, 33), (70, 200, 1000), (130, 40, 4096), (3, 300, 97),
+                                   (129, 257, 77), (300, 130, 3), (200, 64, 515), (257, 1, 36),
+                                   (300, 200, 96), (1030, 260, 33)])
 def test_sequential_fp32_gemm_equals_the_oracle_bit_for_bit(oracle, shape):
     """rlk_det_gemm_seq: one fused multiply-add per k, ascending. Fully specified, so bit-exact against the
     oracle: bf16 and fp32 operands in every combination, both output types, strided views."""
@@ -347,6 +349,30 @@ def test_sequential_fp32_gemm_equals_the_oracle_bit_for_bit(oracle, shape):
     alone = _C.det_gemm_fwd_fp32(a32[row : row + 1].to(DEV), b32.to(DEV).t())
     full = _C.det_gemm_fwd_fp32(a32.to(DEV), b32.to(DEV).t())
     assert torch.equal(alone.view(torch.int32), full[row : row + 1].view(torch.int32))
+
+
+def test_sequential_fp32_gemm_special_values_equal_the_oracle(oracle):
+    """The chain runs as one reduction-length-one fp32 MFMA per k. That instruction must behave as the fused
+    multiply-add of the oracle (the CPU's fmaf) on every kind of value: signed zeros, fp32 and bf16 denormals, the
+    largest finite values, infinities (NaN results compare as NaN), through both loaders."""
+    from rl_engine import _C
+
+    g = torch.Generator().manual_seed(9790)
+    specials = torch.tensor([0.0, -0.0, 1e-39, -3e-40, 2.0**-126, 3.0e38, -3.0e38, float("inf"), -float("inf"), 1.0, -1.0, 2.0**-133])
+    for m, n, k in ((200, 96, 70), (130, 136, 64)):  # element loads with a K tail; 16-byte loads
+        a = torch.randn((m, k), generator=g)
+        b = torch.randn((n, k), generator=g)
+        a.view(-1)[torch.randperm(a.numel(), generator=g)[:900]] = specials[torch.randint(0, len(specials), (900,), generator=g)]
+        b.view(-1)[torch.randperm(b.numel(), generator=g)[:500]] = specials[torch.randint(0, len(specials), (500,), generator=g)]
+        a[7] = 0.0  # a row of zeros against everything: +0 / NaN only
+        a[9] = -0.0
+        for lhs, rhs in ((a, b), (a.to(torch.bfloat16), b.to(torch.bfloat16)), (a, b.to(torch.bfloat16))):
+            with np.errstate(all="ignore"):
+                want = torch.from_numpy(oracle.det_gemm_seq_f32(lhs.float().numpy(), rhs.float().numpy()))
+            got = _C.det_gemm_fwd_fp32(lhs.to(DEV), rhs.to(DEV).t()).cpu()
+            both_nan = torch.isnan(want) & torch.isnan(got)
+            assert torch.equal(torch.where(both_nan, 0, want.view(torch.int32)), torch.where(both_nan, 0, got.view(torch.int32))), (m, lhs.dtype, rhs.dtype)
+            assert bool(torch.isnan(got).any()) and bool(torch.isinf(got).any()) and bool((got == 0).any())
 
 
 def test_sequential_fp32_gemm_order_and_fused_step_known_answers():
