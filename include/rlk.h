@@ -127,8 +127,24 @@ typedef enum rlk_tree_config {
   RLK_TREE_CFG_NODES = 4,    /* any row count: 16 rows x 64 columns per workgroup, the 16 depth-4 nodes on 16 waves
                                 (fp32 MFMA, operands from memory to registers); same eligibility as SKINNY but
                                 trees of 4 to 10 levels */
-  RLK_TREE_CFG_COUNT = 5
+  RLK_TREE_CFG_COUNT = 5,
+  /* OR-ed into RLK_TREE_CFG_AUTO or RLK_TREE_CFG_MFMA_F32: the leaf-space split, a different contract
+   * (rlk_det_gemm_tree_leaf_space_contract_id). */
+  RLK_TREE_CFG_LEAF_SPACE = 0x100
 } rlk_tree_config;
+
+/*
+ * Contract id of the k-tree with the midpoint split in LEAF space (RLK_TREE_CFG_LEAF_SPACE): the leaves are the
+ * fixed K tiles [32 i, min(32 i + 32, K)), each summed as above, and a node over leaves [lo, hi) is
+ * bf16(float(T(lo,mid)) + float(T(mid,hi))) with mid = lo + (hi - lo) / 2 counted in leaves. Same bits as the
+ * element-space contract whenever K / 32 is a power of two (K = 1024, 4096); a different tree otherwise
+ * (K = 12288: 384 leaves of 32 here, 512 leaves of 24 there).
+ *
+ * Stands in for the split of DetGemmTreeReferenceOp (rl_engine/reference/gemm/det_gemm.py:29-60) and of the SM90
+ * kernel (csrc/cuda/gemm/det_gemm_kernel.cu:221-234, 351-379); a leaf here is the same chain of single fused
+ * multiply-adds as in the element-space contract.
+ */
+const char* rlk_det_gemm_tree_leaf_space_contract_id(void);
 
 /* rlk_det_gemm_tree_bf16 with an explicit leaf loop (rlk_tree_config). */
 int rlk_det_gemm_tree_bf16_config(const void* a, int64_t a_row_stride, int64_t a_k_stride, const void* b,

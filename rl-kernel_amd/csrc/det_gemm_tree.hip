@@ -409,9 +409,17 @@ __global__ __launch_bounds__(kTreeWideThreads, MAXD <= 10 ? 4 : 2) void det_gemm
     }
   };
 
+  // A node is a range [lo, hi) of units, split at lo + (hi - lo) / 2. Element-space split (the contract of
+  // rlk_det_gemm_tree_contract_id): a unit is one k, and a node of at most 32 units is a leaf. Leaf-space split
+  // (bit 5 of `fast`): a unit is one of the fixed 32-wide K tiles [32 i, min(32 i + 32, K)), and a node of one
+  // unit is a leaf. The two trees are the same when K / 32 is a power of two.
+  const bool leaf_space = fast & 32;
+  const int unit = leaf_space ? kTreeLeaf : 1;
+  const int units = leaf_space ? (K + kTreeLeaf - 1) / kTreeLeaf : K;
+  const int leaf_units = leaf_space ? 1 : kTreeLeaf;
   auto range_at = [&](int depth, uint32_t path, int& lo, int& hi) {
     lo = 0;
-    hi = K;
+    hi = units;
     for (int d = 1; d <= depth; ++d) {
       const int mid = lo + (hi - lo) / 2;
       if ((path >> d) & 1u) lo = mid; else hi = mid;
@@ -427,13 +435,13 @@ __global__ __launch_bounds__(kTreeWideThreads, MAXD <= 10 ? 4 : 2) void det_gemm
   const int a_row = 32 * (wave & 1) + 16 * (lane >> 5) + (lane & 15);
   const int b_row = kTreeBM + 32 * (wave >> 1) + 16 * ((lane >> 4) & 1) + (lane & 15);
 
-  int depth = 0, lo = 0, hi = K;
+  int depth = 0, lo = 0, hi = units;
   uint32_t path = 0;
-  while (hi - lo > kTreeLeaf) {
+  while (hi - lo > leaf_units) {
     hi = lo + (hi - lo) / 2;
     ++depth;
   }
-  fetch(lo);
+  fetch(lo * unit);
   deposit(0);
   __syncthreads();
 
@@ -460,15 +468,15 @@ __global__ __launch_bounds__(kTreeWideThreads, MAXD <= 10 ? 4 : 2) void det_gemm
         npath = (path & ((1u << nd) - 1u)) | (1u << nd);
         range_at(nd, npath, nlo, nhi);
         ndepth = nd;
-        while (nhi - nlo > kTreeLeaf) {
+        while (nhi - nlo > leaf_units) {
           nhi = nlo + (nhi - nlo) / 2;
           ++ndepth;
         }
       }
     }
-    if (has_next) fetch(nlo);
+    if (has_next) fetch(nlo * unit);
 
-    const int len = hi - lo;
+    const int len = (hi * unit < K ? hi * unit : K) - lo * unit;
     const char* arow = stage_bytes[leaf & 1] + a_row * kRowBytes;
     const char* brow = stage_bytes[leaf & 1] + b_row * kRowBytes;
     f32x16_t acc;
@@ -861,15 +869,39 @@ static void launch_wide(const MatView& A, const MatView& B, bf16_bits* out, int6
 // A[M, K] and B as rows of output columns (B.rows = N), any strides; C[m * ldc + n].
 // config: RLK_TREE_CFG_AUTO, or one of the two leaf loops (same bits).
 hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int64_t ldc, int M, int N, int K,
-                                int config, hipStream_t stream) {
+                                int config, hipStream_t stream, bool leaf_space) {
   const int tiles_m = (M + kTreeBM - 1) / kTreeBM;
   const int tiles_n = (N + kTreeBN - 1) / kTreeBN;
   const int64_t tiles64 = (int64_t)tiles_m * tiles_n;
   if (tiles64 > 0x7fffffff) return hipErrorInvalidValue;
   const unsigned tiles = (unsigned)tiles64;
+  bf16_bits* out = reinterpret_cast<bf16_bits*>(C);
+  if (leaf_space) {
+    // With a power-of-two number of whole leaves the leaf-space tree is the element-space tree: every kernel
+    // below serves it. Otherwise the tiled matrix-pipe kernel walks the tree in units of leaves.
+    const int leaves = (K + kTreeLeaf - 1) / kTreeLeaf;
+    if (K % kTreeLeaf != 0 || (leaves & (leaves - 1)) != 0) {
+      int levels = 0;
+      while ((1 << levels) < leaves) ++levels;
+      if (levels > 20) return hipErrorInvalidValue;
+      auto chunked = [&](const MatView& v) {  // leaves start on multiples of 32; the last one ends at K
+        return K % 8 == 0 && v.k_stride == 1 && v.row_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0;
+      };
+      auto rows8 = [&](const MatView& v, int rows) {
+        return v.row_stride == 1 && rows % 8 == 0 && v.k_stride >= rows && v.k_stride % 8 == 0 &&
+               (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0;
+      };
+      const bool a_chunked = chunked(A), b_chunked = chunked(B);
+      const int fast = 32 | (a_chunked ? 1 : 0) | (b_chunked ? 2 : 0) | (!a_chunked && rows8(A, M) ? 8 : 0) |
+                       (!b_chunked && rows8(B, N) ? 16 : 0);
+      if (levels <= 7) launch_wide<7>(A, B, out, ldc, M, N, K, tiles, tiles_m, fast, stream);
+      else if (levels <= 10) launch_wide<10>(A, B, out, ldc, M, N, K, tiles, tiles_m, fast, stream);
+      else launch_wide<20>(A, B, out, ldc, M, N, K, tiles, tiles_m, fast, stream);
+      return hipGetLastError();
+    }
+  }
   const int depth = tree_depth(K);
   if (depth > 20) return hipErrorInvalidValue;
-  bf16_bits* out = reinterpret_cast<bf16_bits*>(C);
   // Register slots for 7 levels (K <= 4096), 10 (K <= 32768) or 20: the fewer, the more waves per SIMD.
   if (config == RLK_TREE_CFG_VALU) {
     if (depth <= 7) launch_valu<7>(A, B, out, ldc, M, N, K, tiles, tiles_m, stream);

@@ -114,6 +114,7 @@ int rlk_det_gemm_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stride, c
 }
 
 const char* rlk_det_gemm_tree_contract_id(void) { return "rlkernel.det_gemm.hip_ktree32_gfx950.v1"; }
+const char* rlk_det_gemm_tree_leaf_space_contract_id(void) { return "rlkernel.det_gemm.hip_ktree32_leafspace_gfx950.v1"; }
 
 int rlk_det_gemm_tree_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stride, const void* b,
                            int64_t b_k_stride, int64_t b_n_stride, void* c, int64_t ldc, int M, int N, int K,
@@ -125,8 +126,14 @@ int rlk_det_gemm_tree_bf16(const void* a, int64_t a_row_stride, int64_t a_k_stri
 int rlk_det_gemm_tree_bf16_config(const void* a, int64_t a_row_stride, int64_t a_k_stride, const void* b,
                                   int64_t b_k_stride, int64_t b_n_stride, void* c, int64_t ldc, int M, int N,
                                   int K, int config, void* stream) {
+  const bool leaf_space = config >= 0 && (config & RLK_TREE_CFG_LEAF_SPACE) != 0;
+  if (leaf_space) config &= ~RLK_TREE_CFG_LEAF_SPACE;
   if (config < 0 || config >= RLK_TREE_CFG_COUNT) {
     set_last_error("rlk_det_gemm_tree_bf16: unknown configuration %d", config);
+    return RLK_ERR_INVALID_ARGUMENT;
+  }
+  if (leaf_space && config != RLK_TREE_CFG_AUTO && config != RLK_TREE_CFG_MFMA_F32) {
+    set_last_error("rlk_det_gemm_tree_bf16: RLK_TREE_CFG_LEAF_SPACE goes with RLK_TREE_CFG_AUTO or RLK_TREE_CFG_MFMA_F32");
     return RLK_ERR_INVALID_ARGUMENT;
   }
   if (M < 0 || N < 0 || K < 0) {
@@ -158,7 +165,7 @@ int rlk_det_gemm_tree_bf16_config(const void* a, int64_t a_row_stride, int64_t a
   }
   MatView A{reinterpret_cast<const bf16_bits*>(a), a_row_stride, a_k_stride, M};
   MatView B{reinterpret_cast<const bf16_bits*>(b), b_n_stride, b_k_stride, N};
-  hipError_t err = det_gemm_tree_launch(A, B, c, ldc, M, N, K, config, s);
+  hipError_t err = det_gemm_tree_launch(A, B, c, ldc, M, N, K, config, s, leaf_space);
   if (err == hipErrorInvalidValue && (config == RLK_TREE_CFG_SKINNY || config == RLK_TREE_CFG_NODES)) {
     set_last_error(
         "rlk_det_gemm_tree_bf16: RLK_TREE_CFG_SKINNY needs M <= 16, K-contiguous 16-byte aligned operands and a tree "

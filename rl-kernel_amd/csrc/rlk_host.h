@@ -54,8 +54,9 @@ hipError_t det_gemm_launch(const MatView& W, const MatView& X, void* C, int64_t 
 // The k-tree contract (fp32 leaves of at most 32 K values, bf16 midpoint tree). A[M, K]; B holds
 // one row per output column (B.rows == N); any strides. K <= det_gemm_tree_max_k().
 int det_gemm_tree_max_k();
+// leaf_space: the midpoint split counts fixed 32-wide leaves instead of elements (its own contract id).
 hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int64_t ldc, int M, int N, int K,
-                                int config, hipStream_t stream);
+                                int config, hipStream_t stream, bool leaf_space = false);
 
 // The strictly sequential fp32 chain (one fused multiply-add per k, ascending, no rounding below fp32).
 // An operand is bf16 or fp32, addressed as ptr[row * row_stride + k * k_stride] in elements; B holds one

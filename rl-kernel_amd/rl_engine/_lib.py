@@ -44,6 +44,7 @@ GEMM_CONFIGS = {
 }
 # OR-ed into a GEMM or LogP configuration: register-staged main loop (bit-neutral).
 FORCE_STAGED = 0x100
+TREE_LEAF_SPACE = 0x100  # RLK_TREE_CFG_LEAF_SPACE: OR-ed into rlk_tree_config 0 (auto) or 2 (matrix pipe)
 NOALLOC_SCRATCH_BYTES = 32 << 20  # RLK_NOALLOC_SCRATCH_BYTES
 # rlk_dtype (element types of materialised logits)
 DTYPE_BF16, DTYPE_FP16, DTYPE_FP32 = 0, 1, 2
@@ -59,6 +60,7 @@ EXPORTED_SYMBOLS = (
     "rlk_det_gemm_tree_bf16",
     "rlk_det_gemm_tree_bf16_config",
     "rlk_det_gemm_tree_contract_id",
+    "rlk_det_gemm_tree_leaf_space_contract_id",
     "rlk_det_gemm_seq",
     "rlk_det_gemm_seq_contract_id",
     "rlk_linear_logp_contract_id",
@@ -126,6 +128,8 @@ def load() -> ctypes.CDLL:
     lib.rlk_det_gemm_tree_bf16_config.argtypes = [vp, i64, i64, vp, i64, i64, vp, i64, i32, i32, i32, i32, vp]
     lib.rlk_det_gemm_tree_contract_id.restype = c.c_char_p
     lib.rlk_det_gemm_tree_contract_id.argtypes = []
+    lib.rlk_det_gemm_tree_leaf_space_contract_id.restype = c.c_char_p
+    lib.rlk_det_gemm_tree_leaf_space_contract_id.argtypes = []
     lib.rlk_det_gemm_seq.restype = i32
     lib.rlk_det_gemm_seq.argtypes = [vp, i32, i64, i64, vp, i32, i64, i64, vp, i32, i64, i32, i32, i32, vp]
     lib.rlk_det_gemm_seq_contract_id.restype = c.c_char_p

@@ -154,18 +154,26 @@ def mfma_gemm(
     return out
 
 
-def tree_gemm(a: torch.Tensor, b: torch.Tensor, *, out: torch.Tensor | None = None) -> torch.Tensor:
+def tree_gemm(a: torch.Tensor, b: torch.Tensor, *, out: torch.Tensor | None = None, leaf_space: bool = False) -> torch.Tensor:
     """``a[M,K] @ b[K,N]`` in bf16 under the k-tree contract (any strided views).
 
     Equals the specification the reference's tests evaluate
     (tests/ops/gemm/test_det_gemm.py:156-168) bit for bit; a contiguous half of K is
     exactly one child of the root, so K-sharded partial results combined by bf16
     adds in a balanced rank tree reproduce the unsharded result.
+
+    ``leaf_space=True`` splits the tree over the fixed 32-wide K tiles instead of over elements, the shape of
+    the reference's ``DetGemmTreeReferenceOp`` (rl_engine/reference/gemm/det_gemm.py:29-60): the same result
+    when K / 32 is a power of two, another tree (and contract id, ``tree_leaf_space_contract_id()``) otherwise.
     """
     out = _checked_output(a, b, out)
     if out.numel() == 0:
         return out
-    return _C.gemm_tree_strided(a, b, out)
+    return _C.gemm_tree_strided(a, b, out, _lib.TREE_LEAF_SPACE if leaf_space else 0)
+
+
+def tree_leaf_space_contract_id() -> str:
+    return _lib.load().rlk_det_gemm_tree_leaf_space_contract_id().decode()
 
 
 def _strict_gemm(a: torch.Tensor, b: torch.Tensor, *, out: torch.Tensor | None = None) -> torch.Tensor:

@@ -64,6 +64,48 @@ def test_tree_gemm_is_bit_exact_against_the_oracle(gemm, oracle, shape):
     assert _same_bits(gemm.tree_gemm(a_d, w_d.t()), got_linear)  # run to run
 
 
+@pytest.mark.parametrize("shape", [(4, 65, 129), (8, 4096, 128), (4, 12288, 64), (1, 1, 1), (3, 32, 5), (7, 33, 130), (70, 100, 200),
+                                   (65, 1536, 257), (16, 6144, 96), (130, 1000, 70), (9, 3080, 40)])
+def test_leaf_space_tree_is_bit_exact_against_the_oracle(gemm, oracle, shape):
+    """The leaf-space split (fixed 32-wide leaves, midpoints counted in leaves: the tree of the reference's
+    DetGemmTreeReferenceOp): bit-exact against the oracle's restatement in every operand layout; the same bits as
+    the element-space contract exactly when K / 32 is a power of two."""
+    m, k, n = shape
+    a = inputs.randn_bf16(9150 + k, m, k)
+    w = inputs.randn_bf16(9151 + k, n, k, 0.02)  # [N, K]
+    want = oracle.k_tree_gemm(inputs.bits(a), inputs.bits(w), leaf_space=True)
+    a_d, w_d = a.to(DEV), w.to(DEV)
+    got = gemm.tree_gemm(a_d, w_d.t(), leaf_space=True)
+    assert np.array_equal(inputs.bits(got), want)
+    assert _same_bits(gemm.tree_gemm(a_d, w_d.t().contiguous(), leaf_space=True), got)  # B[K, N]
+    assert _same_bits(gemm.tree_gemm(a_d.t().contiguous().t(), w_d.t(), leaf_space=True), got)  # A stored [K, M]
+    wide = torch.zeros((m, k + 3), dtype=torch.bfloat16, device=DEV)
+    wide[:, :k] = a_d
+    assert _same_bits(gemm.tree_gemm(wide[:, :k], w_d.t(), leaf_space=True), got)  # unaligned rows: element loads
+    row = m // 2
+    assert _same_bits(gemm.tree_gemm(a_d[row : row + 1], w_d.t(), leaf_space=True), got[row : row + 1])  # batch invariant
+    element_space = gemm.tree_gemm(a_d, w_d.t())
+    leaves = (k + 31) // 32
+    if k % 32 == 0 and leaves & (leaves - 1) == 0:
+        assert _same_bits(element_space, got)
+    elif k > 64 and m * n > 500:
+        assert not _same_bits(element_space, got)
+    assert gemm.tree_leaf_space_contract_id() != gemm.det_gemm_backend_id()
+
+
+def test_leaf_space_flag_goes_with_the_tiled_kernels_only():
+    from rl_engine import _C, _lib
+
+    a = inputs.randn_bf16(9160, 4, 4096).to(DEV)
+    w = inputs.randn_bf16(9161, 64, 4096, 0.02).to(DEV)
+    out = torch.empty((4, 64), dtype=torch.bfloat16, device=DEV)
+    base = _C.gemm_tree_strided(a, w.t(), out.clone(), _lib.TREE_LEAF_SPACE)
+    assert _same_bits(_C.gemm_tree_strided(a, w.t(), out.clone(), _lib.TREE_LEAF_SPACE | 2), base)
+    for config in (1, 3, 4):
+        with pytest.raises(ValueError, match="LEAF_SPACE"):
+            _C.gemm_tree_strided(a, w.t(), out, _lib.TREE_LEAF_SPACE | config)
+
+
 def test_tree_gemm_differs_from_the_round_once_contract_only_by_rounding(gemm, oracle):
     a = inputs.randn_bf16(9200, 32, 4096).to(DEV)
     w = inputs.randn_bf16(9201, 256, 4096, 0.02).to(DEV)
