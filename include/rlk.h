@@ -124,9 +124,10 @@ typedef enum rlk_tree_config {
   RLK_TREE_CFG_MFMA_F32 = 2, /* one v_mfma_f32_16x16x1_4b_f32 per k (reduction length one: a single fused step) */
   RLK_TREE_CFG_SKINNY = 3,   /* up to 16 rows: the 16 tree nodes at depth 4 on 16 waves, folded in tree order;
                                 needs K-contiguous aligned operands and equal leaves, else invalid argument */
-  RLK_TREE_CFG_NODES = 4,    /* any row count: 16 rows x 64 columns per workgroup, the 16 depth-4 nodes on 16 waves
-                                (fp32 MFMA, operands from memory to registers); same eligibility as SKINNY but
-                                trees of 4 to 10 levels */
+  RLK_TREE_CFG_NODES = 4,    /* any row count: 16 rows x 64 columns per workgroup, the 8 depth-3 nodes on 8 waves
+                                (fp32 MFMA, each wave streams its own leaves through LDS); same eligibility as
+                                SKINNY but trees of 4 to 10 levels and row strides below 2^24 elements. What
+                                RLK_TREE_CFG_AUTO picks above 8 rows whenever it is eligible */
   RLK_TREE_CFG_COUNT = 5,
   /* OR-ed into RLK_TREE_CFG_AUTO or RLK_TREE_CFG_MFMA_F32: the leaf-space split, a different contract
    * (rlk_det_gemm_tree_leaf_space_contract_id). */

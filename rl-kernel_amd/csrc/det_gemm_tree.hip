@@ -17,16 +17,18 @@
 // own order). Two leaf loops evaluate it, bit for bit the same:
 //   * vector ALU (det_gemm_tree_kernel): 256 threads per tile, a thread owns 4 rows x 8
 //     columns and issues one v_fma_f32 per term; operands staged in LDS as fp32, [k][row];
-//   * fp32 matrix pipe (det_gemm_tree_wide_kernel, the default): 512 threads per tile, a wave
+//   * fp32 matrix pipe (det_gemm_tree_wide_kernel, the default for operands the node-per-wave kernel below
+//     does not take): 512 threads per tile, a wave
 //     owns 32 rows x 32 columns and issues one v_mfma_f32_16x16x1_4b_f32 per k. With a
 //     reduction length of one, an instruction adds exactly one product to every accumulator,
 //     and the product of two bf16 values is exact in fp32, so the step is the same single
 //     rounding as the fused multiply-add, at twice the vector rate; operands staged in LDS
 //     as fp32, [row][k].
 //
-// For few rows (decode) two more kernels split K along the contract's own tree: the 16 nodes at
-// depth 4 are independent, a wave evaluates one of them for a block of outputs, and the 16 bf16
-// nodes are folded in tree order (det_gemm_tree_skinny_kernel, det_gemm_tree_nodes_kernel below).
+// Two more kernels split K along the contract's own tree: the 16 nodes at depth 4 (8 at depth 3) are
+// independent, a wave evaluates one of them for a block of outputs, and the bf16 nodes are folded in tree
+// order: det_gemm_tree_skinny_kernel (up to 16 rows, vector ALU) and det_gemm_tree_nodes_kernel (fp32 matrix
+// pipe, any row count; the fastest of all on K-contiguous aligned operands with equal leaves).
 //
 // Tiled kernels: a workgroup owns a 64 x 128 output tile. Leaves are visited left to right, the next leaf
 // is fetched while the current one is summed. The tree is evaluated on the
@@ -34,6 +36,7 @@
 // finished, so a thread holds at most one bf16 node per tree level. Which slot is read or
 // written is the same for every thread (it depends on K only), so the slot index is a
 // uniform branch over compile-time register arrays, never an indexed register access.
+#include "det_gemm_tile.h"
 #include "rlk_device.h"
 #include "rlk_host.h"
 
@@ -703,57 +706,142 @@ __global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_skinny_ke
   }
 }
 
-// The same split for more rows, on the matrix pipe: a workgroup of 16 waves takes 16 rows, wave w evaluates
-// node w at depth 4 with one v_mfma_f32_16x16x1_4b_f32 per k, operands straight from global memory into
-// registers (a lane streams the weight row of its own column and the A row lane % 16), no LDS stage and no
-// barrier until the 16 nodes are folded. 16 x the workgroups of the tiled kernel: for row counts whose tiles
-// do not fill the chip. The four 16 x 16 blocks of the instruction are
+// The same split for more rows, on the matrix pipe: a workgroup of 8 waves takes 16 rows, wave w evaluates
+// node w at depth 3 with one v_mfma_f32_16x16x1_4b_f32 per k, and wave 0 folds the 8 bf16 nodes in tree order.
+// Many more workgroups than the tiled kernel has tiles: for row counts whose tiles do not fill the chip. Two
+// workgroups fit a CU (LDS, registers), so one computes while the other starts or folds. The four 16 x 16
+// blocks of the instruction are
 //   KB = 1: four groups of 16 columns (64 columns per workgroup), the row operand of block 0 broadcast;
-//   KB = 4: the four grandchildren (depth 6) of the wave's node for one group of 16 columns, every block
+//   KB = 4: the four grandchildren (depth 5) of the wave's node for one group of 16 columns, every block
 //           with its own k range; the lane then folds its four blocks in tree order. Four times the
 //           workgroups and a quarter of the leaves per lane: for narrow N, where 64-column workgroups
 //           would leave most CUs idle and a lane's chain of leaves (one memory round trip each) decides.
-// CHUNKS = leaf length / 8. The leaves of a node are fetched two leaves ahead (one where the registers of a
-// third leaf would spill: 64 columns with leaves of 32); every fetch is
-// issued unconditionally (past the node's end it repeats the last leaf), so that the waits the compiler
-// places count loads along one straight path.
-constexpr int kTreeNodeLevels = 6;  // tree levels below a node, KB = 1 (K <= 32768)
+// CHUNKS = leaf length / 8.
+// Operand path: a lane's operand is 16 bytes per 8 k of ITS column, so loads into registers would touch 64
+// different lines per instruction and the address pipe, not memory or the matrix pipe, would set the pace. A
+// wave therefore brings its leaf in through LDS: direct-to-LDS loads whose lanes walk the 16-byte granules
+// (column, chunk) in order - 4 / CHUNKS columns' worth of contiguous bytes per line touched - into a region of
+// LDS that belongs to the wave alone (two leaves: one landing while the other is read), then every lane reads
+// its own column back with ds_read_b128. No barrier: the wave waits for its own loads. The rows of A go the
+// same way for KB = 1 (16 rows of one k range: one load instruction per leaf); for KB = 4 the four blocks
+// need four k ranges of A, which would not fit beside the weight, and those stay register loads.
+// Every load is issued unconditionally (past the node's end it repeats the last leaf), so that the waits
+// count loads along one straight path.
+// Workgroup ids are dealt so that the row groups of one column group run on the same XCD at the same time and
+// share that L2's copy of the weight.
+constexpr int kTreeNodeSplit = 3;                     // depth of the nodes the waves take
+constexpr int kTreeNodeWaves = 1 << kTreeNodeSplit;   // 8: two workgroups per CU, one starts while the other folds
+constexpr int kTreeNodeLevels = 7;                    // tree levels below a node, KB = 1 (K <= 32768)
 
 template <int KB, int CHUNKS>
-__global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_nodes_kernel(
-    MatView A, MatView B, bf16_bits* __restrict__ C, int64_t ldc, int M, int N, int K, int depth) {
+struct TreeNodesLds {
+  static constexpr int kABytes = KB == 1 ? 1024 : 0;  // a leaf of the 16 rows: one load instruction whatever CHUNKS
+  static constexpr int kWBytes = 1024 * CHUNKS;       // a leaf of the wave's 64 (column, k range) pairs, behind the rows
+  static constexpr int kLeafBytes = kABytes + kWBytes;
+  static constexpr int kWaveBytes = 2 * kLeafBytes;
+  static constexpr int kNodesBytes = kTreeNodeWaves * (KB == 4 ? 2 : 8) * 64 * 4;
+  static constexpr int kStageBytes = kTreeNodeWaves * kWaveBytes;
+  static constexpr int kBytes = kStageBytes > kNodesBytes ? kStageBytes : kNodesBytes;
+};
+
+// On this chip a vector-ALU instruction is not hidden behind the fp32 matrix instructions of the other waves of
+// its SIMD: each one adds about three cycles to the 32 of a 16x16x1 step. The leaf loop is therefore written
+// for few of them: two per step to widen the bf16 operands, addresses as a scalar base plus a lane offset that
+// never changes, LDS reads at immediate offsets (the loop handles an even and an odd leaf per turn, so the
+// staging region of each is known at compile time), and the tree bookkeeping once per pair of leaves.
+template <int KB, int CHUNKS>
+__global__ __launch_bounds__(64 * kTreeNodeWaves, 4) void det_gemm_tree_nodes_kernel(
+    MatView A, MatView B, bf16_bits* __restrict__ C, int64_t ldc, int M, int N, int K, int depth, int row_groups) {
+  using L = TreeNodesLds<KB, CHUNKS>;
   constexpr int kLevels = KB == 4 ? kTreeNodeLevels - 2 : kTreeNodeLevels;
   constexpr int kKeep = KB == 4 ? 2 : 8;  // packed registers a wave hands to the fold
-  constexpr int kTreeNodeAhead = (KB == 1 && CHUNKS == 4) ? 1 : 2;
-  __shared__ uint32_t nodes[kTreeSkinnyWaves][kKeep][64];
+  constexpr int kAAhead = 2;              // KB = 4: leaves of A in flight in registers
+  constexpr int kLoadsPerLeaf = CHUNKS + (KB == 1 ? 1 : CHUNKS);
+  extern __shared__ __attribute__((aligned(16))) char tree_lds[];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int n0 = blockIdx.x * (KB == 4 ? 16 : 64), m0 = blockIdx.y * 16;
-  const int col = n0 + (KB == 4 ? (lane & 15) : lane);
-  const int a_index = m0 + (lane & 15);
-  const bf16_bits* wrow = B.ptr + (int64_t)(col < N ? col : N - 1) * B.row_stride;
-  const bf16_bits* arow = A.ptr + (int64_t)(a_index < M ? a_index : M - 1) * A.row_stride;
+  const int id = xcd_compact_id(blockIdx.x, gridDim.x);
+  const int n0 = (id / row_groups) * (KB == 4 ? 16 : 64), m0 = (id % row_groups) * 16;
   constexpr int len = 8 * CHUNKS;  // leaf length
-  const int node_depth = kTreeSkinnySplit + (KB == 4 ? 2 : 0);
-  const int leaves = 1 << (depth - node_depth);  // leaves under this lane's node
-  const int first = (KB == 4 ? 4 * wave + (lane >> 4) : wave) * leaves * len;
+  const int node_depth = kTreeNodeSplit + (KB == 4 ? 2 : 0);
+  const int leaves = 1 << (depth - node_depth);  // leaves under one block's node: a power of two, at least 2
+  // The k range of block b of this wave starts at (KB * wave + b) * leaves * len; block_k = leaves * len.
+  const int block_k = leaves * len;
+  const int wave_k = (KB == 4 ? 4 * wave : wave) * block_k;  // uniform
 
-  uint32_t slot[kLevels][8];
-  uint32_t cur[8];
-  u32x4_t wq[kTreeNodeAhead + 1][CHUNKS], aq[kTreeNodeAhead + 1][CHUNKS];
-  auto fetch = [&](int leaf, u32x4_t (&w)[CHUNKS], u32x4_t (&a)[CHUNKS]) __attribute__((always_inline)) {
-    const int lo = first + (leaf < leaves ? leaf : leaves - 1) * len;
+  // Granule g = 64 j + lane of a leaf: pair g / CHUNKS (KB = 1: column; KB = 4: column % 16 and block), position
+  // g % CHUNKS, which holds chunk position ^ swizzle(pair): the lanes of a ds_read_b128 then spread over the banks.
+  // Addresses are a uniform base (the workgroup's first column or row, the wave's k range, the leaf) plus a lane
+  // offset in bytes that fits 32 bits (the launcher checks the strides).
+  static_assert(CHUNKS == 3 || CHUNKS == 4, "leaves of 24 or 32");
+  auto swizzle = [](int pair) { return CHUNKS == 4 ? (pair >> 2) & 3 : 0; };  // 48-byte pairs spread by themselves
+  const char* const w_base = reinterpret_cast<const char*>(B.ptr + (int64_t)n0 * B.row_stride + wave_k);
+  const char* const a_base = reinterpret_cast<const char*>(A.ptr + (int64_t)m0 * A.row_stride + wave_k);
+  uint32_t w_off[CHUNKS];
 #pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) {
-      w[c] = *reinterpret_cast<const u32x4_t*>(wrow + lo + 8 * c);
-      a[c] = *reinterpret_cast<const u32x4_t*>(arow + lo + 8 * c);
+  for (int j = 0; j < CHUNKS; ++j) {
+    const int g = 64 * j + lane, pair = g / CHUNKS, chunk = (g % CHUNKS) ^ swizzle(pair);
+    const int col = KB == 4 ? (pair & 15) : pair;
+    const int col_in = n0 + col < N ? col : N - 1 - n0;
+    w_off[j] = 2u * (uint32_t)(col_in * (int)B.row_stride + (KB == 4 ? (pair >> 4) * block_k : 0) + 8 * chunk);
+  }
+  uint32_t a_off;
+  if constexpr (KB == 1) {  // lanes past the 16 rows repeat the last granule; their 16 bytes land in the spare of the region
+    const int g = lane < 16 * CHUNKS ? lane : 16 * CHUNKS - 1, row = g / CHUNKS;
+    const int row_in = m0 + row < M ? row : M - 1 - m0;
+    a_off = 2u * (uint32_t)(row_in * (int)A.row_stride + 8 * ((g % CHUNKS) ^ swizzle(row)));
+  } else {
+    const int row = lane & 15;
+    const int row_in = m0 + row < M ? row : M - 1 - m0;
+    a_off = 2u * (uint32_t)(row_in * (int)A.row_stride + (lane >> 4) * block_k);
+  }
+  char* const mine = tree_lds + wave * L::kWaveBytes;
+  // Lane l reads chunk c of its pair l at read_at[c] (+ kABytes for the weight): rows and columns use the same
+  // lane offsets, lanes 16 .. 63 read rows that do not exist (inside the region; the instruction broadcasts block 0).
+  const char* read_at[CHUNKS];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) read_at[c] = mine + lane * (16 * CHUNKS) + 16 * (c ^ swizzle(lane));
+
+  u32x4_t wq[CHUNKS], aq[KB == 1 ? 1 : kAAhead + 1][CHUNKS];
+  // leaf: which leaf of the node (past the end: the last one again); stage: 0 or 1
+  auto issue = [&](int leaf, int stage_index, u32x4_t (&a)[CHUNKS]) __attribute__((always_inline)) {
+    const int lo = (leaf < leaves ? leaf : leaves - 1) * (2 * len);  // uniform, bytes
+    char* const stage = mine + stage_index * L::kLeafBytes;
+    // the leaf's bases stay in scalar registers (the empty statements keep the compiler from folding the leaf
+    // into the lane offsets, which would cost a 64-bit vector add per load)
+    const char* w_leaf = w_base + lo;
+    const char* a_leaf = a_base + lo;
+    asm volatile("" : "+s"(w_leaf));
+    asm volatile("" : "+s"(a_leaf));
+#pragma unroll
+    for (int j = 0; j < CHUNKS; ++j) {
+      uint32_t off = w_off[j];
+      asm volatile("" : "+v"(off));  // widened here, next to the scalar base, not once outside the loop
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(w_leaf + off), (lds_ptr_t)(stage + L::kABytes + 1024 * j), 16, 0, 0);
+    }
+    uint32_t off = a_off;
+    asm volatile("" : "+v"(off));
+    if constexpr (KB == 1) {
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(a_leaf + off), (lds_ptr_t)stage, 16, 0, 0);
+    } else {
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c) a[c] = *reinterpret_cast<const u32x4_t*>(a_leaf + off + 16 * c);
     }
   };
+  auto take = [&](int stage_index) __attribute__((always_inline)) {  // the landed leaf out of LDS into registers
 #pragma unroll
-  for (int p = 0; p < kTreeNodeAhead; ++p) fetch(p, wq[p], aq[p]);
-  for (int i = 0; i < leaves; ++i) {
-    fetch(i + kTreeNodeAhead, wq[kTreeNodeAhead], aq[kTreeNodeAhead]);
+    for (int c = 0; c < CHUNKS; ++c) {
+      wq[c] = *reinterpret_cast<const u32x4_t*>(read_at[c] + stage_index * L::kLeafBytes + L::kABytes);
+      if constexpr (KB == 1) aq[0][c] = *reinterpret_cast<const u32x4_t*>(read_at[c] + stage_index * L::kLeafBytes);
+    }
+  };
+  // Leaf i (stage i & 1, a compile-time constant at every call): start the load of leaf i + 2 into the region leaf i
+  // came from, sum the leaf, round it to bf16, and bring leaf i + 1 into registers.
+  auto leaf_sum = [&](int i, int stage_index, uint32_t (&node)[8]) __attribute__((always_inline)) {
+    __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // leaf i is in registers: its region is free
+    asm volatile("" ::: "memory");
+    issue(i + 2, stage_index, aq[KB == 1 ? 0 : kAAhead]);
     f32x16_t acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.f;
@@ -761,7 +849,7 @@ __global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_nodes_ker
     for (int c = 0; c < CHUNKS; ++c) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const uint32_t wb = wq[0][c][e >> 1], ab = aq[0][c][e >> 1];
+        const uint32_t wb = wq[c][e >> 1], ab = aq[0][c][e >> 1];
         const float b = __uint_as_float((e & 1) ? (wb & 0xffff0000u) : (wb << 16));
         const float a = __uint_as_float((e & 1) ? (ab & 0xffff0000u) : (ab << 16));
         if constexpr (KB == 4) {
@@ -772,36 +860,55 @@ __global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_nodes_ker
       }
     }
 #pragma unroll
-    for (int q = 0; q < 8; ++q) cur[q] = pack_bf16x2(acc[2 * q], acc[2 * q + 1]);
-    // Leaf i closes one node per trailing one bit of i; then it waits at the level of its lowest zero bit.
-    int level = 0;
-    for (int j = i; j & 1; j >>= 1, ++level) {
+    for (int q = 0; q < 8; ++q) node[q] = pack_bf16x2(acc[2 * q], acc[2 * q + 1]);
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt(kLoadsPerLeaf));  // leaf i + 1 has landed (leaf i + 2 may be on its way)
+    asm volatile("" ::: "memory");
+    take(stage_index ^ 1);
+    if constexpr (KB == 4) {
 #pragma unroll
-      for (int l = 0; l < kLevels; ++l) {
+      for (int p = 0; p < kAAhead; ++p)
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) aq[p][c] = aq[p + 1][c];
+    }
+  };
+
+  uint32_t slot[kLevels - 1][8];  // slot[l]: a finished left child l + 1 levels above the leaves
+  uint32_t left[8], cur[8];
+  issue(0, 0, aq[0]);
+  issue(1, 1, aq[KB == 1 ? 0 : 1]);
+  __builtin_amdgcn_s_waitcnt(wait_vmcnt(kLoadsPerLeaf));  // leaf 0 has landed
+  asm volatile("" ::: "memory");
+  take(0);
+  for (int i = 0; i < leaves; i += 2) {
+    leaf_sum(i, 0, left);
+    leaf_sum(i + 1, 1, cur);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) cur[r] = bf16x2_add(left[r], cur[r]);
+    // Pair i / 2 closes one node per trailing one bit of i / 2; then it waits at the level of its lowest zero bit.
+    int level = 0;
+    for (int j = i >> 1; j & 1; j >>= 1, ++level) {
+#pragma unroll
+      for (int l = 0; l < kLevels - 1; ++l) {
         if (l == level) {
 #pragma unroll
           for (int r = 0; r < 8; ++r) cur[r] = bf16x2_add(slot[l][r], cur[r]);
         }
       }
     }
-    if (i + 1 < leaves) {
+    if (i + 2 < leaves) {
 #pragma unroll
-      for (int l = 0; l < kLevels; ++l) {
+      for (int l = 0; l < kLevels - 1; ++l) {
         if (l == level) {
 #pragma unroll
           for (int r = 0; r < 8; ++r) slot[l][r] = cur[r];
         }
       }
     }
-#pragma unroll
-    for (int p = 0; p < kTreeNodeAhead; ++p) {
-#pragma unroll
-      for (int c = 0; c < CHUNKS; ++c) {
-        wq[p][c] = wq[p + 1][c];
-        aq[p][c] = aq[p + 1][c];
-      }
-    }
   }
+  // The fold's table takes the place of the staging regions: every wave's loads must have landed first.
+  __builtin_amdgcn_s_waitcnt(kWaitAll0);
+  __syncthreads();
+  uint32_t(*nodes)[kKeep][64] = reinterpret_cast<uint32_t(*)[kKeep][64]>(tree_lds);
   // Accumulator r: block r / 4; row 4 (lane / 16) + r % 4, column lane % 16 of the block.
   // cur[q] packs accumulators 2 q, 2 q + 1 (two consecutive rows of one column), block q / 2.
   if constexpr (KB == 4) {
@@ -819,11 +926,11 @@ __global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_nodes_ker
   const int out_row = m0 + 4 * (lane >> 4);
 #pragma unroll
   for (int q = 0; q < kKeep; ++q) {
-    uint32_t v[kTreeSkinnyWaves];
+    uint32_t v[kTreeNodeWaves];
 #pragma unroll
-    for (int w = 0; w < kTreeSkinnyWaves; ++w) v[w] = nodes[w][q][lane];
+    for (int w = 0; w < kTreeNodeWaves; ++w) v[w] = nodes[w][q][lane];
 #pragma unroll
-    for (int width = kTreeSkinnyWaves / 2; width >= 1; width /= 2)
+    for (int width = kTreeNodeWaves / 2; width >= 1; width /= 2)
 #pragma unroll
       for (int w = 0; w < width; ++w) v[w] = bf16x2_add(v[2 * w], v[2 * w + 1]);
     const int c = out_col + (KB == 4 ? 0 : 16 * (q >> 1));
@@ -835,18 +942,30 @@ __global__ __launch_bounds__(64 * kTreeSkinnyWaves) void det_gemm_tree_nodes_ker
   }
 }
 
-template <int KB>
-static void launch_nodes(const MatView& A, const MatView& B, bf16_bits* out, int64_t ldc, int M, int N, int K, int depth,
-                         hipStream_t stream) {
+template <int KB, int CHUNKS>
+static hipError_t launch_nodes_leaf(const MatView& A, const MatView& B, bf16_bits* out, int64_t ldc, int M, int N, int K,
+                                    int depth, hipStream_t stream) {
+  using L = TreeNodesLds<KB, CHUNKS>;
+  static PerDeviceOnce once;
+  auto kernel = det_gemm_tree_nodes_kernel<KB, CHUNKS>;
+  hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), L::kBytes, once);
+  if (err != hipSuccess) return err;
   constexpr int kCols = KB == 4 ? 16 : 64;
-  const dim3 grid((unsigned)((N + kCols - 1) / kCols), (unsigned)((M + 15) / 16)), block(64 * kTreeSkinnyWaves);
-  auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, block, 0, stream, A, B, out, ldc, M, N, K, depth); };
-  switch ((K >> depth) / 8) {  // leaf length 8 ... 32
-    case 1: launch(det_gemm_tree_nodes_kernel<KB, 1>); break;
-    case 2: launch(det_gemm_tree_nodes_kernel<KB, 2>); break;
-    case 3: launch(det_gemm_tree_nodes_kernel<KB, 3>); break;
-    default: launch(det_gemm_tree_nodes_kernel<KB, 4>); break;
-  }
+  const int row_groups = (M + 15) / 16;
+  const int64_t groups = (int64_t)((N + kCols - 1) / kCols) * row_groups;
+  if (groups > 0x7fffffff) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)groups), dim3(64 * kTreeNodeWaves), L::kBytes, stream, A, B, out, ldc, M, N,
+                     K, depth, row_groups);
+  return hipGetLastError();
+}
+
+template <int KB>
+static hipError_t launch_nodes(const MatView& A, const MatView& B, bf16_bits* out, int64_t ldc, int M, int N, int K,
+                               int depth, hipStream_t stream) {
+  // equal leaves that are a multiple of 8 long are 24 or 32 long: a tree stops splitting at 32, so its leaves are
+  // longer than 16
+  return (K >> depth) == 24 ? launch_nodes_leaf<KB, 3>(A, B, out, ldc, M, N, K, depth, stream)
+                            : launch_nodes_leaf<KB, 4>(A, B, out, ldc, M, N, K, depth, stream);
 }
 
 int det_gemm_tree_max_k() { return kTreeLeaf << 20; }
@@ -929,32 +1048,26 @@ hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int
   const bool skinny_ok = M <= 16 && a_chunked && b_chunked && depth >= kTreeSkinnySplit &&
                          depth - kTreeSkinnySplit <= kTreeSkinnyLevels;
   if (config == RLK_TREE_CFG_SKINNY && !skinny_ok) return hipErrorInvalidValue;
-  const bool nodes_ok = a_chunked && b_chunked && depth >= kTreeSkinnySplit &&
-                        depth - kTreeSkinnySplit <= kTreeNodeLevels && (M + 15) / 16 <= 65535;
+  // (at least two leaves under a wave's node; lane offsets of up to 64 rows and the reduction length in 32 bits)
+  const bool nodes_ok = a_chunked && b_chunked && depth > kTreeNodeSplit && depth - kTreeNodeSplit <= kTreeNodeLevels &&
+                        ((K >> depth) == 24 || (K >> depth) == 32) && A.row_stride < (1 << 24) && B.row_stride < (1 << 24);
   if (config == RLK_TREE_CFG_NODES && !nodes_ok) return hipErrorInvalidValue;
   // The node-per-wave kernel splits a node over the four blocks of its instruction where 64-column workgroups
   // would not give every CU one; that needs two more tree levels above the leaves.
   const int64_t wide_groups = (int64_t)((N + 63) / 64) * ((M + 15) / 16);
-  const bool split_blocks = nodes_ok && wide_groups < 256 && depth >= kTreeSkinnySplit + 2;
-  if (config == RLK_TREE_CFG_AUTO && nodes_ok && M > 8) {
-    // Node-per-wave kernel against the tiled one (fitted to the Qwen3-8B projections at 8 ... 4096 rows):
-    // the first runs at about 50 TFLOP/s on rows padded to 16 whatever the grid; the second needs about
-    // 2.25 us per leaf per round of 512 tiles and reaches about 80 TFLOP/s once the chip is full.
-    const double work = 2.0 * N * (double)K;
-    const double t_nodes = work * (16.0 * ((M + 15) / 16)) / 50e12;
-    const double rounds = (double)((tiles64 + 511) / 512);
-    const double t_tiled_latency = rounds * (double)(1 << depth) * 2.25e-6;
-    const double t_tiled_rate = work * M / 80e12;
-    if (t_nodes < (t_tiled_latency > t_tiled_rate ? t_tiled_latency : t_tiled_rate)) config = RLK_TREE_CFG_NODES;
-  }
+  const bool split_blocks = nodes_ok && wide_groups < 256 && depth > kTreeNodeSplit + 2;
+  // More than 8 rows: the node-per-wave kernel wherever it is eligible. Measured on the Qwen3-8B projections it is
+  // ahead of the tiled kernel at every row count (gate_up: 58 against 279 us at 16 rows, 157 against 281 us at 64,
+  // 8.8 against 9.6 ms at 4096; down 4.7 against 6.2 ms at 4096): its waves never meet at a barrier inside a node
+  // and its operands need no conversion pass.
+  if (config == RLK_TREE_CFG_AUTO && nodes_ok && M > 8) config = RLK_TREE_CFG_NODES;
   // Up to 8 rows and narrow N (from HBM, Qwen3-8B down at one token 76 -> 39 us, o_proj 24 -> 15 us; the wide
   // projections measure the same on either kernel): the split blocks shorten a lane's chain of leaves to a
   // quarter, which the vector-ALU kernel's wave halves only halve.
   if (config == RLK_TREE_CFG_AUTO && M <= 8 && split_blocks && N <= kTreeHalvesMaxN) config = RLK_TREE_CFG_NODES;
   if (config == RLK_TREE_CFG_NODES) {
-    if (split_blocks) launch_nodes<4>(A, B, out, ldc, M, N, K, depth, stream);
-    else launch_nodes<1>(A, B, out, ldc, M, N, K, depth, stream);
-    return hipGetLastError();
+    return split_blocks ? launch_nodes<4>(A, B, out, ldc, M, N, K, depth, stream)
+                        : launch_nodes<1>(A, B, out, ldc, M, N, K, depth, stream);
   }
   if (skinny_ok && (config == RLK_TREE_CFG_SKINNY || (config == RLK_TREE_CFG_AUTO && (M <= 8 || !nodes_ok)))) {
     // Narrow N: 32 columns per workgroup and the wave halves on the two children of a node (down at one

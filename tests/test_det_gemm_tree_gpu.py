@@ -252,9 +252,10 @@ def test_skinny_kernel_folds_the_depth_4_nodes_to_the_same_bits(oracle):
 
 
 def test_node_per_wave_kernel_computes_the_same_bits(oracle):
-    # 16 rows per workgroup, one depth-4 node per wave on the fp32 matrix pipe: any row count, ragged M and N,
-    # against the vector-ALU kernel; one case against the oracle. Narrow problems split a node over the four
-    # blocks of the instruction (16 columns per workgroup), problems of 256 and more 64-column groups do not.
+    # 16 rows per workgroup, one depth-3 node per wave on the fp32 matrix pipe: any row count, ragged M and N,
+    # leaves of 24 and of 32, against the vector-ALU kernel; one case against the oracle. Narrow problems split
+    # a node over the four blocks of the instruction (16 columns per workgroup), problems of 256 and more
+    # 64-column groups do not.
     from rl_engine import _C
 
     def run(a_d, b_kn, config):
@@ -273,6 +274,12 @@ def test_node_per_wave_kernel_computes_the_same_bits(oracle):
     a = inputs.randn_bf16(9910, 37, 4096)
     w = inputs.randn_bf16(9911, 70, 4096, 0.02)
     assert np.array_equal(inputs.bits(run(a.to(DEV), w.to(DEV).t(), 4)), _oracle_tree(oracle, a, w))
+    # rows that are views into wider storage (row pitch above K), both operands
+    a_wide = torch.zeros((37, 4096 + 64), dtype=torch.bfloat16, device=DEV)
+    w_wide = torch.zeros((70, 4096 + 8), dtype=torch.bfloat16, device=DEV)
+    a_wide[:, :4096], w_wide[:, 8:] = a.to(DEV), w.to(DEV)
+    assert np.array_equal(inputs.bits(run(a_wide[:, :4096], w_wide[:, 8:].t(), 4)), _oracle_tree(oracle, a, w))
+    assert np.array_equal(inputs.bits(run(a_wide[:, :4096], w_wide[:, 8:].t(), 0)), _oracle_tree(oracle, a, w))
     finite = np.array([0x0000, 0x8000, 0x3F80, 0xBF80, 0x0080, 0x8080, 0x0001, 0x8001, 0x7F7F, 0xFF7F, 0x4000, 0x3F00], dtype=np.uint16)
     rng = np.random.default_rng(9912)
     a_bits, w_bits = rng.choice(finite, size=(40, 1024)), rng.choice(finite[:7], size=(70, 1024))
