@@ -44,7 +44,12 @@ Pinning (which check fixes which function; see tests/test_oracle.py):
 * ``det_gemm_ref_torch`` / ``native_gemm_torch`` / ``linear_logp_chunked_torch`` (the torch forms the CPU baseline
   times): against the numpy forms on seeded inputs (tests/test_oracle.py).
 
-No function here is "parity unpinned".
+One function is "parity unpinned" against the reference: ``det_gemm_seq_f32`` with general fp32 operands
+(``oracle_gemm_seq_fma_f32in``). Its step is one fused multiply-add; the sources it follows
+(csrc/musa/det_gemm.mu:43-44, ``_det_gemm_fp32_kernel``) leave fusion to their compilers and the reference holds
+no fixture with fp32 operands. The function itself is pinned (exact small-integer products, an order-sensitive
+case, a case where fused and unfused steps differ); with bf16-valued operands products are exact and the
+question does not arise. Every other function here is pinned against the reference as listed above.
 """
 
 from __future__ import annotations

@@ -62,7 +62,8 @@ void oracle_gemm_seq_f32(const uint16_t* a, const uint16_t* bt, uint16_t* c, int
  * (csrc/musa/det_gemm.mu:25-48 instantiated for float, its det_gemm_fwd_fp32) and the role of the
  * reference's fp32-output strict GEMM, rl_engine/backends/shared/triton/gemm/det_gemm.py:680-749. The
  * step is written as one fused multiply-add (for bf16-valued operands the product is exact, so the fused
- * step equals multiply-then-add; for general fp32 operands this is the stated choice).
+ * step equals multiply-then-add; for general fp32 operands this is the stated choice: the reference's sources leave
+ * fusion to their compilers and hold no fp32-operand fixture, so against the reference that case is PARITY UNPINNED).
  */
 void oracle_gemm_seq_fma_f32in(const float* a, const float* bt, float* c, int M, int N, int K) {
   for (int i = 0; i < M; ++i)
