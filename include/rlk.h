@@ -127,7 +127,7 @@ typedef enum rlk_tree_config {
   RLK_TREE_CFG_NODES = 4,    /* any row count: 16 rows x 64 columns per workgroup, the 8 depth-3 nodes on 8 waves
                                 (fp32 MFMA, each wave streams its own leaves through LDS); same eligibility as
                                 SKINNY but trees of 4 to 10 levels and row strides below 2^24 elements. What
-                                RLK_TREE_CFG_AUTO picks above 8 rows whenever it is eligible */
+                                RLK_TREE_CFG_AUTO picks whenever it is eligible */
   RLK_TREE_CFG_COUNT = 5,
   /* OR-ed into RLK_TREE_CFG_AUTO or RLK_TREE_CFG_MFMA_F32: the leaf-space split, a different contract
    * (rlk_det_gemm_tree_leaf_space_contract_id). */

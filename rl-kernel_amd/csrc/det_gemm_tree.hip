@@ -27,8 +27,9 @@
 //
 // Two more kernels split K along the contract's own tree: the 16 nodes at depth 4 (8 at depth 3) are
 // independent, a wave evaluates one of them for a block of outputs, and the bf16 nodes are folded in tree
-// order: det_gemm_tree_skinny_kernel (up to 16 rows, vector ALU) and det_gemm_tree_nodes_kernel (fp32 matrix
-// pipe, any row count; the fastest of all on K-contiguous aligned operands with equal leaves).
+// order: det_gemm_tree_nodes_kernel (fp32 matrix pipe, any row count; the fastest of all on K-contiguous aligned
+// operands with equal leaves, and what RLK_TREE_CFG_AUTO picks for them) and det_gemm_tree_skinny_kernel (up to
+// 16 rows, vector ALU; trees of 11 and 12 levels, which the former has no register slots for).
 //
 // Tiled kernels: a workgroup owns a 64 x 128 output tile. Leaves are visited left to right, the next leaf
 // is fetched while the current one is summed. The tree is evaluated on the
@@ -1056,20 +1057,18 @@ hipError_t det_gemm_tree_launch(const MatView& A, const MatView& B, void* C, int
   // would not give every CU one; that needs two more tree levels above the leaves.
   const int64_t wide_groups = (int64_t)((N + 63) / 64) * ((M + 15) / 16);
   const bool split_blocks = nodes_ok && wide_groups < 256 && depth > kTreeNodeSplit + 2;
-  // More than 8 rows: the node-per-wave kernel wherever it is eligible. Measured on the Qwen3-8B projections it is
-  // ahead of the tiled kernel at every row count (gate_up: 58 against 279 us at 16 rows, 157 against 281 us at 64,
-  // 8.8 against 9.6 ms at 4096; down 4.7 against 6.2 ms at 4096): its waves never meet at a barrier inside a node
-  // and its operands need no conversion pass.
-  if (config == RLK_TREE_CFG_AUTO && nodes_ok && M > 8) config = RLK_TREE_CFG_NODES;
-  // Up to 8 rows and narrow N (from HBM, Qwen3-8B down at one token 76 -> 39 us, o_proj 24 -> 15 us; the wide
-  // projections measure the same on either kernel): the split blocks shorten a lane's chain of leaves to a
-  // quarter, which the vector-ALU kernel's wave halves only halve.
-  if (config == RLK_TREE_CFG_AUTO && M <= 8 && split_blocks && N <= kTreeHalvesMaxN) config = RLK_TREE_CFG_NODES;
+  // The node-per-wave kernel wherever it is eligible. Measured on the Qwen3-8B projections it is ahead of the tiled
+  // kernel at every row count (gate_up: 58 against 279 us at 16 rows, 157 against 281 us at 64, 8.8 against 9.6 ms at
+  // 4096; down 4.7 against 6.2 ms at 4096): its waves never meet at a barrier inside a node and its operands need no
+  // conversion pass. Up to 8 rows it is ahead of the vector-ALU kernel below as well, with weights that come from HBM
+  // (gate_up at one token 59 against 84 us, the lm_head 287 against 403 us, down 33 against 75 us).
+  if (config == RLK_TREE_CFG_AUTO && nodes_ok) config = RLK_TREE_CFG_NODES;
   if (config == RLK_TREE_CFG_NODES) {
     return split_blocks ? launch_nodes<4>(A, B, out, ldc, M, N, K, depth, stream)
                         : launch_nodes<1>(A, B, out, ldc, M, N, K, depth, stream);
   }
-  if (skinny_ok && (config == RLK_TREE_CFG_SKINNY || (config == RLK_TREE_CFG_AUTO && (M <= 8 || !nodes_ok)))) {
+  // Up to 16 rows of a tree the node kernel does not take (11 or 12 levels): the vector-ALU node kernel.
+  if (skinny_ok && (config == RLK_TREE_CFG_SKINNY || config == RLK_TREE_CFG_AUTO)) {
     // Narrow N: 32 columns per workgroup and the wave halves on the two children of a node (down at one
     // token 78 -> 61 us, o_proj 24 -> 20 us; gate_up 66 -> 73 us, and 16 rows twice as slow: not there).
     const bool halves = depth > kTreeSkinnySplit && depth - kTreeSkinnySplit - 1 <= kTreeSkinnyLevels && M <= 8 &&

@@ -267,7 +267,8 @@ def test_node_per_wave_kernel_computes_the_same_bits(oracle):
             a = inputs.randn_bf16(9900 + k + m, m, k).to(DEV)
             w = inputs.randn_bf16(9901 + k + m, n, k, 0.02).to(DEV)
             assert _same_bits(run(a, w.t(), 4), run(a, w.t(), 1)), (m, k, n)
-    for m, n, k in ((40, 5500, 4096), (16, 16400, 2048), (33, 5504, 6144)):  # 258, 257 and 258 groups of 64 columns
+    # 258, 257 and 258 groups of 64 columns; then one to eight rows against 257 groups (no split of the blocks)
+    for m, n, k in ((40, 5500, 4096), (16, 16400, 2048), (33, 5504, 6144), (1, 16400, 2048), (3, 16448, 4096), (8, 16400, 3072)):
         a = inputs.randn_bf16(9920 + m, m, k).to(DEV)
         w = inputs.randn_bf16(9921 + m, n, k, 0.02).to(DEV)
         assert _same_bits(run(a, w.t(), 4), run(a, w.t(), 1)), (m, k, n)
