@@ -367,7 +367,7 @@ using Shape64x16 = TileShape<64, 16, 4, 1>;
 using Shape16x16 = TileShape<16, 16, 1, 1>;
 
 static bool view_is_vectorizable(const MatView& v) {
-  return v.k_stride == 1 && (v.row_stride % kChunkElems) == 0 &&
+  return v.k_stride == 1 && (v.row_stride % kChunkElems) == 0 && pitch_fits_lane_offsets(v.row_stride) &&
          (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0;
 }
 
@@ -476,7 +476,7 @@ int pick_det_gemm_config(int M, int N, int K) {
 // weight operand, or the transposed operands of a weight gradient) that the transposing
 // ping-pong loop can take.
 static bool view_is_kmajor_fast(const MatView& v) {
-  return v.row_stride == 1 && v.k_stride >= v.rows && (v.k_stride % kChunkElems) == 0 &&
+  return v.row_stride == 1 && v.k_stride >= v.rows && (v.k_stride % kChunkElems) == 0 && pitch_fits_lane_offsets(v.k_stride) &&
          (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0 && (v.rows % kChunkElems) == 0;
 }
 

@@ -481,7 +481,8 @@ hipError_t linear_logp_launch(const MatView& H, const MatView& W, const int64_t*
   a.group_m = 1;
   const bool vec = W.k_stride == 1 && H.k_stride == 1 && (W.row_stride % kChunkElems) == 0 &&
                    (H.row_stride % kChunkElems) == 0 && (reinterpret_cast<uintptr_t>(W.ptr) & 15) == 0 &&
-                   (reinterpret_cast<uintptr_t>(H.ptr) & 15) == 0 && (D % kChunkElems) == 0;
+                   (reinterpret_cast<uintptr_t>(H.ptr) & 15) == 0 && (D % kChunkElems) == 0 &&
+                   pitch_fits_lane_offsets(W.row_stride) && pitch_fits_lane_offsets(H.row_stride);
   const bool force_staged = (config & RLK_LOGP_CFG_FORCE_STAGED) != 0;
   config &= ~RLK_LOGP_CFG_FORCE_STAGED;
   const int requested = config;

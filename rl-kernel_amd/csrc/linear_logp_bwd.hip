@@ -324,7 +324,8 @@ hipError_t linear_logp_bwd_launch(const MatView& H, const MatView& W, const int6
 
   const bool vec = W.k_stride == 1 && H.k_stride == 1 && (W.row_stride % kChunkElems) == 0 &&
                    (H.row_stride % kChunkElems) == 0 && (reinterpret_cast<uintptr_t>(W.ptr) & 15) == 0 &&
-                   (reinterpret_cast<uintptr_t>(H.ptr) & 15) == 0 && (D % kChunkElems) == 0;
+                   (reinterpret_cast<uintptr_t>(H.ptr) & 15) == 0 && (D % kChunkElems) == 0 &&
+                   pitch_fits_lane_offsets(W.row_stride) && pitch_fits_lane_offsets(H.row_stride);
   const bool force_staged = (config & RLK_LOGP_CFG_FORCE_STAGED) != 0;
   config &= ~RLK_LOGP_CFG_FORCE_STAGED;
   if (config == RLK_LOGP_CFG_AUTO) config = pick_linear_logp_config(T, V);

@@ -31,6 +31,11 @@ inline hipError_t allow_dynamic_lds(const void* kernel, int bytes, PerDeviceOnce
   return err;
 }
 
+// The direct-to-LDS loaders keep a lane's offset inside its block of rows (up to 64 rows of a tile) as a 32-bit
+// element count; a row (or K-row) pitch below 2^24 elements keeps that exact. Larger pitches take the element loaders,
+// which index in 64 bits.
+inline bool pitch_fits_lane_offsets(int64_t ld) { return ld >= 0 && ld < (int64_t(1) << 24); }
+
 // Compute units of the current device (hipDeviceProp_t::multiProcessorCount, read once per device; 256 on an
 // MI355X, which is also the answer when no device can be asked).
 int device_cu_count();

@@ -256,7 +256,8 @@ static bool streams_gated(int M, int K) { return M <= 16 && K >= 1024; }
 
 bool det_gemm_swiglu_fused_supported(const MatView& W, const MatView& X, int M, int K) {
   auto native = [](const MatView& v) {
-    return v.k_stride == 1 && (v.row_stride % kChunkElems) == 0 && (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0;
+    return v.k_stride == 1 && (v.row_stride % kChunkElems) == 0 && pitch_fits_lane_offsets(v.row_stride) &&
+           (reinterpret_cast<uintptr_t>(v.ptr) & 15) == 0;
   };
   return native(W) && native(X) && (K % kTileK) == 0 && (M > 128 || streams_gated(M, K));
 }
