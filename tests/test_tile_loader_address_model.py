@@ -1,6 +1,6 @@
 """A CPU model of the lane addresses of the native-layout direct-to-LDS loader (DmaLoader in csrc/det_gemm_tile.h):
 its row maps, chunk swizzle and edge clamping, with the widths the kernel computes in (64-bit pointers, 32-bit lane
-offsets). Walks launch grids of the GEMM, the gated projection and the stream-group LogP kernel - including the
+offsets), and of its K-major weight form. Walks launch grids of the GEMM, the gated projection and the stream-group LogP kernel - including the
 workgroups whose origin lies past the last vocabulary row - and asserts that every lane reads 16 bytes inside its
 operand, at the row and K position the stage layout expects. As a control, the same walk with the edge path's row
 distance computed in 32 bits (a form that once faulted the GPU) must leave the operand."""
@@ -121,3 +121,30 @@ def test_lane_offsets_fit_32_bits_below_the_pitch_the_launchers_admit():
     for tn in (1, 2, 3, 4):
         rows = max(lane_offset(p, r, 4 * tn) for p in (0, 1) for r in range(8))
         assert rows < 64 and rows * ((1 << 24) - 8) + 56 < U32
+
+
+def kmajor_weight_addresses(bn: int, n0: int, rows: int, ld: int, k0: int):
+    """K-major weight w[k * ld + n]: (block, lane) -> (element address relative to W.ptr, K row, first feature)."""
+    for b, lane in itertools.product(range(bn // 8), range(64)):
+        rib = lane >> 3
+        lane_chunk = (lane & 7) ^ (4 * ((rib >> 1) & 1))  # kmajor_swizzle_of_row_in_block
+        col, kblk = b >> 3, b & 7
+        chunk = lane_chunk ^ (2 * ((kblk ^ (kblk >> 1)) & 1))  # kmajor_swizzle_of_block
+        at = col * 64 + chunk * 8
+        if n0 + col * 64 + 64 > rows:
+            at = min(at, rows - 8 - n0)
+        lane_off = (rib * ld) % U32  # 32 bits
+        yield b, lane, n0 + (k0 + kblk * 8) * ld + lane_off + at, k0 + kblk * 8 + rib, n0 + at
+
+
+@pytest.mark.parametrize("bn,n,k,ld", [(256, 4096, 151936, 4096), (256, 4104, 128, 4104), (128, 72, 64, 80), (64, 8, 64, 8), (256, 24576, 4096, 24576)])
+def test_kmajor_weight_tiles_read_inside_the_weight(bn, n, k, ld):
+    for n0 in sorted({0, (n - 1) // bn * bn}):
+        for k0 in (0, k - 64):
+            seen = set()
+            for b, lane, addr, k_row, feat in kmajor_weight_addresses(bn, n0, n, ld, k0):
+                assert 0 <= addr and addr + 8 <= (k - 1) * ld + n, (n0, k0, b, lane)
+                assert addr == k_row * ld + feat and k0 <= k_row < k0 + 64 and n0 <= feat <= n - 8
+                seen.add((k_row, feat))
+            if n0 + bn <= n:  # an interior tile: every 8-feature chunk of every K row exactly once
+                assert len(seen) == 64 * (bn // 8)
